@@ -1,0 +1,188 @@
+// Fragment-to-register maps for gfx950 (CDNA4) matrix cores.
+//
+// This header is plain constexpr C++ (no HIP) so the maps can be enumerated and checked on
+// the host.  It answers one question: which matrix element does register element `e` of
+// lane `l` hold, for each kind of fragment?
+//
+// Design (differs on purpose from rocWMMA's layout-dependent register formats,
+// reference: library/include/rocwmma/internal/io_layout.hpp:39-308 and layout/*):
+//
+//  * The register layout of a fragment depends on (context, BlockM, BlockN, BlockK, element
+//    size) only -- never on the in-memory data layout.  Fragments are always held in the
+//    order the MFMA instruction consumes, so mma_sync needs no shuffles, applyDataLayout and
+//    applyTranspose are free, and accumulator fragments of different element types or layout
+//    tags agree element by element.
+//
+//  * Input fragments (matrix_a: BlockDim=BlockM rows x BlockK; matrix_b: BlockK x
+//    BlockDim=BlockN columns; described here in the A orientation, "dim" index x k index):
+//        tile   = 32 if BlockM and BlockN are multiples of 32, else 16   (MFMA edge)
+//        groups = 64 / tile                                              (lane groups along K)
+//        kpack  = elements each lane holds per MFMA (contiguous in K)
+//        kstep  = kpack * groups                                         (K extent of one MFMA)
+//      element e = (db * nk + ks) * kpack + j   holds
+//        dim = db * tile + lane % tile
+//        k   = ks * kstep + (lane / tile) * kpack + j
+//    which is exactly the operand layout of v_mfma_*_16x16x{16,32,64,128} /
+//    v_mfma_*_32x32x{8,16,32,64}: one lane = one row (column) and a contiguous run of K.
+//
+//  * Accumulators are held TRANSPOSED with respect to the MFMA result (mma_sync swaps the
+//    two multiplicands), so that a lane owns runs of 4 consecutive columns of one row:
+//        tile 16: e = (bi * nbj + bj) * 4 + i      row = bi*16 + lane%16
+//                                                  col = bj*16 + (lane/16)*4 + i
+//        tile 32: e = (bi * nbj + bj) * 16 + i     row = bi*32 + lane%32
+//                                                  col = bj*32 + 8*(i/4) + (lane/32)*4 + i%4
+//    Row-major C/D tiles therefore move with 16-byte vector accesses.
+#ifndef ROCWMMA_FRAGMENT_MAP_HPP
+#define ROCWMMA_FRAGMENT_MAP_HPP
+
+#include <cstdint>
+
+namespace rocwmma
+{
+    namespace detail
+    {
+        constexpr uint32_t kWaveSize = 64u;
+
+        // Operand class as far as the K packing rules care.
+        enum class PackClass : uint32_t
+        {
+            Bits16, // f16, bf16
+            Fp8, // e4m3, e5m2
+            Int8,
+            Bits32, // f32 inputs
+            Other // 64-bit etc: load / store only
+        };
+
+        constexpr uint32_t mmaTileDim(uint32_t blockM, uint32_t blockN)
+        {
+            return (blockM % 32u == 0u && blockN % 32u == 0u) ? 32u : 16u;
+        }
+
+        // Largest per-lane K run (elements) for which an MFMA exists, given the class.
+        constexpr uint32_t maxKPack(PackClass c)
+        {
+            switch(c)
+            {
+            case PackClass::Bits16:
+                return 8u; // v_mfma_f32_16x16x32_f16 / 32x32x16: 8 halves per lane
+            case PackClass::Fp8:
+                return 32u; // v_mfma_f32_16x16x128_f8f6f4 / 32x32x64: 32 bytes per lane
+            case PackClass::Int8:
+                return 16u; // v_mfma_i32_16x16x64_i8 / 32x32x32: 16 bytes per lane
+            default:
+                return 1u;
+            }
+        }
+
+        // A K run of 16 bytes of fp8 has no instruction (128/64-wide use 32, 32/16-wide use 8).
+        constexpr bool kPackAllowed(PackClass c, uint32_t p)
+        {
+            return !(c == PackClass::Fp8 && p == 16u);
+        }
+
+        constexpr uint32_t chooseKPack(PackClass c, uint32_t tile, uint32_t blockK)
+        {
+            uint32_t groups = kWaveSize / tile;
+            uint32_t p      = maxKPack(c);
+            while(p > 1u && !(kPackAllowed(c, p) && blockK % (p * groups) == 0u))
+                p >>= 1u;
+            return p;
+        }
+
+        // Geometry of an input (matrix_a / matrix_b) fragment.
+        template <uint32_t BlockDim, uint32_t BlockK, uint32_t Tile, PackClass Class>
+        struct InputMap
+        {
+            static_assert(Tile == 16u || Tile == 32u, "MFMA tile edge is 16 or 32");
+            static_assert(BlockDim % Tile == 0u, "block dimension must be a multiple of the MFMA tile");
+
+            static constexpr uint32_t tile    = Tile;
+            static constexpr uint32_t groups  = kWaveSize / Tile;
+            static constexpr uint32_t kpack   = chooseKPack(Class, Tile, BlockK);
+            static constexpr uint32_t kstep   = kpack * groups;
+            static constexpr uint32_t nk      = BlockK / kstep;
+            static constexpr uint32_t ndim    = BlockDim / Tile;
+            static constexpr uint32_t nchunks = ndim * nk; // MFMA operands held
+            static constexpr uint32_t size    = nchunks * kpack; // elements per lane
+
+            static_assert(BlockK % kstep == 0u && nk >= 1u,
+                          "BlockK must be a multiple of 64 / tile (4 for 16-wide, 2 for 32-wide blocks)");
+            static_assert(size * kWaveSize == BlockDim * BlockK, "map must cover the block exactly");
+
+            // chunk c (one MFMA operand) -> (dim block, k step)
+            static constexpr uint32_t chunkDimBlock(uint32_t c)
+            {
+                return c / nk;
+            }
+            static constexpr uint32_t chunkKStep(uint32_t c)
+            {
+                return c % nk;
+            }
+            static constexpr uint32_t chunkIndex(uint32_t dimBlock, uint32_t kStep)
+            {
+                return dimBlock * nk + kStep;
+            }
+            // coordinates of the first element of chunk c held by `lane`
+            static constexpr uint32_t chunkDim(uint32_t c, uint32_t lane)
+            {
+                return chunkDimBlock(c) * Tile + lane % Tile;
+            }
+            static constexpr uint32_t chunkK(uint32_t c, uint32_t lane)
+            {
+                return chunkKStep(c) * kstep + (lane / Tile) * kpack;
+            }
+            // coordinates of element e held by `lane`
+            static constexpr uint32_t dimOf(uint32_t e, uint32_t lane)
+            {
+                return chunkDim(e / kpack, lane);
+            }
+            static constexpr uint32_t kOf(uint32_t e, uint32_t lane)
+            {
+                return chunkK(e / kpack, lane) + e % kpack;
+            }
+        };
+
+        // Geometry of an accumulator fragment.
+        template <uint32_t BlockM, uint32_t BlockN, uint32_t Tile>
+        struct AccMap
+        {
+            static_assert(Tile == 16u || Tile == 32u, "MFMA tile edge is 16 or 32");
+            static_assert(BlockM % Tile == 0u && BlockN % Tile == 0u,
+                          "accumulator block must be a multiple of the MFMA tile");
+
+            static constexpr uint32_t tile     = Tile;
+            static constexpr uint32_t nbi      = BlockM / Tile;
+            static constexpr uint32_t nbj      = BlockN / Tile;
+            static constexpr uint32_t perBlock = Tile * Tile / kWaveSize; // 4 or 16
+            static constexpr uint32_t runs     = perBlock / 4u; // 4-column runs per block per lane
+            static constexpr uint32_t nruns    = nbi * nbj * runs;
+            static constexpr uint32_t size     = nbi * nbj * perBlock;
+
+            static constexpr uint32_t blockIndex(uint32_t bi, uint32_t bj)
+            {
+                return bi * nbj + bj;
+            }
+            // run r = 4 consecutive columns of one row
+            static constexpr uint32_t runRow(uint32_t r, uint32_t lane)
+            {
+                return ((r / runs) / nbj) * Tile + lane % Tile;
+            }
+            static constexpr uint32_t runCol(uint32_t r, uint32_t lane)
+            {
+                return ((r / runs) % nbj) * Tile + (Tile == 16u ? 0u : 8u * (r % runs))
+                       + (lane / Tile) * 4u;
+            }
+            static constexpr uint32_t rowOf(uint32_t e, uint32_t lane)
+            {
+                return runRow(e / 4u, lane);
+            }
+            static constexpr uint32_t colOf(uint32_t e, uint32_t lane)
+            {
+                return runCol(e / 4u, lane) + e % 4u;
+            }
+        };
+
+    } // namespace detail
+} // namespace rocwmma
+
+#endif // ROCWMMA_FRAGMENT_MAP_HPP

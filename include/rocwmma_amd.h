@@ -1,0 +1,254 @@
+/*
+ * rocwmma_amd.h -- C ABI of librocwmma_amd.so: the GEMM / GEMV / DLRM workloads built on the
+ * gfx950 wave-level MMA headers in include/rocwmma/.
+ *
+ * The reference (rocWMMA) is a header-only device library with no host library; what a caller
+ * of its workloads binds to today are the kernel launches inside its sample / test hosts.  Each
+ * entry point below names the reference launch it stands in for.
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is allocated or freed;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the null stream) and
+ *     the call returns without waiting for it;
+ *   - leading dimensions are in elements;
+ *   - the return value is a rocwmma_amd_status (0 = success); a non-zero status means nothing
+ *     was launched.  The reference's hosts exit() on HIP errors (samples/common.hpp:34-46) and
+ *     print "Unsupported size!" for shapes they reject (samples/simple_hgemm.cpp:144-149);
+ *     here both become status codes;
+ *   - no global mutable state: calls are re-entrant and thread safe.
+ */
+#ifndef ROCWMMA_AMD_H
+#define ROCWMMA_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum rocwmma_amd_dtype
+{
+    ROCWMMA_AMD_F16  = 0, /* IEEE binary16                       */
+    ROCWMMA_AMD_BF16 = 1, /* bfloat16                            */
+    ROCWMMA_AMD_E4M3 = 2, /* OCP FP8 E4M3 (rocwmma::float8_t)    */
+    ROCWMMA_AMD_E5M2 = 3, /* OCP FP8 E5M2 (rocwmma::bfloat8_t)   */
+    ROCWMMA_AMD_I8   = 4,
+    ROCWMMA_AMD_F32  = 5,
+    ROCWMMA_AMD_I32  = 6
+} rocwmma_amd_dtype;
+
+typedef enum rocwmma_amd_layout
+{
+    ROCWMMA_AMD_ROW_MAJOR = 0,
+    ROCWMMA_AMD_COL_MAJOR = 1
+} rocwmma_amd_layout;
+
+typedef enum rocwmma_amd_status
+{
+    ROCWMMA_AMD_OK                = 0,
+    ROCWMMA_AMD_INVALID_ARGUMENT  = 1, /* null pointer, zero size, bad enum                  */
+    ROCWMMA_AMD_UNSUPPORTED_TYPE  = 2, /* dtype combination has no kernel                    */
+    ROCWMMA_AMD_UNSUPPORTED_SHAPE = 3, /* size not a multiple of the block the kernel needs  */
+    ROCWMMA_AMD_BAD_ALIGNMENT     = 4, /* pointer or leading dimension not 16-byte aligned   */
+    ROCWMMA_AMD_BAD_LEADING_DIM   = 5, /* leading dimension smaller than the matrix extent   */
+    ROCWMMA_AMD_NO_DEVICE         = 6, /* no gfx950 device is current                        */
+    ROCWMMA_AMD_LAUNCH_FAILED     = 7  /* hipGetLastError() reported a launch failure        */
+} rocwmma_amd_status;
+
+/* Which GEMM kernel family rocwmma_amd_gemm_ex runs. */
+typedef enum rocwmma_amd_gemm_algo
+{
+    ROCWMMA_AMD_GEMM_AUTO      = 0, /* blocked kernel when the shape allows, else wave-tile */
+    ROCWMMA_AMD_GEMM_WAVE_TILE = 1, /* one block per wave, operands straight from global    */
+    ROCWMMA_AMD_GEMM_BLOCKED   = 2  /* LDS multi-buffered macro-tile kernel                 */
+} rocwmma_amd_gemm_algo;
+
+/* Library identification: returns 10000*major + 100*minor + patch. */
+int rocwmma_amd_version(void);
+
+/* Static, human readable text for a status code. */
+const char* rocwmma_amd_status_string(int status);
+
+/* Properties of the current device the benchmarks report next to their numbers:
+ * compute-unit count, peak engine clock in MHz, and whether it is gfx950. */
+int rocwmma_amd_device_info(int* compute_units, int* clock_mhz, int* is_gfx950);
+
+/*
+ * D = alpha * A * B + beta * C.
+ *
+ * Stands in for the kernel launches of the reference's GEMM hosts, whose kernels all take
+ * (m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta):
+ *   samples/simple_hgemm.cpp:81-93,202      (hgemm_rocwmma_d: one block per wave)
+ *   samples/perf_hgemm.cpp:518-530,848-870  (gemm_rocwmma_d: LDS double-buffered macro tile)
+ *   test/gemm/gemm_kernel_base.hpp          (KernelFunc, the test-suite generalisation)
+ *
+ * A is m x k, B is k x n, C and D are m x n; C and D share `layout_c`.
+ * dtype_in  : element type of A and B (F16, BF16, E4M3, E5M2, I8).
+ * dtype_out : element type of C and D: F32 for the float inputs (F16 also allowed with F16
+ *             inputs), I32 for I8.  The compute type is f32 (i32 for I8); alpha and beta are
+ *             converted to it (for I8 they must be integers).
+ * c may be NULL when beta == 0.  c may equal d.
+ * Shapes: m and n multiples of 16, k a multiple of 32 bytes' worth of elements per row is the
+ * minimum every kernel accepts (k % 16 == 0 for 16-bit types, k % 32 == 0 for 8-bit types);
+ * the blocked kernel additionally needs whole macro tiles and is chosen automatically.
+ * Alignment: base pointers and leading dimensions must be multiples of 16 bytes.
+ */
+int rocwmma_amd_gemm(int         dtype_in,
+                     int         dtype_out,
+                     int         layout_a,
+                     int         layout_b,
+                     int         layout_c,
+                     uint32_t    m,
+                     uint32_t    n,
+                     uint32_t    k,
+                     const void* a,
+                     uint32_t    lda,
+                     const void* b,
+                     uint32_t    ldb,
+                     const void* c,
+                     uint32_t    ldc,
+                     void*       d,
+                     uint32_t    ldd,
+                     float       alpha,
+                     float       beta,
+                     void*       stream);
+
+/* Same as rocwmma_amd_gemm with the kernel family forced (`algo` is a rocwmma_amd_gemm_algo).
+ * ROCWMMA_AMD_GEMM_BLOCKED returns ROCWMMA_AMD_UNSUPPORTED_SHAPE when the shape does not fill
+ * whole macro tiles, like the reference's perf_hgemm host (samples/perf_hgemm.cpp:735-765). */
+int rocwmma_amd_gemm_ex(int         algo,
+                        int         dtype_in,
+                        int         dtype_out,
+                        int         layout_a,
+                        int         layout_b,
+                        int         layout_c,
+                        uint32_t    m,
+                        uint32_t    n,
+                        uint32_t    k,
+                        const void* a,
+                        uint32_t    lda,
+                        const void* b,
+                        uint32_t    ldb,
+                        const void* c,
+                        uint32_t    ldc,
+                        void*       d,
+                        uint32_t    ldd,
+                        float       alpha,
+                        float       beta,
+                        void*       stream);
+
+/*
+ * Skinny GEMV / GEMM:  Y = alpha * A * X + beta * Y,  in place on Y.
+ *
+ * Stands in for sgemv_rocwmma_d and its host (samples/simple_sgemv.cpp:103-155,207-227), whose
+ * semantics are those of its CPU twin sgemv_cpu_h (samples/simple_sgemv.cpp:46-66); here for
+ * f16 A and up to 8 right-hand sides, as a pure bandwidth kernel (no MFMA).
+ *
+ * A : m x k, f16, row-major, leading dimension lda >= k.
+ * X : k x ncols, f16, column-major (each right-hand side contiguous), ldx >= k.
+ * Y : m x ncols, f32, column-major, ldy >= m.  Read only when beta != 0.
+ * ncols in {1, 2, 4, 8}; k a multiple of 8; A, X 16-byte aligned with lda, ldx multiples of 8.
+ */
+int rocwmma_amd_gemv(uint32_t    m,
+                     uint32_t    k,
+                     uint32_t    ncols,
+                     const void* a,
+                     uint32_t    lda,
+                     const void* x,
+                     uint32_t    ldx,
+                     float*      y,
+                     uint32_t    ldy,
+                     float       alpha,
+                     float       beta,
+                     void*       stream);
+
+/*
+ * DLRM dot-interaction, forward.  f16 in / out, f32 accumulate.
+ *
+ * Stands in for dlrmDotFwd and its launch (samples/simple_dlrm.cpp:184-284,504-529;
+ * test/dlrm/device/dlrm_dot_fwd.hpp:38).  Semantics = dlrm_fwd_CPU
+ * (test/reference_impl.hpp:83-119):
+ *   input  : batch x m x k   (row 0 of every sample is the bottom-MLP output)
+ *   output : batch x (k + m(m-1)/2):  [ input[b,0,:] , Z[1,0], Z[2,0], Z[2,1], Z[3,0], ... ]
+ *            with Z = input[b] * input[b]^T.
+ * Unlike the reference kernel this one needs no f32 m x m scratch (`acc`) and accepts any
+ * m <= 32 (the reference GPU kernels need m % 16 == 0, test/dlrm/dlrm_kernel_base_impl.hpp:146-150).
+ * k must be a multiple of 16 and at most 256; input must be 16-byte aligned.
+ */
+int rocwmma_amd_dlrm_fwd(const void* input,
+                         void*       output,
+                         uint32_t    m,
+                         uint32_t    k,
+                         uint32_t    batch,
+                         void*       stream);
+
+/*
+ * DLRM dot-interaction, backward.
+ *
+ * Stands in for trilReconstruct + dlrmDotBwd and their launches
+ * (samples/simple_dlrm.cpp:290-441,534-587; test/dlrm/device/dlrm_dot_bwd.hpp:36,80) in ONE
+ * launch with no m x m scratch and no host synchronisation in between.  Semantics =
+ * dlrm_bwd_CPU (test/reference_impl.hpp:121-179):
+ *   upstream_grad   : batch x (k + m(m-1)/2)
+ *   bottom_mlp_grad : batch x k        = upstream_grad[b, 0:k]
+ *   grad            : batch x m x k    = G * input[b],  G = symmetric matrix rebuilt from the
+ *                     packed strict lower triangle upstream_grad[b, k:], zero diagonal.
+ * The bottom-MLP gradient is NOT added into grad row 0 (neither does the reference).
+ * Same shape limits as the forward pass.
+ */
+int rocwmma_amd_dlrm_bwd(const void* input,
+                         const void* upstream_grad,
+                         void*       grad,
+                         void*       bottom_mlp_grad,
+                         uint32_t    m,
+                         uint32_t    k,
+                         uint32_t    batch,
+                         void*       stream);
+
+/*
+ * Fragment API self-tests (device side of the API-semantics tests; each launches a tiny kernel
+ * written only with the public rocwmma:: API and returns a status).
+ *
+ * rocwmma_amd_selftest_roundtrip: out = store(load(in)) for one fragment kind; mirrors the
+ * reference unit test test/unit/load_store_matrix_sync_test/device/load_store_matrix_sync.hpp:35-117
+ * (and, with coop != 0, the cooperative twin load_store_matrix_coop_sync_test).
+ *   context : 0 matrix_a, 1 matrix_b, 2 accumulator
+ *   `in`/`out` are rows x cols matrices of `dtype` in `layout` with leading dimension ld; the
+ *   grid covers the matrix with one fragment per wave (or per workgroup of 4 waves when coop).
+ *   block   : 16 or 32 (BlockM = BlockN), blockk : K extent of the fragment.
+ */
+int rocwmma_amd_selftest_roundtrip(int         context,
+                                   int         dtype,
+                                   int         layout,
+                                   int         block,
+                                   int         blockk,
+                                   int         coop,
+                                   uint32_t    rows,
+                                   uint32_t    cols,
+                                   const void* in,
+                                   void*       out,
+                                   uint32_t    ld,
+                                   void*       stream);
+
+/* Runs the reference's perf_hgemm data flow (cooperative global read -> applyDataLayout /
+ * applyTranspose -> cooperative LDS write -> LDS read -> mma_sync) written only against the
+ * public API, f16 in / f32 out, for the four A/B layout combinations.  Used to test the
+ * cooperative and transform API end to end. */
+int rocwmma_amd_selftest_coop_gemm(int         layout_a,
+                                   int         layout_b,
+                                   uint32_t    m,
+                                   uint32_t    n,
+                                   uint32_t    k,
+                                   const void* a,
+                                   const void* b,
+                                   const float* c,
+                                   float*      d,
+                                   float       alpha,
+                                   float       beta,
+                                   void*       stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ROCWMMA_AMD_H */

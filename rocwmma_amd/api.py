@@ -1,0 +1,156 @@
+"""ctypes binding of librocwmma_amd.so plus thin torch-tensor wrappers.
+
+The wrappers mirror the argument lists of the reference's workload hosts
+(samples/simple_hgemm.cpp:141 gemm_test, samples/perf_hgemm.cpp:716 gemm_test,
+samples/simple_sgemv.cpp sgemv_test, samples/simple_dlrm.cpp:443 dlrm_test) but take device
+tensors, run on torch's current stream and raise RocwmmaError instead of exiting.
+torch is used for device memory and streams only."""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_NAME = "librocwmma_amd.so"
+
+F16, BF16, E4M3, E5M2, I8, F32, I32 = range(7)
+ROW_MAJOR, COL_MAJOR = 0, 1
+GEMM_AUTO, GEMM_WAVE_TILE, GEMM_BLOCKED = 0, 1, 2
+
+EXPORTS = [
+    "rocwmma_amd_version", "rocwmma_amd_status_string", "rocwmma_amd_device_info", "rocwmma_amd_gemm",
+    "rocwmma_amd_gemm_ex", "rocwmma_amd_gemv", "rocwmma_amd_dlrm_fwd", "rocwmma_amd_dlrm_bwd",
+    "rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm",
+]
+
+
+class RocwmmaError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        super().__init__(f"{where}: status {status} ({status_string(status)})")
+
+
+def library_path():
+    return os.path.join(HERE, _LIB_NAME)
+
+
+_lib = None
+
+
+def library():
+    """Loads the built library.  It is never built implicitly on import: run
+    ``python -c "import __graft_entry__ as g; g.build()"`` (or rocwmma_amd/build.py) first."""
+    global _lib
+    if _lib is None:
+        path = library_path()
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `python rocwmma_amd/build.py`")
+        L = ctypes.CDLL(path)
+        i, u, vp, f = ctypes.c_int, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_float
+        L.rocwmma_amd_version.restype = i
+        L.rocwmma_amd_status_string.argtypes = [i]
+        L.rocwmma_amd_status_string.restype = ctypes.c_char_p
+        L.rocwmma_amd_device_info.argtypes = [ctypes.POINTER(i)] * 3
+        L.rocwmma_amd_device_info.restype = i
+        gemm_args = [i, i, i, i, i, u, u, u, vp, u, vp, u, vp, u, vp, u, f, f, vp]
+        L.rocwmma_amd_gemm.argtypes = gemm_args
+        L.rocwmma_amd_gemm.restype = i
+        L.rocwmma_amd_gemm_ex.argtypes = [i] + gemm_args
+        L.rocwmma_amd_gemm_ex.restype = i
+        L.rocwmma_amd_gemv.argtypes = [u, u, u, vp, u, vp, u, vp, u, f, f, vp]
+        L.rocwmma_amd_gemv.restype = i
+        L.rocwmma_amd_dlrm_fwd.argtypes = [vp, vp, u, u, u, vp]
+        L.rocwmma_amd_dlrm_fwd.restype = i
+        L.rocwmma_amd_dlrm_bwd.argtypes = [vp, vp, vp, vp, u, u, u, vp]
+        L.rocwmma_amd_dlrm_bwd.restype = i
+        L.rocwmma_amd_selftest_roundtrip.argtypes = [i, i, i, i, i, i, u, u, vp, vp, u, vp]
+        L.rocwmma_amd_selftest_roundtrip.restype = i
+        L.rocwmma_amd_selftest_coop_gemm.argtypes = [i, i, u, u, u, vp, vp, vp, vp, f, f, vp]
+        L.rocwmma_amd_selftest_coop_gemm.restype = i
+        _lib = L
+    return _lib
+
+
+def version():
+    return library().rocwmma_amd_version()
+
+
+def status_string(status):
+    return library().rocwmma_amd_status_string(int(status)).decode()
+
+
+def device_info():
+    cu, mhz, ok = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    rc = library().rocwmma_amd_device_info(ctypes.byref(cu), ctypes.byref(mhz), ctypes.byref(ok))
+    if rc != 0:
+        raise RocwmmaError(rc, "device_info")
+    return {"compute_units": cu.value, "clock_mhz": mhz.value, "is_gfx950": bool(ok.value)}
+
+
+def _check(rc, where):
+    if rc != 0:
+        raise RocwmmaError(rc, where)
+
+
+def _stream():
+    import torch
+
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def gemm_raw(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, lda, b, ldb, c, ldc, d, ldd,
+             alpha, beta, algo=GEMM_AUTO, stream=None):
+    """Straight call of rocwmma_amd_gemm_ex with raw device pointers (ints / c_void_p)."""
+    rc = library().rocwmma_amd_gemm_ex(algo, dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k,
+                                       a, lda, b, ldb, c, ldc, d, ldd, alpha, beta,
+                                       stream if stream is not None else _stream())
+    _check(rc, "gemm")
+
+
+def gemm(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, b, c, d, alpha, beta,
+         lda=None, ldb=None, ldc=None, ldd=None, algo=GEMM_AUTO):
+    """D = alpha*A*B + beta*C on device tensors (any shape; only data_ptr is used), natural
+    leading dimensions unless given.  Kernel argument order of the reference
+    (m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta)."""
+    lda = lda if lda is not None else (k if layout_a == ROW_MAJOR else m)
+    ldb = ldb if ldb is not None else (n if layout_b == ROW_MAJOR else k)
+    nat = n if layout_c == ROW_MAJOR else m
+    ldc = ldc if ldc is not None else nat
+    ldd = ldd if ldd is not None else nat
+    gemm_raw(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, _ptr(a), lda, _ptr(b), ldb,
+             _ptr(c), ldc, _ptr(d), ldd, alpha, beta, algo)
+    return d
+
+
+def gemv(m, k, ncols, a, x, y, alpha=1.0, beta=0.0, lda=None, ldx=None, ldy=None):
+    """Y = alpha*A*X + beta*Y in place; A f16 row-major m x k, X f16 k x ncols column-major,
+    Y f32 m x ncols column-major."""
+    rc = library().rocwmma_amd_gemv(m, k, ncols, _ptr(a), lda or k, _ptr(x), ldx or k, _ptr(y), ldy or m,
+                                    alpha, beta, _stream())
+    _check(rc, "gemv")
+    return y
+
+
+def dlrm_fwd(inp, out, m, k, batch):
+    _check(library().rocwmma_amd_dlrm_fwd(_ptr(inp), _ptr(out), m, k, batch, _stream()), "dlrm_fwd")
+    return out
+
+
+def dlrm_bwd(inp, upstream, grad, mlp_grad, m, k, batch):
+    _check(library().rocwmma_amd_dlrm_bwd(_ptr(inp), _ptr(upstream), _ptr(grad), _ptr(mlp_grad), m, k, batch,
+                                          _stream()), "dlrm_bwd")
+    return grad, mlp_grad
+
+
+def selftest_roundtrip(context, dtype, layout, block, blockk, coop, rows, cols, inp, out, ld):
+    _check(library().rocwmma_amd_selftest_roundtrip(context, dtype, layout, block, blockk, int(coop), rows, cols,
+                                                    _ptr(inp), _ptr(out), ld, _stream()), "selftest_roundtrip")
+    return out
+
+
+def selftest_coop_gemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta):
+    _check(library().rocwmma_amd_selftest_coop_gemm(layout_a, layout_b, m, n, k, _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+                                                    alpha, beta, _stream()), "selftest_coop_gemm")
+    return d

@@ -1,0 +1,343 @@
+// extern "C" entry points of librocwmma_amd.so: argument validation and dispatch to the kernel
+// families.  Declarations and the reference interfaces they stand in for: include/rocwmma_amd.h.
+#include "common.hpp"
+
+#include <atomic>
+#include <cmath>
+#include <cstring>
+
+namespace rocwmma_amd
+{
+    int launchGemv(uint32_t m, uint32_t k, uint32_t ncols, const void* a, uint32_t lda, const void* x, uint32_t ldx,
+                   float* y, uint32_t ldy, float alpha, float beta, hipStream_t stream);
+    int launchDlrmFwd(const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, hipStream_t stream);
+    int launchDlrmBwd(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t k,
+                      uint32_t batch, hipStream_t stream);
+    int selftestRoundtrip(int context, int dtype, int layout, int block, int blockk, int coop, uint32_t rows, uint32_t cols,
+                          const void* in, void* out, uint32_t ld, hipStream_t stream);
+    int selftestCoopGemm(int layoutA, int layoutB, uint32_t m, uint32_t n, uint32_t k, const void* a, const void* b,
+                         const float* c, float* d, float alpha, float beta, hipStream_t stream);
+
+    namespace
+    {
+        bool validLayout(int l)
+        {
+            return l == ROCWMMA_AMD_ROW_MAJOR || l == ROCWMMA_AMD_COL_MAJOR;
+        }
+
+        // Whether the current device is a gfx950.  The answer never changes for a device, so it
+        // is remembered per device ordinal (0 = not asked yet, 1 = yes, 2 = no).
+        bool isGfx950Current()
+        {
+            constexpr int           kMaxDevices = 64;
+            static std::atomic<int> known[kMaxDevices];
+            int                     dev = 0;
+            if(hipGetDevice(&dev) != hipSuccess)
+                return false;
+            if(dev >= 0 && dev < kMaxDevices)
+            {
+                const int cached = known[dev].load(std::memory_order_relaxed);
+                if(cached != 0)
+                    return cached == 1;
+            }
+            hipDeviceProp_t props;
+            if(hipGetDeviceProperties(&props, dev) != hipSuccess)
+                return false;
+            const bool yes = std::strncmp(props.gcnArchName, "gfx950", 6) == 0;
+            if(dev >= 0 && dev < kMaxDevices)
+                known[dev].store(yes ? 1 : 2, std::memory_order_relaxed);
+            return yes;
+        }
+
+        // Pure argument checks of the GEMM entry points (no device access): shared by the
+        // entry points and testable without a GPU.
+        int checkGemm(int dtypeIn, int dtypeOut, int layoutA, int layoutB, int layoutC, uint32_t m, uint32_t n, uint32_t k,
+                      const void* a, uint32_t lda, const void* b, uint32_t ldb, const void* c, uint32_t ldc, void* d,
+                      uint32_t ldd, float alpha, float beta)
+        {
+            if(!a || !b || !d || m == 0u || n == 0u || k == 0u)
+                return ROCWMMA_AMD_INVALID_ARGUMENT;
+            if(!validLayout(layoutA) || !validLayout(layoutB) || !validLayout(layoutC))
+                return ROCWMMA_AMD_INVALID_ARGUMENT;
+            if(!c && beta != 0.0f)
+                return ROCWMMA_AMD_INVALID_ARGUMENT;
+            const bool floatIn = dtypeIn == ROCWMMA_AMD_F16 || dtypeIn == ROCWMMA_AMD_BF16 || dtypeIn == ROCWMMA_AMD_E4M3
+                                 || dtypeIn == ROCWMMA_AMD_E5M2;
+            const bool okTypes = (floatIn && dtypeOut == ROCWMMA_AMD_F32)
+                                 || (dtypeIn == ROCWMMA_AMD_F16 && dtypeOut == ROCWMMA_AMD_F16)
+                                 || (dtypeIn == ROCWMMA_AMD_I8 && dtypeOut == ROCWMMA_AMD_I32);
+            if(!okTypes)
+                return ROCWMMA_AMD_UNSUPPORTED_TYPE;
+            if(dtypeIn == ROCWMMA_AMD_I8 && (alpha != std::nearbyint(alpha) || beta != std::nearbyint(beta)))
+                return ROCWMMA_AMD_INVALID_ARGUMENT;
+            const uint32_t inSize  = dtypeSize(dtypeIn);
+            const uint32_t outSize = dtypeSize(dtypeOut);
+            if(m % 16u != 0u || n % 16u != 0u || (k * inSize) % 32u != 0u)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            const uint32_t minLda = layoutA == ROCWMMA_AMD_ROW_MAJOR ? k : m;
+            const uint32_t minLdb = layoutB == ROCWMMA_AMD_ROW_MAJOR ? n : k;
+            const uint32_t minLdc = layoutC == ROCWMMA_AMD_ROW_MAJOR ? n : m;
+            if(lda < minLda || ldb < minLdb || ldd < minLdc || (c && ldc < minLdc))
+                return ROCWMMA_AMD_BAD_LEADING_DIM;
+            if(!aligned16(a) || !aligned16(b) || !aligned16(d) || (c && !aligned16(c)))
+                return ROCWMMA_AMD_BAD_ALIGNMENT;
+            if((lda * inSize) % 16u != 0u || (ldb * inSize) % 16u != 0u || (ldd * outSize) % 16u != 0u
+               || (c && (ldc * outSize) % 16u != 0u))
+                return ROCWMMA_AMD_BAD_ALIGNMENT;
+            return ROCWMMA_AMD_OK;
+        }
+
+        int flip(int layout)
+        {
+            return layout == ROCWMMA_AMD_ROW_MAJOR ? ROCWMMA_AMD_COL_MAJOR : ROCWMMA_AMD_ROW_MAJOR;
+        }
+    } // namespace
+} // namespace rocwmma_amd
+
+using namespace rocwmma_amd;
+
+extern "C" {
+
+int rocwmma_amd_version(void)
+{
+    return ROCWMMA_VERSION_MAJOR * 10000 + ROCWMMA_VERSION_MINOR * 100 + ROCWMMA_VERSION_PATCH;
+}
+
+const char* rocwmma_amd_status_string(int status)
+{
+    switch(status)
+    {
+    case ROCWMMA_AMD_OK:
+        return "success";
+    case ROCWMMA_AMD_INVALID_ARGUMENT:
+        return "invalid argument (null pointer, zero size or bad enum)";
+    case ROCWMMA_AMD_UNSUPPORTED_TYPE:
+        return "unsupported element type combination";
+    case ROCWMMA_AMD_UNSUPPORTED_SHAPE:
+        return "unsupported size: not a multiple of the block the kernel needs";
+    case ROCWMMA_AMD_BAD_ALIGNMENT:
+        return "pointer or leading dimension is not 16-byte aligned";
+    case ROCWMMA_AMD_BAD_LEADING_DIM:
+        return "leading dimension smaller than the matrix extent";
+    case ROCWMMA_AMD_NO_DEVICE:
+        return "no gfx950 device is current";
+    case ROCWMMA_AMD_LAUNCH_FAILED:
+        return "kernel launch failed";
+    default:
+        return "unknown status";
+    }
+}
+
+int rocwmma_amd_device_info(int* compute_units, int* clock_mhz, int* is_gfx950)
+{
+    int dev = 0;
+    if(hipGetDevice(&dev) != hipSuccess)
+        return ROCWMMA_AMD_NO_DEVICE;
+    hipDeviceProp_t props;
+    if(hipGetDeviceProperties(&props, dev) != hipSuccess)
+        return ROCWMMA_AMD_NO_DEVICE;
+    if(compute_units)
+        *compute_units = props.multiProcessorCount;
+    if(clock_mhz)
+        *clock_mhz = props.clockRate / 1000;
+    if(is_gfx950)
+        *is_gfx950 = std::strncmp(props.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
+    return ROCWMMA_AMD_OK;
+}
+
+int rocwmma_amd_gemm_ex(int         algo,
+                        int         dtype_in,
+                        int         dtype_out,
+                        int         layout_a,
+                        int         layout_b,
+                        int         layout_c,
+                        uint32_t    m,
+                        uint32_t    n,
+                        uint32_t    k,
+                        const void* a,
+                        uint32_t    lda,
+                        const void* b,
+                        uint32_t    ldb,
+                        const void* c,
+                        uint32_t    ldc,
+                        void*       d,
+                        uint32_t    ldd,
+                        float       alpha,
+                        float       beta,
+                        void*       stream)
+{
+    int rc = checkGemm(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, lda, b, ldb, c, ldc, d, ldd, alpha, beta);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(algo != ROCWMMA_AMD_GEMM_AUTO && algo != ROCWMMA_AMD_GEMM_WAVE_TILE && algo != ROCWMMA_AMD_GEMM_BLOCKED)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+
+    GemmArgs args{m, n, k, a, b, c, d, lda, ldb, c ? ldc : ldd, ldd, alpha, beta, layout_c};
+    if(algo != ROCWMMA_AMD_GEMM_WAVE_TILE)
+    {
+        // The blocked kernel writes row-major C/D; a column-major result is the row-major
+        // result of the transposed problem D^T = B^T * A^T.
+        GemmArgs blocked = args;
+        int      la = layout_a, lb = layout_b;
+        if(layout_c == ROCWMMA_AMD_COL_MAJOR)
+        {
+            blocked.m       = n;
+            blocked.n       = m;
+            blocked.a       = b;
+            blocked.b       = a;
+            blocked.lda     = ldb;
+            blocked.ldb     = lda;
+            la              = flip(layout_b);
+            lb              = flip(layout_a);
+            blocked.layoutC = ROCWMMA_AMD_ROW_MAJOR;
+        }
+        rc = launchGemmBlocked(dtype_in, dtype_out, la, lb, blocked, asStream(stream));
+        if(rc == ROCWMMA_AMD_OK || algo == ROCWMMA_AMD_GEMM_BLOCKED)
+            return rc;
+        if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE && rc != ROCWMMA_AMD_UNSUPPORTED_TYPE)
+            return rc;
+    }
+    return launchGemmWaveTile(dtype_in, dtype_out, layout_a, layout_b, args, asStream(stream));
+}
+
+int rocwmma_amd_gemm(int         dtype_in,
+                     int         dtype_out,
+                     int         layout_a,
+                     int         layout_b,
+                     int         layout_c,
+                     uint32_t    m,
+                     uint32_t    n,
+                     uint32_t    k,
+                     const void* a,
+                     uint32_t    lda,
+                     const void* b,
+                     uint32_t    ldb,
+                     const void* c,
+                     uint32_t    ldc,
+                     void*       d,
+                     uint32_t    ldd,
+                     float       alpha,
+                     float       beta,
+                     void*       stream)
+{
+    return rocwmma_amd_gemm_ex(ROCWMMA_AMD_GEMM_AUTO, dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, lda, b,
+                               ldb, c, ldc, d, ldd, alpha, beta, stream);
+}
+
+int rocwmma_amd_gemv(uint32_t    m,
+                     uint32_t    k,
+                     uint32_t    ncols,
+                     const void* a,
+                     uint32_t    lda,
+                     const void* x,
+                     uint32_t    ldx,
+                     float*      y,
+                     uint32_t    ldy,
+                     float       alpha,
+                     float       beta,
+                     void*       stream)
+{
+    if(!a || !x || !y || m == 0u || k == 0u)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(ncols != 1u && ncols != 2u && ncols != 4u && ncols != 8u)
+        return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+    if(k % 8u != 0u)
+        return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+    if(lda < k || ldx < k || ldy < m)
+        return ROCWMMA_AMD_BAD_LEADING_DIM;
+    if(!aligned16(a) || !aligned16(x) || lda % 8u != 0u || ldx % 8u != 0u || (reinterpret_cast<uintptr_t>(y) & 3u))
+        return ROCWMMA_AMD_BAD_ALIGNMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return launchGemv(m, k, ncols, a, lda, x, ldx, y, ldy, alpha, beta, asStream(stream));
+}
+
+static int checkDlrm(uint32_t m, uint32_t k, uint32_t batch)
+{
+    if(m == 0u || batch == 0u)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(m > 32u || (k != 32u && k != 64u && k != 128u && k != 256u))
+        return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+    return ROCWMMA_AMD_OK;
+}
+
+int rocwmma_amd_dlrm_fwd(const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, void* stream)
+{
+    if(!input || !output)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    int rc = checkDlrm(m, k, batch);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(!aligned16(input) || !aligned16(output))
+        return ROCWMMA_AMD_BAD_ALIGNMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return launchDlrmFwd(input, output, m, k, batch, asStream(stream));
+}
+
+int rocwmma_amd_dlrm_bwd(const void* input,
+                         const void* upstream_grad,
+                         void*       grad,
+                         void*       bottom_mlp_grad,
+                         uint32_t    m,
+                         uint32_t    k,
+                         uint32_t    batch,
+                         void*       stream)
+{
+    if(!input || !upstream_grad || !grad || !bottom_mlp_grad)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    int rc = checkDlrm(m, k, batch);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(!aligned16(input) || !aligned16(upstream_grad) || !aligned16(grad) || !aligned16(bottom_mlp_grad))
+        return ROCWMMA_AMD_BAD_ALIGNMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return launchDlrmBwd(input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
+}
+
+int rocwmma_amd_selftest_roundtrip(int         context,
+                                   int         dtype,
+                                   int         layout,
+                                   int         block,
+                                   int         blockk,
+                                   int         coop,
+                                   uint32_t    rows,
+                                   uint32_t    cols,
+                                   const void* in,
+                                   void*       out,
+                                   uint32_t    ld,
+                                   void*       stream)
+{
+    if(!in || !out || rows == 0u || cols == 0u || !validLayout(layout))
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(!aligned16(in) || !aligned16(out) || (ld * dtypeSize(dtype)) % 16u != 0u)
+        return ROCWMMA_AMD_BAD_ALIGNMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return selftestRoundtrip(context, dtype, layout, block, blockk, coop, rows, cols, in, out, ld, asStream(stream));
+}
+
+int rocwmma_amd_selftest_coop_gemm(int          layout_a,
+                                   int          layout_b,
+                                   uint32_t     m,
+                                   uint32_t     n,
+                                   uint32_t     k,
+                                   const void*  a,
+                                   const void*  b,
+                                   const float* c,
+                                   float*       d,
+                                   float        alpha,
+                                   float        beta,
+                                   void*        stream)
+{
+    if(!a || !b || !c || !d || !validLayout(layout_a) || !validLayout(layout_b))
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return selftestCoopGemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta, asStream(stream));
+}
+
+} // extern "C"

@@ -1,0 +1,71 @@
+// Host-side helpers shared by the workload translation units of librocwmma_amd.so.
+#ifndef ROCWMMA_AMD_CSRC_COMMON_HPP
+#define ROCWMMA_AMD_CSRC_COMMON_HPP
+
+#include <cstdint>
+#include <hip/hip_runtime.h>
+
+#include <rocwmma/rocwmma.hpp>
+#include <rocwmma_amd.h>
+
+static_assert(ROCWMMA_AMD_GFX950_NATIVE == 1,
+              "the toolchain's own rocWMMA headers were picked up: put -I<repo>/include first");
+
+namespace rocwmma_amd
+{
+    inline hipStream_t asStream(void* stream)
+    {
+        return reinterpret_cast<hipStream_t>(stream);
+    }
+
+    inline bool aligned16(const void* p)
+    {
+        return (reinterpret_cast<uintptr_t>(p) & 15u) == 0u;
+    }
+
+    inline uint32_t dtypeSize(int dtype)
+    {
+        switch(dtype)
+        {
+        case ROCWMMA_AMD_F16:
+        case ROCWMMA_AMD_BF16:
+            return 2;
+        case ROCWMMA_AMD_E4M3:
+        case ROCWMMA_AMD_E5M2:
+        case ROCWMMA_AMD_I8:
+            return 1;
+        case ROCWMMA_AMD_F32:
+        case ROCWMMA_AMD_I32:
+            return 4;
+        default:
+            return 0;
+        }
+    }
+
+    inline int launchStatus()
+    {
+        return hipGetLastError() == hipSuccess ? ROCWMMA_AMD_OK : ROCWMMA_AMD_LAUNCH_FAILED;
+    }
+
+    // Argument block every GEMM kernel family takes: the reference kernels' argument list
+    // (m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta) plus the run-time C/D layout.
+    struct GemmArgs
+    {
+        uint32_t    m, n, k;
+        const void* a;
+        const void* b;
+        const void* c;
+        void*       d;
+        uint32_t    lda, ldb, ldc, ldd;
+        float       alpha, beta;
+        int         layoutC;
+    };
+
+    // Family launchers (one translation unit each).  Return a rocwmma_amd_status;
+    // ROCWMMA_AMD_UNSUPPORTED_SHAPE / _TYPE mean "this family has no kernel for it".
+    int launchGemmWaveTile(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
+    int launchGemmBlocked(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
+
+} // namespace rocwmma_amd
+
+#endif // ROCWMMA_AMD_CSRC_COMMON_HPP

@@ -1,0 +1,102 @@
+"""DLRM dot-interaction parity: the HIP kernels against the reference's golden files and the
+CPU oracle (dlrm_fwd_CPU / dlrm_bwd_CPU, test/reference_impl.hpp:83-179).
+Tolerance: 10 * eps(f16) in the compareEqual metric (test/dlrm/dlrm_kernel_base_impl.hpp:472-478)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle as orc
+import rocwmma_amd as rw
+from util import to_device, uniform_bits
+
+pytestmark = pytest.mark.gpu
+TOL = 10 * 2.0 ** -10
+
+
+def gpu_fwd(inp, m, k, b):
+    import torch
+
+    width = k + m * (m - 1) // 2
+    out = to_device(np.full(b * width, 0x7E00, dtype=np.uint16))
+    rw.dlrm_fwd(to_device(inp), out, m, k, b)
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16).reshape(b, width)
+
+
+def gpu_bwd(inp, up, m, k, b):
+    import torch
+
+    grad = to_device(np.full(b * m * k, 0x7E00, dtype=np.uint16))
+    mlp = to_device(np.full(b * k, 0x7E00, dtype=np.uint16))
+    rw.dlrm_bwd(to_device(inp), to_device(up), grad, mlp, m, k, b)
+    torch.cuda.synchronize()
+    return (grad.cpu().numpy().view(np.uint16).reshape(b, m, k), mlp.cpu().numpy().view(np.uint16).reshape(b, k))
+
+
+def close(got, want, tol=TOL):
+    err, inf, nan = orc.compare_equal(orc.F16, got, orc.F16, want)
+    assert not inf and not nan and err <= tol, (err, inf, nan)
+    return err
+
+
+def _golden(golden_dir, name, shape):
+    return np.fromfile(os.path.join(golden_dir, f"dlrm_{name}.bin"), dtype=np.uint16).reshape(shape)
+
+
+def test_forward_against_reference_golden_files(golden_dir):
+    b, m, k = 64, 27, 128
+    inp = _golden(golden_dir, "input_fp16", (b, m, k))
+    want = _golden(golden_dir, "output_fp16", (b, k + m * (m - 1) // 2))
+    got = gpu_fwd(inp, m, k, b)
+    close(got, want)
+    assert np.array_equal(got[:, :k], inp[:, 0, :])
+    close(got, orc.dlrm_fwd(inp, m, k, b))
+
+
+def test_backward_against_reference_golden_files(golden_dir):
+    b, m, k = 64, 27, 128
+    inp = _golden(golden_dir, "input_fp16", (b, m, k))
+    up = _golden(golden_dir, "input_grad_fp16", (b, k + m * (m - 1) // 2))
+    grad, mlp = gpu_bwd(inp, up, m, k, b)
+    assert np.array_equal(mlp, _golden(golden_dir, "output_mlp_input_grad_fp16", (b, k)))
+    close(grad, _golden(golden_dir, "output_input_grad_fp16", (b, m, k)))
+    wgrad, wmlp = orc.dlrm_bwd(inp, up, m, k, b)
+    close(grad, wgrad)
+    assert np.array_equal(mlp, wmlp)
+
+
+@pytest.mark.parametrize("b,m,k", [(2048, 27, 128), (13, 27, 128), (1, 27, 128), (40, 32, 128), (24, 5, 64),
+                                   (9, 16, 32), (17, 2, 256), (8, 1, 128)])
+def test_forward_and_backward_against_oracle(b, m, k):
+    width = k + m * (m - 1) // 2
+    inp = uniform_bits(0x5EED0005 + b, orc.F16, b * m * k)
+    up = uniform_bits(0x5EED0105 + b, orc.F16, b * width)
+    got = gpu_fwd(inp, m, k, b)
+    close(got, orc.dlrm_fwd(inp, m, k, b))
+    grad, mlp = gpu_bwd(inp, up, m, k, b)
+    wgrad, wmlp = orc.dlrm_bwd(inp, up, m, k, b)
+    close(grad, wgrad)
+    assert np.array_equal(mlp, wmlp)
+
+
+def test_backward_is_linear_in_upstream_gradient():
+    """Scaling the upstream gradient by a power of two scales grad exactly (size-independent
+    property, checked at a batch the oracle would take long on)."""
+    b, m, k = 16384, 27, 128
+    width = k + m * (m - 1) // 2
+    inp = uniform_bits(1, orc.F16, b * m * k)
+    up = uniform_bits(2, orc.F16, b * width)
+    g1, _ = gpu_bwd(inp, up, m, k, b)
+    half = (up.view(np.float16) * np.float16(0.5)).view(np.uint16)
+    g2, _ = gpu_bwd(inp, half, m, k, b)
+    assert np.array_equal(g2.view(np.float16), g1.view(np.float16) * np.float16(0.5))
+    # forward: Gram matrix entries are symmetric in the two rows -> permuting rows 1 and 2 of
+    # every sample swaps the corresponding outputs
+    f1 = gpu_fwd(inp, m, k, b)
+    perm = inp.reshape(b, m, k).copy()
+    perm[:, [1, 2]] = perm[:, [2, 1]]
+    f2 = gpu_fwd(perm, m, k, b)
+    assert np.array_equal(f2[:, k + 0], f1[:, k + 1])            # new Z[1,0] = F2.F0 = old Z[2,0]
+    assert np.array_equal(f2[:, k + 1], f1[:, k + 0])            # new Z[2,0] = F1.F0 = old Z[1,0]
+    assert np.array_equal(f2[:, k + 2], f1[:, k + 2])            # Z[2,1] is symmetric under the swap

@@ -1,0 +1,214 @@
+"""GEMM parity on the GPU: the HIP kernels (through the C ABI) against the CPU oracle on the same
+seeded bits.  Bar: int8 -> int32 bit-exact; f16 / bf16 <= 1e-3 and fp8 <= 1e-2 in the reference's
+compareEqual metric (max |a-b| / (|a|+|b|+1)); the exact-integer fill pattern must match bit for
+bit for every type."""
+import numpy as np
+import pytest
+
+import oracle as orc
+import rocwmma_amd as rw
+from util import CM, RM, exact_int_bits, normal_fp8_bits, to_device, to_host, tol_for, uniform_bits
+
+pytestmark = pytest.mark.gpu
+
+OUT_OF = {orc.F16: orc.F32, orc.BF16: orc.F32, orc.E4M3: orc.F32, orc.E5M2: orc.F32, orc.I8: orc.I32}
+
+
+def run_gemm(dtype_in, dtype_out, la, lb, lc, m, n, k, a, b, c, alpha, beta, algo):
+    import torch
+
+    np_out = orc.storage_dtype(dtype_out)
+    # D pre-filled with NaN / a sentinel so unwritten elements are caught
+    if dtype_out == orc.F32:
+        d0 = np.full(m * n, np.nan, dtype=np.float32)
+    elif dtype_out == orc.I32:
+        d0 = np.full(m * n, -123456789, dtype=np.int32)
+    else:
+        d0 = np.full(m * n, 0x7E00, dtype=np.uint16)
+    d = to_device(d0)
+    rw.gemm(dtype_in, dtype_out, la, lb, lc, m, n, k, to_device(a), to_device(b),
+            None if c is None else to_device(c), d, alpha, beta, algo=algo)
+    torch.cuda.synchronize()
+    return to_host(d, np_out)
+
+
+def check(dtype_in, dtype_out, got, want, tol):
+    if tol == 0.0:
+        assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} elements differ"
+        return 0.0
+    err, inf, nan = orc.compare_equal(dtype_out, got, dtype_out, want)
+    assert not inf and not nan, (inf, nan)
+    assert err <= tol, f"max relative error {err} > {tol}"
+    return err
+
+
+# ---------------------------------------------------------------- config 1: simple_hgemm workload
+@pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED, rw.GEMM_AUTO])
+def test_config1_256_cubed_f16_alpha_beta_2(algo):
+    m = n = k = 256
+    a = uniform_bits(0x5EED0001, orc.F16, m * k)
+    b = uniform_bits(0x5EED0101, orc.F16, k * n)
+    c = np.random.default_rng(0x5EED0201).uniform(-1, 1, m * n).astype(np.float32)
+    got = run_gemm(orc.F16, orc.F32, RM, CM, RM, m, n, k, a, b, c, 2.0, 2.0, algo)
+    want = orc.gemm(orc.F16, orc.F32, RM, CM, RM, RM, m, n, k, a, b, c, 2.0, 2.0)
+    check(orc.F16, orc.F32, got, want, 1e-3)
+
+
+# ---------------------------------------------------------------- all types x layouts, both families
+@pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED])
+@pytest.mark.parametrize("lc", [RM, CM])
+@pytest.mark.parametrize("lb", [RM, CM])
+@pytest.mark.parametrize("la", [RM, CM])
+@pytest.mark.parametrize("dtype_in", [orc.F16, orc.BF16])
+def test_16bit_types_all_layouts(dtype_in, la, lb, lc, algo):
+    m, n, k = 256, 384, 192
+    a = uniform_bits(21, dtype_in, m * k)
+    b = uniform_bits(22, dtype_in, k * n)
+    c = np.random.default_rng(23).uniform(-1, 1, m * n).astype(np.float32)
+    got = run_gemm(dtype_in, orc.F32, la, lb, lc, m, n, k, a, b, c, 1.0, 1.0, algo)
+    want = orc.gemm(dtype_in, orc.F32, la, lb, lc, lc, m, n, k, a, b, c, 1.0, 1.0)
+    check(dtype_in, orc.F32, got, want, 1e-3)
+
+
+@pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED])
+@pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3, orc.E5M2])
+def test_8bit_types_k_contiguous(dtype_in, algo):
+    m, n, k = 256, 256, 512
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(31, orc.I8, m * k), uniform_bits(32, orc.I8, k * n)
+        c = uniform_bits(33, orc.I32, m * n)
+        alpha, beta = 1.0, 0.0
+    else:
+        a, b = normal_fp8_bits(31, dtype_in, m * k), normal_fp8_bits(32, dtype_in, k * n)
+        c = np.random.default_rng(33).uniform(-1, 1, m * n).astype(np.float32)
+        alpha, beta = 1.0, 0.0
+    out = OUT_OF[dtype_in]
+    got = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, c, alpha, beta, algo)
+    want = orc.gemm(dtype_in, out, RM, CM, RM, RM, m, n, k, a, b, c, alpha, beta)
+    check(dtype_in, out, got, want, tol_for(dtype_in))
+    # beta != 0 path
+    got = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, c, 2.0, 3.0, algo)
+    want = orc.gemm(dtype_in, out, RM, CM, RM, RM, m, n, k, a, b, c, 2.0, 3.0)
+    check(dtype_in, out, got, want, tol_for(dtype_in))
+
+
+@pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3])
+@pytest.mark.parametrize("la,lb", [(RM, RM), (CM, CM), (CM, RM)])
+def test_8bit_types_other_layouts_wave_tile(dtype_in, la, lb):
+    m, n, k = 64, 96, 256
+    a = uniform_bits(41, orc.I8, m * k) if dtype_in == orc.I8 else normal_fp8_bits(41, dtype_in, m * k)
+    b = uniform_bits(42, orc.I8, k * n) if dtype_in == orc.I8 else normal_fp8_bits(42, dtype_in, k * n)
+    out = OUT_OF[dtype_in]
+    got = run_gemm(dtype_in, out, la, lb, RM, m, n, k, a, b, None, 1.0, 0.0, rw.GEMM_AUTO)
+    want = orc.gemm(dtype_in, out, la, lb, RM, RM, m, n, k, a, b, None, 1.0, 0.0)
+    check(dtype_in, out, got, want, tol_for(dtype_in))
+
+
+@pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED])
+@pytest.mark.parametrize("dtype_in", [orc.F16, orc.BF16, orc.E4M3, orc.E5M2, orc.I8])
+def test_exact_integer_pattern_is_bit_exact(dtype_in, algo):
+    """The reference's fill makes every partial sum an exact integer, so any summation order
+    must reproduce the CPU result bit for bit (all types, not only int8)."""
+    m, n, k = 256, 256, 1024
+    a = exact_int_bits(dtype_in, m, k, RM)
+    b = exact_int_bits(dtype_in, k, n, CM)
+    out = OUT_OF[dtype_in]
+    c = exact_int_bits(out, m, n, RM)
+    got = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, c, 2.0, 2.0, algo)
+    want = orc.gemm(dtype_in, out, RM, CM, RM, RM, m, n, k, a, b, c, 2.0, 2.0)
+    assert np.array_equal(got, want)
+
+
+def test_narrow_k_and_small_tiles_wave_tile():
+    """K that only the half-width instructions divide, 16-wide blocks, f16 output."""
+    for (m, n, k) in [(16, 48, 48), (32, 32, 24), (48, 16, 16), (64, 64, 40)]:
+        a = uniform_bits(51, orc.F16, m * k)
+        b = uniform_bits(52, orc.F16, k * n)
+        c = np.random.default_rng(53).uniform(-1, 1, m * n).astype(np.float32)
+        got = run_gemm(orc.F16, orc.F32, RM, CM, RM, m, n, k, a, b, c, 2.0, 2.0, rw.GEMM_AUTO)
+        want = orc.gemm(orc.F16, orc.F32, RM, CM, RM, RM, m, n, k, a, b, c, 2.0, 2.0)
+        check(orc.F16, orc.F32, got, want, 1e-3)
+    m, n, k = 64, 64, 64
+    a, b = uniform_bits(54, orc.F16, m * k), uniform_bits(55, orc.F16, k * n)
+    c = uniform_bits(56, orc.F16, m * n)
+    got = run_gemm(orc.F16, orc.F16, RM, CM, RM, m, n, k, a, b, c, 2.0, 2.0, rw.GEMM_AUTO)
+    want = orc.gemm(orc.F16, orc.F16, RM, CM, RM, RM, m, n, k, a, b, c, 2.0, 2.0)
+    err, inf, nan = orc.compare_equal(orc.F16, got, orc.F16, want)
+    assert not inf and not nan and err <= 10 * 2.0 ** -10
+
+
+def test_leading_dimensions_larger_than_extent():
+    """Padded leading dimensions: only the m x n window of D may be written."""
+    import torch
+
+    m, n, k = 256, 256, 128
+    lda, ldb, ldc = k + 64, k + 32, n + 16
+    rng = np.random.default_rng(61)
+    A = orc.encode(orc.F16, rng.uniform(-1, 1, (m, lda)).astype(np.float32))
+    B = orc.encode(orc.F16, rng.uniform(-1, 1, (n, ldb)).astype(np.float32))  # col-major B: n columns of ldb
+    C = rng.uniform(-1, 1, (m, ldc)).astype(np.float32)
+    for algo in (rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED):
+        d = torch.full((m, ldc), 777.0, device="cuda")
+        rw.gemm(orc.F16, orc.F32, RM, CM, RM, m, n, k, to_device(A), to_device(B), to_device(C), d, 1.0, 1.0,
+                lda=lda, ldb=ldb, ldc=ldc, ldd=ldc, algo=algo)
+        torch.cuda.synchronize()
+        got = d.cpu().numpy()
+        want = orc.gemm(orc.F16, orc.F32, RM, CM, RM, RM, m, n, k, A[:, :k], B[:, :k], C[:, :n], 1.0, 1.0)
+        check(orc.F16, orc.F32, np.ascontiguousarray(got[:, :n]).reshape(-1), want, 1e-3)
+        assert np.all(got[:, n:] == 777.0)
+
+
+# ---------------------------------------------------------------- config 3: quantised shapes
+@pytest.mark.parametrize("m", [16, 128, 4096])
+@pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3])
+def test_config3_quantised_inference_shapes(dtype_in, m):
+    n, k = 14336, 4096
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(0x5EED0003, orc.I8, m * k), uniform_bits(0x5EED0103, orc.I8, k * n)
+    else:
+        a, b = normal_fp8_bits(0x5EED0003, dtype_in, m * k), normal_fp8_bits(0x5EED0103, dtype_in, k * n)
+    out = OUT_OF[dtype_in]
+    got = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, None, 1.0, 0.0, rw.GEMM_AUTO)
+    # every element for M = 16 / 128; a seeded sample of 64 full rows for M = 4096
+    rows = None if m <= 128 else np.sort(np.random.default_rng(7).choice(m, 64, replace=False)).astype(np.uint32)
+    want = orc.gemm(dtype_in, out, RM, CM, RM, RM, m, n, k, a, b, None, 1.0, 0.0, rows=rows)
+    if rows is None:
+        check(dtype_in, out, got, want, tol_for(dtype_in))
+    else:
+        check(dtype_in, out, got.reshape(m, n)[rows].reshape(-1), want.reshape(m, n)[rows].reshape(-1),
+              tol_for(dtype_in))
+
+
+# ---------------------------------------------------------------- config 2: 8192^3, 4 layouts x 2 types
+@pytest.mark.parametrize("la", [RM, CM])
+@pytest.mark.parametrize("lb", [RM, CM])
+@pytest.mark.parametrize("dtype_in", [orc.F16, orc.BF16])
+def test_config2_8192_cubed_sampled_rows(dtype_in, la, lb):
+    """Full-size case: 64 seeded output rows are recomputed by the oracle (same dot-product
+    loop, every column), plus a row-sum identity over the whole result."""
+    import torch
+
+    m = n = k = 8192
+    g = torch.Generator(device="cuda").manual_seed(0x5EED0002 + 8 * dtype_in + 2 * la + lb)
+    tdt = torch.float16 if dtype_in == orc.F16 else torch.bfloat16
+    A = (torch.rand(m * k, device="cuda", generator=g) * 2 - 1).to(tdt)
+    B = (torch.rand(k * n, device="cuda", generator=g) * 2 - 1).to(tdt)
+    C = torch.rand(m * n, device="cuda", generator=g) * 2 - 1
+    D = torch.full((m * n,), float("nan"), device="cuda")
+    rw.gemm(dtype_in, orc.F32, la, lb, RM, m, n, k, A, B, C, D, 1.0, 1.0)
+    torch.cuda.synchronize()
+    assert not torch.isnan(D).any()
+    rows = np.sort(np.random.default_rng(9).choice(m, 64, replace=False)).astype(np.uint32)
+    a_bits = A.view(torch.int16).cpu().numpy().view(np.uint16)
+    b_bits = B.view(torch.int16).cpu().numpy().view(np.uint16)
+    c_host = C.cpu().numpy()
+    want = orc.gemm(dtype_in, orc.F32, la, lb, RM, RM, m, n, k, a_bits, b_bits, c_host, 1.0, 1.0, rows=rows)
+    got = D.cpu().numpy().reshape(m, n)[rows]
+    check(dtype_in, orc.F32, got.reshape(-1), want.reshape(m, n)[rows].reshape(-1), 1e-3)
+    # size-independent property: D 1 = A (B 1) + C 1 (float64 on the device, whole matrix)
+    Am = (A.view(m, k) if la == RM else A.view(k, m).t()).double()
+    Bm = (B.view(k, n) if lb == RM else B.view(n, k).t()).double()
+    ones = torch.ones(n, 1, dtype=torch.float64, device="cuda")
+    lhs = D.view(m, n).double() @ ones
+    rhs = Am @ (Bm @ ones) + C.view(m, n).double() @ ones
+    assert torch.allclose(lhs, rhs, rtol=0, atol=0.5), float((lhs - rhs).abs().max())
