@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[1]): D = A*B + C at M = N = K = 8192 with f16 and with
+bf16 inputs, f32 C/D, all four A/B layout combinations.  One "step" is one pass over those
+eight GEMMs; the reported value is total flops / total time in TFLOP/s (2*M*N*K per GEMM,
+reference formula test/performance.hpp:424-433).  Inputs are synthetic, uniform[-1, 1], already
+resident in HBM when the timed region starts.
+
+Prints ONE JSON line.  Besides the contract fields it carries
+  roofline     : the dominant kernel (f16, A row-major, B col-major) against the 2.5 PFLOP/s dense
+                 f16 MFMA peak, timed with events on the launch stream;
+  cpu_baseline : the CPU oracle (a port of the reference's OpenMP gemm_CPU) timed on this box's
+                 host cores on a bounded sample of the same workload;
+  extra        : the other configurations (quantised GEMMs, GEMV, DLRM) with their own rooflines.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0, "i8": 5000.0}  # dense MFMA, MI355X
+PEAK_HBM_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--size", type=int, default=8192, help="M = N = K of the headline GEMM")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--only", default=None,
+                    help="run one headline case only, e.g. f16_rc (dtype_{r|c}{r|c} = A,B layout): for profiling")
+    return ap.parse_args()
+
+
+def event_ms(fn, iters, torch):
+    """Average duration of fn() in ms over `iters` launches, events on the current stream."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import rocwmma_amd as rw
+
+    if not os.path.exists(rw.library_path()):
+        import __graft_entry__ as g
+
+        g.build()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    info = rw.device_info()
+    assert info["is_gfx950"], info
+    dev = torch.device("cuda:0")
+    RM, CM = rw.ROW_MAJOR, rw.COL_MAJOR
+    S = args.size
+    gen = torch.Generator(device=dev).manual_seed(0x5EED0002)
+
+    def rand(count, dtype):
+        return (torch.rand(count, device=dev, generator=gen) * 2 - 1).to(dtype)
+
+    # ------------------------------------------------------------------ headline: 8 GEMMs
+    data = {
+        "f16": (rw.F16, rand(S * S, torch.float16), rand(S * S, torch.float16)),
+        "bf16": (rw.BF16, rand(S * S, torch.bfloat16), rand(S * S, torch.bfloat16)),
+    }
+    C = rand(S * S, torch.float32)
+    D = torch.empty(S * S, device=dev, dtype=torch.float32)
+    cases = []
+    for name, (code, A, B) in data.items():
+        for la in (RM, CM):
+            for lb in (RM, CM):
+                tag = f"{name}_{'rc'[la]}{'rc'[lb]}"
+                if args.only and tag != args.only:
+                    continue
+                cases.append((tag, code, la, lb, A, B))
+    assert cases, f"no case matches --only {args.only}"
+
+    def run_case(case):
+        _, code, la, lb, A, B = case
+        rw.gemm(code, rw.F32, la, lb, RM, S, S, S, A, B, C, D, 1.0, 1.0)
+
+    def step():
+        for case in cases:
+            run_case(case)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    flops_per_gemm = 2.0 * S * S * S
+    value = flops_per_gemm * len(cases) / (ms_per_step * 1e-3) / 1e12
+
+    # per-case kernel time (events on the launch stream)
+    per_case = {}
+    for case in cases:
+        ms = event_ms(lambda: run_case(case), max(args.steps, 5), torch)
+        per_case[case[0]] = {"ms": round(ms, 4), "tflops": round(flops_per_gemm / ms / 1e9, 1)}
+    dom = "f16_rc" if "f16_rc" in per_case else cases[0][0]
+    dom_peak = PEAK_TFLOPS["bf16" if dom.startswith("bf16") else "f16"]
+    roofline = {
+        "bound": "mfma", "kernel": f"gemmBlockedKernel {dom} {S}^3",
+        "achieved": per_case[dom]["tflops"], "peak": dom_peak, "unit": "TFLOP/s",
+        "frac": round(per_case[dom]["tflops"] / dom_peak, 4), "traffic": None,
+        "ms": per_case[dom]["ms"],
+    }
+
+    # ------------------------------------------------------------------ CPU baseline (oracle port)
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        import oracle as orc
+
+        rows_n = 1024 if S >= 4096 else S
+        rows = np.arange(0, S, S // rows_n, dtype=np.uint32)[:rows_n]
+        code, A, B = data["f16"]
+        a_bits = A.view(torch.int16).cpu().numpy().view(np.uint16)
+        b_bits = B.view(torch.int16).cpu().numpy().view(np.uint16)
+        c_host = C.cpu().numpy()
+        t0 = time.perf_counter()
+        orc.gemm(orc.F16, orc.F32, 0, 1, 0, 0, S, S, S, a_bits, b_bits, c_host, 1.0, 1.0, rows=rows)
+        dt = time.perf_counter() - t0
+        cpu_baseline = {
+            "value": round(2.0 * rows.size * S * S / dt / 1e12, 5), "unit": "TFLOP/s",
+            "cores": orc.num_threads(), "kind": "port",
+            "sample": f"{rows.size} of {S} output rows (every column) of the f16 A-row/B-col {S}^3 case, "
+                      f"{dt:.1f} s incl. operand decode",
+        }
+        del a_bits, b_bits, c_host
+
+    # ------------------------------------------------------------------ other configurations
+    extra = {"device": info, "cases": per_case}
+    if not args.no_extras and not args.only:
+        extra.update(run_extras(rw, torch, dev, gen, args))
+
+    print(json.dumps({
+        "metric": "gemm_tflops_8192cubed_f16_bf16_4layouts", "value": round(value, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16/bf16 in, f32 accumulate",
+        "data": "synthetic uniform[-1,1], resident in HBM",
+        "config": {"workload": f"D = A*B + C, M=N=K={S}, f16 and bf16 inputs, f32 C/D, A,B in row/col x row/col "
+                               f"({len(cases)} GEMMs per step), alpha=beta=1"},
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "extra": extra,
+    }))
+
+
+def run_extras(rw, torch, dev, gen, args):
+    """Quantised GEMMs (config 3), GEMV (config 4), DLRM (config 5): kernel time by events."""
+    RM, CM = rw.ROW_MAJOR, rw.COL_MAJOR
+    out = {}
+    iters = 20
+
+    # config 3: N = 14336, K = 4096, M in {16, 128, 4096}; int8 and e4m3, A row / B col
+    n, k = 14336, 4096
+    Bq = torch.randint(-128, 128, (k * n,), device=dev, dtype=torch.int8, generator=gen)
+    Bf = (torch.randn(k * n, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+    for m in (16, 128, 4096):
+        Aq = torch.randint(-128, 128, (m * k,), device=dev, dtype=torch.int8, generator=gen)
+        Af = (torch.randn(m * k, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+        Di = torch.empty(m * n, device=dev, dtype=torch.int32)
+        Df = torch.empty(m * n, device=dev, dtype=torch.float32)
+        flops = 2.0 * m * n * k
+        for tag, code, ocode, A, B, Dx in (("i8", rw.I8, rw.I32, Aq, Bq, Di), ("fp8", rw.E4M3, rw.F32, Af, Bf, Df)):
+            fn = lambda: rw.gemm(code, ocode, RM, CM, RM, m, n, k, A, B, None, Dx, 1.0, 0.0)
+            fn()
+            ms = event_ms(fn, iters, torch)
+            byts = m * k + n * k + 4.0 * m * n
+            out[f"gemm_{tag}_m{m}"] = {
+                "ms": round(ms, 4), "tops": round(flops / ms / 1e9, 1),
+                "frac_mfma": round(flops / ms / 1e9 / PEAK_TFLOPS[tag], 4),
+                "gbs": round(byts / ms / 1e6, 1), "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4),
+            }
+
+    # config 4: GEMV, buffers rotated over > 512 MB so the 256 MB Infinity Cache cannot serve A
+    for (m, kk) in ((8192, 8192), (14336, 4096)):
+        copies = 5
+        As = [(torch.rand(m * kk, device=dev, generator=gen) * 2 - 1).to(torch.float16) for _ in range(copies)]
+        for ncols in (1, 4, 8):
+            x = (torch.rand(kk * ncols, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+            y = torch.zeros(m * ncols, device=dev)
+            state = {"i": 0}
+
+            def fn():
+                rw.gemv(m, kk, ncols, As[state["i"] % copies], x, y, 1.0, 0.0)
+                state["i"] += 1
+
+            fn()
+            ms = event_ms(fn, iters, torch)
+            byts = 2.0 * m * kk + 2.0 * kk * ncols + 4.0 * m * ncols
+            out[f"gemv_{m}x{kk}_n{ncols}"] = {"ms": round(ms, 5), "gbs": round(byts / ms / 1e6, 1),
+                                             "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        del As
+
+    # config 5: DLRM, batch 2048 (cache resident, latency bound) and a batch that streams from HBM
+    mm, kd = 27, 128
+    width = kd + mm * (mm - 1) // 2
+    for batch, copies in ((2048, 1), (262144, 3)):
+        Fs = [(torch.rand(batch * mm * kd, device=dev, generator=gen) * 2 - 1).to(torch.float16) for _ in range(copies)]
+        up = (torch.rand(batch * width, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        o = torch.empty(batch * width, device=dev, dtype=torch.float16)
+        gr = torch.empty(batch * mm * kd, device=dev, dtype=torch.float16)
+        mg = torch.empty(batch * kd, device=dev, dtype=torch.float16)
+        state = {"i": 0}
+
+        def fwd():
+            rw.dlrm_fwd(Fs[state["i"] % copies], o, mm, kd, batch)
+            state["i"] += 1
+
+        def bwd():
+            rw.dlrm_bwd(Fs[state["i"] % copies], up, gr, mg, mm, kd, batch)
+            state["i"] += 1
+
+        fwd(), bwd()
+        ms_f = event_ms(fwd, iters, torch)
+        ms_b = event_ms(bwd, iters, torch)
+        bf = batch * (mm * kd * 2.0 + width * 2.0)
+        bb = batch * (mm * kd * 2.0 + width * 2.0 + mm * kd * 2.0 + kd * 2.0)
+        out[f"dlrm_fwd_b{batch}"] = {"ms": round(ms_f, 5), "gbs": round(bf / ms_f / 1e6, 1),
+                                     "frac_hbm": round(bf / ms_f / 1e6 / PEAK_HBM_GBS, 4)}
+        out[f"dlrm_bwd_b{batch}"] = {"ms": round(ms_b, 5), "gbs": round(bb / ms_b / 1e6, 1),
+                                     "frac_hbm": round(bb / ms_b / 1e6 / PEAK_HBM_GBS, 4)}
+        del Fs
+    return out
+
+
+if __name__ == "__main__":
+    main()

@@ -23,7 +23,13 @@ namespace rocwmma_amd
         {
 #pragma unroll
             for(int i = 0; i < 4; ++i)
-                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a[i]), __builtin_bit_cast(half2_t, x[i]), acc, false);
+            {
+                // copy the lanes out first: a bit cast applied directly to a vector element
+                // reads the vector's first word
+                const uint32_t ai = a[i];
+                const uint32_t xi = x[i];
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, ai), __builtin_bit_cast(half2_t, xi), acc, false);
+            }
             return acc;
         }
 

@@ -64,7 +64,7 @@ def test_cooperative_lds_gemm_flow_matches_oracle(la, lb):
     applyTranspose, LDS, mma_sync)."""
     import torch
 
-    m, n, k = 128, 192, 160
+    m, n, k = 128, 256, 160
     a = uniform_bits(11, orc.F16, m * k)
     b = uniform_bits(12, orc.F16, k * n)
     c = np.random.default_rng(13).uniform(-1, 1, m * n).astype(np.float32)
@@ -84,7 +84,7 @@ def test_cooperative_flow_exact_on_integer_pattern(la, lb):
 
     from util import exact_int_bits
 
-    m, n, k = 64, 64, 256
+    m, n, k = 128, 128, 256
     a = exact_int_bits(orc.F16, m, k, la)
     b = exact_int_bits(orc.F16, k, n, lb)
     c = exact_int_bits(orc.F32, m, n, RM)
@@ -92,4 +92,5 @@ def test_cooperative_flow_exact_on_integer_pattern(la, lb):
     rw.selftest_coop_gemm(la, lb, m, n, k, to_device(a), to_device(b), to_device(c), d, 2.0, 2.0)
     torch.cuda.synchronize()
     want = orc.gemm(orc.F16, orc.F32, la, lb, RM, RM, m, n, k, a, b, c, 2.0, 2.0)
-    assert np.array_equal(d.cpu().numpy(), want)
+    same = np.array_equal(d.cpu().numpy(), want)
+    assert same
