@@ -7,15 +7,16 @@
 //   * global_load_lds_dwordx4: each lane copies 16 bytes from global memory straight into
 //     LDS (lane i of the issuing wave lands at ldsBase + 16*i) without touching VGPRs;
 //   * LDS tiles whose 16-byte chunks are XOR-swizzled so that the ds_read_b128 of an MFMA
-//     operand (16 or 32 consecutive rows, same K chunk) touches every bank once;
+//     operand (32 consecutive rows, same K chunk) touches every bank once;
 //   * ds_read_b64_tr_b16 for operands stored with the non-K dimension contiguous
 //     (column-major A, row-major B): the transposing LDS read returns, to lane i of each
 //     16-lane group, the i-th column of a 4 x 16 block whose rows the lanes addressed.
 //
-// Two LDS tile formats, both for a macro-tile operand of `Dim` rows/columns by 128 bytes of K
-// (64 halves or 128 bytes) and both filled by whole-wave 1 KiB direct loads:
+// Two LDS tile formats for one pipeline stage of a macro-tile operand of `Dim` rows/columns
+// by RowBytes bytes of K (RowBytes = 64: 32 halves or 64 bytes), both filled by whole-wave
+// 1 KiB direct copies whose per-lane source offset does not depend on the copy index:
 //
-//   KMajorTile  -- one operand row per 128-byte LDS row (row-major A / col-major B).
+//   KMajorTile   -- one operand row per LDS row (row-major A / col-major B).
 //   DimMajorTile -- one K index per LDS row of Dim elements (col-major A / row-major B),
 //                   16-bit elements only.
 #ifndef ROCWMMA_LDS_HPP
@@ -37,57 +38,94 @@ namespace rocwmma
             __builtin_amdgcn_global_load_lds((GlobalPtr)src, (LdsPtr)ldsBase, 16, 0, 0);
         }
 
-        // Waits until all of this wave's direct-to-LDS copies (and other vector memory loads)
-        // have landed.  Follow with synchronize_workgroup() before other waves read the data.
-        ROCWMMA_DEVICE ROCWMMA_INLINE void asyncCopyWait()
+        // The same copy with buffer addressing: source address = resource base + waveOffset
+        // (scalar) + laneOffset (one VGPR).  Nothing but scalar arithmetic is needed per copy,
+        // which keeps the vector ALU and the VGPR file out of the copy path.
+        using BufferRsrc = __amdgpu_buffer_rsrc_t;
+
+        ROCWMMA_DEVICE ROCWMMA_INLINE BufferRsrc makeSource(const void* base)
         {
-            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0), expcnt / lgkmcnt untouched
+            // raw buffer, no stride, 2 GiB window from `base`, 32-bit data format
+            return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7FFFFFFF, 0x00020000);
+        }
+
+        ROCWMMA_DEVICE ROCWMMA_INLINE void asyncCopy16(void* ldsBase, BufferRsrc src, uint32_t laneOffset, uint32_t waveOffset)
+        {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                src, (LdsPtr)ldsBase, 16, static_cast<int>(laneOffset), static_cast<int>(waveOffset), 0, 0);
+        }
+
+        // s_waitcnt with "at most MaxLoads vector-memory operations still in flight" and all of
+        // this wave's LDS reads returned.  Direct-to-LDS copies complete in issue order, so
+        // leaving the newest MaxLoads outstanding means every older copy has landed.
+        template <uint32_t MaxLoads>
+        ROCWMMA_DEVICE ROCWMMA_INLINE void waitCopiesAndReads()
+        {
+            static_assert(MaxLoads < 64u, "vmcnt is a 6-bit counter");
+            // gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
+            constexpr uint32_t imm = (MaxLoads & 15u) | (7u << 4) | (0u << 8) | ((MaxLoads >> 4) << 14);
+            __builtin_amdgcn_s_waitcnt(imm);
+        }
+
+        // Waits until every LDS read this wave has issued has returned (vector-memory copies may
+        // stay in flight).  Needed before the registers filled by DimMajorTile::readBlock32 are
+        // used: those reads are issued outside the compiler's dependency tracking.
+        ROCWMMA_DEVICE ROCWMMA_INLINE void waitReads()
+        {
+            __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0), vmcnt / expcnt untouched
+        }
+
+        // Bare workgroup barrier (no implied memory waits: pair it with waitCopiesAndReads).
+        ROCWMMA_DEVICE ROCWMMA_INLINE void barrier()
+        {
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
         }
 
         // ---------------------------------------------------------------------------------
-        // K-major tile: Dim rows of 128 bytes; chunk c (16 bytes) of row r lives at chunk
-        // position c ^ swz(r).  swz makes any 8 consecutive rows and any 16 consecutive rows
-        // of one chunk column fall into distinct banks (32- and 64-bank views of the LDS).
+        // K-major stage: Dim rows of 64 bytes (four 16-byte chunks).  Chunk c of row r lives at
+        // chunk position c ^ swz(r); swz is chosen so that the 16 rows a quarter-wave reads in
+        // one ds_read_b128 fall into 16 distinct 16-byte bank groups (64 banks x 4 bytes), and
+        // any 8 aligned rows into 8 distinct groups of the 32-bank view.
         // ---------------------------------------------------------------------------------
         template <uint32_t Dim>
         struct KMajorTile
         {
-            static constexpr uint32_t rowBytes  = 128u;
-            static constexpr uint32_t chunks    = 8u;
-            static constexpr uint32_t bytes     = Dim * rowBytes;
-            static constexpr uint32_t waveLoads = bytes / 1024u; // whole-wave copies per tile
+            static constexpr uint32_t rowBytes    = 64u;
+            static constexpr uint32_t chunks      = 4u;
+            static constexpr uint32_t rowsPerCopy = 1024u / rowBytes; // 16
+            static constexpr uint32_t bytes       = Dim * rowBytes;
+            static constexpr uint32_t copies      = bytes / 1024u; // whole-wave copies per stage
 
             ROCWMMA_HOST_DEVICE static constexpr uint32_t swz(uint32_t row)
             {
-                return (row ^ (row >> 3)) & 7u;
+                return ((row >> 1) & 3u) ^ ((row >> 3) & 1u);
             }
             ROCWMMA_HOST_DEVICE static constexpr uint32_t offset(uint32_t row, uint32_t chunk)
             {
                 return row * rowBytes + ((chunk ^ swz(row)) << 4);
             }
-
-            // Wave `waveIndex` of `WaveCount` issues its share of the copies of one tile.
-            // `src` points at element (row 0, k 0) of the tile in global memory, rows
-            // `ldBytes` apart, K contiguous.
-            template <uint32_t WaveCount>
-            ROCWMMA_DEVICE static ROCWMMA_INLINE void
-                asyncLoad(char* ldsTile, const char* src, uint32_t ldBytes, uint32_t waveIndex, uint32_t lane)
+            // Source byte offset of `lane` inside any copy, relative to the copy's first row at
+            // the stage's first K byte: lane i owns LDS position (row i/4, chunk position i%4).
+            // (swz only looks at row bits 1..3, so the copy index does not matter.)
+            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t laneSourceOffset(uint32_t lane, uint32_t /*wave*/, uint32_t ldBytes)
             {
-                static_assert(waveLoads % WaveCount == 0u, "tile must split evenly over the waves");
-                // a copy covers 8 rows; lane i owns LDS position (row i/8, chunk position i%8)
-                const uint32_t rowInCopy = lane >> 3;
-                const uint32_t pos       = lane & 7u;
-#pragma unroll
-                for(uint32_t i = 0; i < waveLoads / WaveCount; ++i)
-                {
-                    const uint32_t copy  = i * WaveCount + waveIndex;
-                    const uint32_t row   = copy * 8u + rowInCopy;
-                    const uint32_t chunk = pos ^ swz(row);
-                    asyncCopy16(ldsTile + copy * 1024u, src + row * ldBytes + (chunk << 4));
-                }
+                const uint32_t row = lane >> 2;
+                return row * ldBytes + (((lane & 3u) ^ swz(row)) << 4);
+            }
+            // Source byte offset of copy `copy` (wave uniform)
+            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t copySourceOffset(uint32_t copy, uint32_t ldBytes)
+            {
+                return copy * rowsPerCopy * ldBytes;
+            }
+            // Bytes between consecutive stages along K in global memory
+            ROCWMMA_DEVICE static ROCWMMA_INLINE size_t stageStep(uint32_t /*ldBytes*/)
+            {
+                return rowBytes;
             }
 
-            // Reads the operand of one 32-wide MFMA block: rows [row0, row0+32), K step `ks`.
+            // Operand of one 32-wide MFMA block: rows [row0, row0+32), K step `ks` of the stage.
             // KPackBytes = bytes of K each lane holds per MFMA (16, or 32 for wide fp8).
             template <uint32_t KPackBytes>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
@@ -104,7 +142,7 @@ namespace rocwmma
         };
 
         // ---------------------------------------------------------------------------------
-        // Dim-major tile (16-bit elements): 64 LDS rows (one per K index) of Dim elements.
+        // Dim-major stage (16-bit elements): 32 LDS rows (one per K index) of Dim elements.
         // Rows are cut into 32-byte segments (16 elements); segment s of K row k lives at
         // segment position s ^ swz(k), which spreads the four K rows and two segments a
         // half-wave touches in one transposing read over all banks.
@@ -113,11 +151,15 @@ namespace rocwmma
         struct DimMajorTile
         {
             static_assert(Dim % 128u == 0u, "tile rows must hold at least eight 32-byte segments");
-            static constexpr uint32_t kRows     = 64u;
-            static constexpr uint32_t rowBytes  = Dim * 2u;
-            static constexpr uint32_t bytes     = kRows * rowBytes;
-            static constexpr uint32_t waveLoads = bytes / 1024u;
+            static constexpr uint32_t kRows       = 32u;
+            static constexpr uint32_t rowBytes    = Dim * 2u;
+            static constexpr uint32_t bytes       = kRows * rowBytes;
+            static constexpr uint32_t copies      = bytes / 1024u;
             static constexpr uint32_t slotsPerRow = rowBytes / 16u; // 16-byte copy slots per K row
+            static_assert(slotsPerRow <= 64u ? (64u % slotsPerRow == 0u) : (slotsPerRow % 64u == 0u),
+                          "a copy must cover whole K rows or an even part of one");
+            static constexpr uint32_t rowsPerCopy = slotsPerRow <= 64u ? 64u / slotsPerRow : 1u;
+            static_assert(slotsPerRow <= 64u, "tiles wider than 512 elements are not supported");
 
             ROCWMMA_HOST_DEVICE static constexpr uint32_t swz(uint32_t k)
             {
@@ -127,45 +169,52 @@ namespace rocwmma
             {
                 return k * rowBytes + ((seg ^ swz(k)) << 5);
             }
-
-            // `src` points at element (k 0, dim 0) of the tile, K rows `ldBytes` apart.
-            template <uint32_t WaveCount>
-            ROCWMMA_DEVICE static ROCWMMA_INLINE void
-                asyncLoad(char* ldsTile, const char* src, uint32_t ldBytes, uint32_t waveIndex, uint32_t lane)
+            // Source byte offset of `lane` inside a copy issued by wave `wave` of a pool whose
+            // size times rowsPerCopy is a multiple of 4 (so k & 3 is the same for all its copies).
+            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t laneSourceOffset(uint32_t lane, uint32_t wave, uint32_t ldBytes)
             {
-                static_assert(waveLoads % WaveCount == 0u, "tile must split evenly over the waves");
-                static_assert(slotsPerRow >= 64u ? (slotsPerRow % 64u == 0u) : (64u % slotsPerRow == 0u),
-                              "copy must cover whole or even parts of K rows");
-#pragma unroll
-                for(uint32_t i = 0; i < waveLoads / WaveCount; ++i)
-                {
-                    const uint32_t copy = i * WaveCount + waveIndex;
-                    const uint32_t slot = copy * 64u + lane; // global 16-byte slot index in the tile
-                    const uint32_t k    = slot / slotsPerRow;
-                    const uint32_t pos  = slot % slotsPerRow; // physical slot within the row
-                    const uint32_t seg  = (pos >> 1) ^ swz(k); // logical 32-byte segment
-                    asyncCopy16(ldsTile + copy * 1024u, src + k * ldBytes + (seg << 5) + ((pos & 1u) << 4));
-                }
+                const uint32_t kInCopy = lane / slotsPerRow;
+                const uint32_t pos     = lane % slotsPerRow;
+                const uint32_t k       = wave * rowsPerCopy + kInCopy; // only k & 3 matters
+                const uint32_t seg     = (pos >> 1) ^ swz(k);
+                return kInCopy * ldBytes + (seg << 5) + ((pos & 1u) << 4);
+            }
+            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t copySourceOffset(uint32_t copy, uint32_t ldBytes)
+            {
+                return copy * rowsPerCopy * ldBytes;
+            }
+            ROCWMMA_DEVICE static ROCWMMA_INLINE size_t stageStep(uint32_t ldBytes)
+            {
+                return static_cast<size_t>(kRows) * ldBytes;
             }
 
             // Operand of one 32-wide MFMA block with 8 K values per lane (v_mfma_*_32x32x16):
             // lane l ends up with dim = dim0 + l % 32 and k = ks*16 + (l/32)*8 + 0..7.
+            //
+            // The transposing reads are written as inline assembly on purpose: as compiler
+            // intrinsics they are assumed to alias every direct-to-LDS copy in flight and get a
+            // full vmcnt(0) wait in front of them, which serialises the copy pipeline.  The price
+            // is that the caller must call lds::waitReads() before the registers are consumed.
+            template <uint32_t KPackBytes = 16u>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
                 readBlock32(void* regs, const char* ldsTile, uint32_t dim0, uint32_t ks, uint32_t lane)
             {
+                static_assert(KPackBytes == 16u, "transposing reads feed the 8-halves-per-lane MFMA shapes");
                 typedef short s16x4 __attribute__((ext_vector_type(4)));
-                using LdsVec = __attribute__((address_space(3))) s16x4*;
-                const uint32_t group  = lane >> 4; // 16-lane group
-                const uint32_t s      = lane & 15u; // source index inside the group
-                const uint32_t seg    = (dim0 >> 4) + (group & 1u);
-                const uint32_t kBase  = ks * 16u + (group >> 1) * 8u + (s >> 2);
-                const uint32_t inSeg  = (s & 3u) << 3; // 4 elements = 8 bytes per source lane
+                const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsPtr)ldsTile));
+                const uint32_t group   = lane >> 4; // 16-lane group
+                const uint32_t s     = lane & 15u; // source index inside the group
+                const uint32_t seg   = (dim0 >> 4) + (group & 1u);
+                const uint32_t kBase = ks * 16u + (group >> 1) * 8u + (s >> 2);
+                const uint32_t inSeg = (s & 3u) << 3; // 4 elements = 8 bytes per source lane
 #pragma unroll
                 for(uint32_t kk = 0; kk < 2u; ++kk)
                 {
-                    const uint32_t k = kBase + kk * 4u;
-                    reinterpret_cast<s16x4*>(regs)[kk]
-                        = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsVec)(ldsTile + offset(k, seg) + inSeg));
+                    const uint32_t k    = kBase + kk * 4u;
+                    const uint32_t addr = ldsBase + offset(k, seg) + inSeg;
+                    s16x4          v;
+                    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+                    reinterpret_cast<s16x4*>(regs)[kk] = v;
                 }
             }
         };

@@ -219,6 +219,8 @@ namespace rocwmma_amd
                     {
                         FragF ff;
                         FTile::readBlock32(ff.x, tile, nb * 32u, ks, lane);
+                        lds::waitReads();
+                        __builtin_amdgcn_sched_barrier(0);
                         mma_sync(acc[nb], fg[ks], ff, acc[nb]);
                     }
                 }

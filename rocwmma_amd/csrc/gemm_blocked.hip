@@ -6,12 +6,13 @@
 // re-plumbed for CDNA4:
 //
 //   reference (gfx9 params)                      this kernel
-//   macro tile 128 x 128 x 16, 4 waves           256 x 256 x (128 bytes of K), 4 waves (2 x 2)
+//   macro tile 128 x 128 x 16, 4 waves           256 x 256 x (64 bytes of K) x 4-stage LDS ring, 4 waves
 //   wave tile 2 x 2 blocks of 32x32x16 (2 MFMA)  4 x 4 blocks of 32x32, one wide-K MFMA per step
 //   global -> VGPR -> shuffle -> LDS             global -> LDS directly (global_load_lds_dwordx4)
 //   LDS -> VGPR -> shuffle (AOS<->SOA)           swizzled ds_read_b128, or ds_read_b64_tr_b16
 //                                                for operands whose K is not contiguous
-//   8 MFMA between barriers                      64 MFMA (256 passes) between barriers
+//   2 LDS buffers, wait + barrier per step       copies 3 stages ahead, one bare barrier per stage
+//   8 MFMA between barriers                      32 MFMA (256 passes) between barriers
 //   grid (m/128, n/128)                          1-D grid, tiles dealt to XCDs in L2-friendly patches
 //
 // Column-major C/D is handled by the caller as the transposed problem (D^T = B^T A^T).
@@ -34,53 +35,66 @@ namespace rocwmma_amd
                   uint32_t WavesM_,
                   uint32_t WavesN_,
                   uint32_t BlocksM_,
-                  uint32_t BlocksN_>
+                  uint32_t BlocksN_,
+                  uint32_t Stages_       = 4u, // LDS ring depth
+                  uint32_t WavesPerSimd_ = 1u> // resident waves per SIMD the register budget must allow
         struct BlockedConfig
         {
             using InT   = InT_;
             using OutT  = OutT_;
             using CompT = CompT_;
 
-            static constexpr bool     AKMajor  = AKMajor_;
-            static constexpr bool     BKMajor  = BKMajor_;
-            static constexpr uint32_t WavesM   = WavesM_;
-            static constexpr uint32_t WavesN   = WavesN_;
-            static constexpr uint32_t BlocksM  = BlocksM_;
-            static constexpr uint32_t BlocksN  = BlocksN_;
-            static constexpr uint32_t Waves    = WavesM * WavesN;
-            static constexpr uint32_t Threads  = Waves * 64u;
-            static constexpr uint32_t Block    = 32u; // MFMA edge
-            static constexpr uint32_t WaveM    = BlocksM * Block;
-            static constexpr uint32_t WaveN    = BlocksN * Block;
-            static constexpr uint32_t MacroM   = WavesM * WaveM;
-            static constexpr uint32_t MacroN   = WavesN * WaveN;
-            static constexpr uint32_t TileKB   = 128u; // bytes of K per LDS tile
-            static constexpr uint32_t MacroK   = TileKB / sizeof(InT);
+            static constexpr bool     AKMajor = AKMajor_;
+            static constexpr bool     BKMajor = BKMajor_;
+            static constexpr uint32_t WavesM  = WavesM_;
+            static constexpr uint32_t WavesN  = WavesN_;
+            static constexpr uint32_t BlocksM = BlocksM_;
+            static constexpr uint32_t BlocksN = BlocksN_;
+            static constexpr uint32_t Waves   = WavesM * WavesN;
+            static constexpr uint32_t Threads = Waves * 64u;
+            static constexpr uint32_t Block   = 32u; // MFMA edge
+            static constexpr uint32_t WaveM   = BlocksM * Block;
+            static constexpr uint32_t WaveN   = BlocksN * Block;
+            static constexpr uint32_t MacroM  = WavesM * WaveM;
+            static constexpr uint32_t MacroN  = WavesN * WaveN;
+            static constexpr uint32_t StageKB = 64u; // bytes of K per pipeline stage
+            static constexpr uint32_t MacroK  = StageKB / sizeof(InT); // K elements per stage
 
             // Fragments of one MFMA step.  BlockK = K of the widest single instruction.
             static constexpr uint32_t KPack      = detail::maxKPack(detail::packClassOf<InT>());
             static constexpr uint32_t BlockK     = KPack * 2u; // 32-wide blocks: 2 lane groups along K
             static constexpr uint32_t KPackBytes = KPack * sizeof(InT);
-            static constexpr uint32_t KSteps     = MacroK / BlockK;
+            static constexpr uint32_t KSteps     = MacroK / BlockK; // MFMA steps per stage (1 or 2)
 
             using FragA   = fragment<matrix_a, Block, Block, BlockK, InT, row_major>;
             using FragB   = fragment<matrix_b, Block, Block, BlockK, InT, col_major>;
             using FragAcc = fragment<accumulator, Block, Block, BlockK, CompT>;
             using FragC   = fragment<accumulator, Block, Block, BlockK, OutT, row_major>;
 
-            using TileAK = lds::KMajorTile<MacroM>;
-            using TileBK = lds::KMajorTile<MacroN>;
-            using TileAD = lds::DimMajorTile<MacroM>;
-            using TileBD = lds::DimMajorTile<MacroN>;
+            using TileA = std::conditional_t<AKMajor, lds::KMajorTile<MacroM>, lds::DimMajorTile<MacroM>>;
+            using TileB = std::conditional_t<BKMajor, lds::KMajorTile<MacroN>, lds::DimMajorTile<MacroN>>;
 
-            static constexpr uint32_t BytesA   = MacroM * TileKB;
-            static constexpr uint32_t BytesB   = MacroN * TileKB;
-            static constexpr uint32_t StageB   = BytesA + BytesB;
-            static constexpr uint32_t Stages   = 2u;
-            static constexpr uint32_t LdsBytes = Stages * StageB;
+            static constexpr uint32_t BytesA     = MacroM * StageKB;
+            static constexpr uint32_t BytesB     = MacroN * StageKB;
+            static constexpr uint32_t StageBytes = BytesA + BytesB;
+            static constexpr uint32_t Stages     = Stages_; // ring of K stages in LDS
+            static constexpr uint32_t WavesPerSimd = WavesPerSimd_;
+            static constexpr uint32_t LdsBytes   = Stages * StageBytes;
+            static constexpr uint32_t CopiesA    = BytesA / 1024u / Waves; // direct copies per wave per stage
+            static constexpr uint32_t CopiesB    = BytesB / 1024u / Waves;
+            static constexpr uint32_t Copies     = CopiesA + CopiesB;
+            // LDS read instructions per MFMA step: b128 reads per block (K-major) or two transposing b64 reads
+            static constexpr uint32_t ReadsA       = BlocksM * (AKMajor ? KPackBytes / 16u : 2u);
+            static constexpr uint32_t ReadsB       = BlocksN * (BKMajor ? KPackBytes / 16u : 2u);
+            static constexpr uint32_t ReadsPerStep = ReadsA + ReadsB;
+            static constexpr uint32_t MfmasPerStep = BlocksM * BlocksN;
 
             static_assert(AKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
             static_assert(BKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
+            static_assert(TileA::bytes == BytesA && TileB::bytes == BytesB, "stage geometry mismatch");
+            static_assert(BytesA % (1024u * Waves) == 0u && BytesB % (1024u * Waves) == 0u,
+                          "a stage must split into whole-wave copies evenly");
+            static_assert((Stages - 1u) * Copies < 64u, "too many copies in flight for vmcnt");
             static_assert(LdsBytes <= Constants::AMDGCN_LDS_MAX_SIZE_BYTES, "macro tile does not fit the LDS");
         };
 
@@ -94,18 +108,58 @@ namespace rocwmma_amd
             if(total % kXcds == 0u)
                 id = (wg % kXcds) * (total / kXcds) + wg / kXcds;
             // panels of 8 tile rows, walked column by column
-            constexpr uint32_t panel      = 8u;
-            const uint32_t     perPanel   = panel * tilesN;
-            const uint32_t     panelIdx   = id / perPanel;
-            const uint32_t     firstRow   = panelIdx * panel;
-            const uint32_t     rowsHere   = (tilesM - firstRow) < panel ? (tilesM - firstRow) : panel;
-            const uint32_t     inPanel    = id - panelIdx * perPanel;
-            tm                            = firstRow + inPanel % rowsHere;
-            tn                            = inPanel / rowsHere;
+            constexpr uint32_t panel    = 8u;
+            const uint32_t     perPanel = panel * tilesN;
+            const uint32_t     panelIdx = id / perPanel;
+            const uint32_t     firstRow = panelIdx * panel;
+            const uint32_t     rowsHere = (tilesM - firstRow) < panel ? (tilesM - firstRow) : panel;
+            const uint32_t     inPanel  = id - panelIdx * perPanel;
+            tm                          = firstRow + inPanel % rowsHere;
+            tn                          = inPanel / rowsHere;
         }
 
+        // Scheduling hint: within the current scheduling region, issue `Mfmas` matrix instructions
+        // with `Reads` LDS reads and `Copies` global -> LDS copies spread evenly between them.
+        template <uint32_t Mfmas, uint32_t Reads, uint32_t Copies>
+        ROCWMMA_DEVICE ROCWMMA_INLINE void scheduleInterleaved()
+        {
+#pragma unroll
+            for(uint32_t j = 0; j < Mfmas; ++j)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
+                const uint32_t r = ((j + 1u) * Reads) / Mfmas - (j * Reads) / Mfmas;
+                const uint32_t c = ((j + 1u) * Copies) / Mfmas - (j * Copies) / Mfmas;
+                if(r == 1u)
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
+                else if(r == 2u)
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                else if(r > 2u)
+                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                if(c == 1u)
+                    __builtin_amdgcn_sched_group_barrier(0x010, 1, 0); // VMEM
+                else if(c >= 2u)
+                    __builtin_amdgcn_sched_group_barrier(0x010, 2, 0);
+            }
+        }
+
+        // Main loop schedule (per wave; S = 4 LDS stages of 64 bytes of K, F0/F1 = fragment
+        // register sets of the first / last MFMA step of a stage):
+        //
+        //   prologue : copies for stages 0..2 in flight; wait for stage 0; barrier; read F0(0)
+        //   iteration i:
+        //       issue copies of stage i+3 (into the ring slot everybody finished reading at
+        //         the barrier of iteration i-1)
+        //       [two-step stages] read F1(i) while the MFMAs of F0(i) run
+        //       wait: stage i+1 landed (copies of stages i+2, i+3 may stay in flight) and own
+        //         LDS reads returned;  barrier
+        //       read F0(i+1) while the MFMAs of the last step of stage i run
+        //
+        // So every LDS read has a full MFMA step (16 instructions, 512 cycles) to return, every
+        // global -> LDS copy has almost three iterations, and the barrier is the only
+        // synchronisation per stage.
         template <typename Cfg>
-        __global__ void __launch_bounds__(Cfg::Threads) gemmBlockedKernel(uint32_t                   m,
+        __global__ void __launch_bounds__(Cfg::Threads) __attribute__((amdgpu_waves_per_eu(Cfg::WavesPerSimd, Cfg::WavesPerSimd)))
+        gemmBlockedKernel(uint32_t                   m,
                                                                            uint32_t                   n,
                                                                            uint32_t                   k,
                                                                            typename Cfg::InT const*   a,
@@ -122,59 +176,77 @@ namespace rocwmma_amd
             using InT   = typename Cfg::InT;
             using OutT  = typename Cfg::OutT;
             using CompT = typename Cfg::CompT;
+            using TileA = typename Cfg::TileA;
+            using TileB = typename Cfg::TileB;
 
             extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
 
-            const uint32_t lane   = threadIdx.x & 63u;
-            const uint32_t wave   = threadIdx.x >> 6;
-            const uint32_t waveM  = wave / Cfg::WavesN;
-            const uint32_t waveN  = wave % Cfg::WavesN;
+            const uint32_t lane  = threadIdx.x & 63u;
+            const uint32_t wave  = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave uniform
+            const uint32_t waveM = wave / Cfg::WavesN;
+            const uint32_t waveN = wave % Cfg::WavesN;
 
             uint32_t tm, tn;
             tileOfWorkgroup(blockIdx.x, m / Cfg::MacroM, n / Cfg::MacroN, tm, tn);
             const uint32_t row0 = tm * Cfg::MacroM;
             const uint32_t col0 = tn * Cfg::MacroN;
 
-            // Global sources of the first K tile (byte pointers)
-            const char* aSrc;
-            const char* bSrc;
-            uint32_t    aStep, bStep; // bytes to the next K tile
+            // Global sources: uniform tile pointer + uniform per-copy offset + per-lane offset
             const uint32_t ldaB = lda * sizeof(InT);
             const uint32_t ldbB = ldb * sizeof(InT);
-            if constexpr(Cfg::AKMajor)
-            {
-                aSrc  = reinterpret_cast<const char*>(a) + static_cast<size_t>(row0) * ldaB;
-                aStep = Cfg::TileKB;
-            }
-            else
-            {
-                aSrc  = reinterpret_cast<const char*>(a) + static_cast<size_t>(row0) * sizeof(InT);
-                aStep = Cfg::MacroK * ldaB;
-            }
-            if constexpr(Cfg::BKMajor)
-            {
-                bSrc  = reinterpret_cast<const char*>(b) + static_cast<size_t>(col0) * ldbB;
-                bStep = Cfg::TileKB;
-            }
-            else
-            {
-                bSrc  = reinterpret_cast<const char*>(b) + static_cast<size_t>(col0) * sizeof(InT);
-                bStep = Cfg::MacroK * ldbB;
-            }
+            const char*    aSrc = reinterpret_cast<const char*>(a)
+                               + static_cast<size_t>(row0) * (Cfg::AKMajor ? ldaB : static_cast<uint32_t>(sizeof(InT)));
+            const char* bSrc = reinterpret_cast<const char*>(b)
+                               + static_cast<size_t>(col0) * (Cfg::BKMajor ? ldbB : static_cast<uint32_t>(sizeof(InT)));
+            const size_t   aStep    = TileA::stageStep(ldaB);
+            const size_t   bStep    = TileB::stageStep(ldbB);
+            const uint32_t aLaneOff = TileA::laneSourceOffset(lane, wave, ldaB);
+            const uint32_t bLaneOff = TileB::laneSourceOffset(lane, wave, ldbB);
 
-            auto issueTile = [&](uint32_t stage) {
-                char* ldsA = ldsRaw + stage * Cfg::StageB;
-                char* ldsB = ldsA + Cfg::BytesA;
-                if constexpr(Cfg::AKMajor)
-                    Cfg::TileAK::template asyncLoad<Cfg::Waves>(ldsA, aSrc, ldaB, wave, lane);
-                else
-                    Cfg::TileAD::template asyncLoad<Cfg::Waves>(ldsA, aSrc, ldaB, wave, lane);
-                if constexpr(Cfg::BKMajor)
-                    Cfg::TileBK::template asyncLoad<Cfg::Waves>(ldsB, bSrc, ldbB, wave, lane);
-                else
-                    Cfg::TileBD::template asyncLoad<Cfg::Waves>(ldsB, bSrc, ldbB, wave, lane);
+            // A stage is copied in two halves (the A operand, then the B operand) so that each
+            // MFMA phase of an iteration carries half of the copy instructions.
+            auto issueA = [&](uint32_t slot) {
+                char*                 ldsA = ldsRaw + slot * Cfg::StageBytes;
+                const lds::BufferRsrc src  = lds::makeSource(aSrc);
+#pragma unroll
+                for(uint32_t i = 0; i < Cfg::CopiesA; ++i)
+                {
+                    const uint32_t copy = i * Cfg::Waves + wave;
+                    lds::asyncCopy16(ldsA + copy * 1024u, src, aLaneOff, TileA::copySourceOffset(copy, ldaB));
+                }
                 aSrc += aStep;
+            };
+            auto issueB = [&](uint32_t slot) {
+                char*                 ldsB = ldsRaw + slot * Cfg::StageBytes + Cfg::BytesA;
+                const lds::BufferRsrc src  = lds::makeSource(bSrc);
+#pragma unroll
+                for(uint32_t i = 0; i < Cfg::CopiesB; ++i)
+                {
+                    const uint32_t copy = i * Cfg::Waves + wave;
+                    lds::asyncCopy16(ldsB + copy * 1024u, src, bLaneOff, TileB::copySourceOffset(copy, ldbB));
+                }
                 bSrc += bStep;
+            };
+            auto issueStage = [&](uint32_t slot) {
+                issueA(slot);
+                issueB(slot);
+            };
+
+            struct Frags
+            {
+                typename Cfg::FragA a[Cfg::BlocksM];
+                typename Cfg::FragB b[Cfg::BlocksN];
+            };
+
+            auto readFrags = [&](Frags& f, uint32_t slot, uint32_t ks) {
+                const char* ldsA = ldsRaw + slot * Cfg::StageBytes;
+                const char* ldsB = ldsA + Cfg::BytesA;
+#pragma unroll
+                for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
+                    TileA::template readBlock32<Cfg::KPackBytes>(f.a[i].x, ldsA, waveM * Cfg::WaveM + i * Cfg::Block, ks, lane);
+#pragma unroll
+                for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
+                    TileB::template readBlock32<Cfg::KPackBytes>(f.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, ks, lane);
             };
 
             typename Cfg::FragAcc acc[Cfg::BlocksM][Cfg::BlocksN];
@@ -184,80 +256,126 @@ namespace rocwmma_amd
                 for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
                     fill_fragment(acc[i][j], static_cast<CompT>(0));
 
-            auto computeTile = [&](uint32_t stage) {
-                const char* ldsA = ldsRaw + stage * Cfg::StageB;
-                const char* ldsB = ldsA + Cfg::BytesA;
+            auto multiply = [&](Frags const& f) {
 #pragma unroll
-                for(uint32_t ks = 0; ks < Cfg::KSteps; ++ks)
-                {
-                    typename Cfg::FragA fa[Cfg::BlocksM];
-                    typename Cfg::FragB fb[Cfg::BlocksN];
-#pragma unroll
-                    for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
-                    {
-                        const uint32_t r = waveM * Cfg::WaveM + i * Cfg::Block;
-                        if constexpr(Cfg::AKMajor)
-                            Cfg::TileAK::template readBlock32<Cfg::KPackBytes>(fa[i].x, ldsA, r, ks, lane);
-                        else
-                            Cfg::TileAD::readBlock32(fa[i].x, ldsA, r, ks, lane);
-                    }
+                for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
 #pragma unroll
                     for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
-                    {
-                        const uint32_t cc = waveN * Cfg::WaveN + j * Cfg::Block;
-                        if constexpr(Cfg::BKMajor)
-                            Cfg::TileBK::template readBlock32<Cfg::KPackBytes>(fb[j].x, ldsB, cc, ks, lane);
-                        else
-                            Cfg::TileBD::readBlock32(fb[j].x, ldsB, cc, ks, lane);
-                    }
-#pragma unroll
-                    for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
-#pragma unroll
-                        for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
-                            mma_sync(acc[i][j], fa[i], fb[j], acc[i][j]);
-                }
+                        mma_sync(acc[i][j], f.a[i], f.b[j], acc[i][j]);
             };
 
-            // Prologue: first K tile into stage 0
-            const uint32_t kTiles = k / Cfg::MacroK;
-            issueTile(0);
-            lds::asyncCopyWait();
-            synchronize_workgroup();
+            constexpr uint32_t S      = Cfg::Stages;
+            const uint32_t     stages = k / Cfg::MacroK; // >= S - 1 (checked by the host)
 
-            for(uint32_t kt = 0; kt + 1 < kTiles; ++kt)
+            // Prologue
+#pragma unroll
+            for(uint32_t s = 0; s < S - 1u; ++s)
+                issueStage(s);
+            lds::waitCopiesAndReads<(S - 2u) * Cfg::Copies>();
+            lds::barrier();
+            Frags f0, f1;
+            readFrags(f0, 0u, 0u);
+
+            // Steady state: a new stage is issued every iteration
+            uint32_t i = 0;
+            for(; i + (S - 1u) < stages; ++i)
             {
-                const uint32_t stage = kt & 1u;
-                issueTile(stage ^ 1u); // next tile streams into the other buffer ...
-                computeTile(stage); // ... while this one is multiplied
-                lds::asyncCopyWait();
-                synchronize_workgroup();
+                if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
+                {
+                    lds::waitReads(); // fragments read during the previous phase
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr(Cfg::KSteps == 2u)
+                {
+                    issueA((i + S - 1u) % S);
+                    readFrags(f1, i % S, 1u);
+                    multiply(f0);
+                    // LDS reads ride on the first half of the MFMAs (so they are back at the
+                    // barrier), the copies on the second half, two MFMAs per copy
+                    scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
+                    scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::CopiesA>();
+                    __builtin_amdgcn_sched_barrier(0); // nothing moves across the synchronisation point
+                    // stage i+1 has landed once only stage i+2 and the A half of stage i+3 are in flight
+                    lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies + Cfg::CopiesA>();
+                    lds::barrier();
+                    __builtin_amdgcn_sched_barrier(0);
+                    issueB((i + S - 1u) % S);
+                    readFrags(f0, (i + 1u) % S, 0u);
+                    multiply(f1);
+                    scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
+                    scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::CopiesB>();
+                }
+                else
+                {
+                    issueStage((i + S - 1u) % S);
+                    __builtin_amdgcn_sched_barrier(0);
+                    lds::waitCopiesAndReads<(S - 2u) * Cfg::Copies>();
+                    lds::barrier();
+                    __builtin_amdgcn_sched_barrier(0);
+                    readFrags(f1, (i + 1u) % S, 0u);
+                    multiply(f0);
+                    scheduleInterleaved<Cfg::MfmasPerStep, Cfg::ReadsPerStep, 0u>();
+                    f0 = f1;
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            computeTile((kTiles - 1u) & 1u);
+            // Drain: nothing left to issue; the remaining stages are already in flight
+            for(; i < stages; ++i)
+            {
+                const bool more = i + 1u < stages;
+                if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
+                {
+                    lds::waitReads();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr(Cfg::KSteps == 2u)
+                {
+                    readFrags(f1, i % S, 1u);
+                    multiply(f0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                lds::waitCopiesAndReads<0u>();
+                lds::barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr(Cfg::KSteps == 2u)
+                {
+                    if(more)
+                        readFrags(f0, (i + 1u) % S, 0u);
+                    multiply(f1);
+                }
+                else
+                {
+                    if(more)
+                        readFrags(f1, (i + 1u) % S, 0u);
+                    multiply(f0);
+                    f0 = f1;
+                }
+            }
 
             // Epilogue: D = alpha * acc + beta * C, block by block (16-byte accesses per lane)
             const uint32_t wRow = row0 + waveM * Cfg::WaveM;
             const uint32_t wCol = col0 + waveN * Cfg::WaveN;
 #pragma unroll
-            for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
+            for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
             {
 #pragma unroll
-                for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
+                for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
                 {
-                    const size_t rr = wRow + i * Cfg::Block;
-                    const size_t cc = wCol + j * Cfg::Block;
+                    const size_t rr = wRow + bi * Cfg::Block;
+                    const size_t cc = wCol + bj * Cfg::Block;
                     typename Cfg::FragC fc;
                     if(beta != static_cast<CompT>(0))
                     {
                         load_matrix_sync(fc, c + rr * ldc + cc, ldc);
 #pragma unroll
                         for(uint32_t e = 0; e < fc.num_elements; ++e)
-                            fc.x[e] = static_cast<OutT>(alpha * acc[i][j].x[e] + beta * static_cast<CompT>(fc.x[e]));
+                            fc.x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e] + beta * static_cast<CompT>(fc.x[e]));
                     }
                     else
                     {
 #pragma unroll
                         for(uint32_t e = 0; e < fc.num_elements; ++e)
-                            fc.x[e] = static_cast<OutT>(alpha * acc[i][j].x[e]);
+                            fc.x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e]);
                     }
                     store_matrix_sync(d + rr * ldd + cc, fc, ldd);
                 }
@@ -267,8 +385,18 @@ namespace rocwmma_amd
         template <typename Cfg>
         int launchCfg(GemmArgs const& g, hipStream_t stream)
         {
-            if(g.m % Cfg::MacroM != 0u || g.n % Cfg::MacroN != 0u || g.k % Cfg::MacroK != 0u || g.k < Cfg::MacroK)
+            if(g.m % Cfg::MacroM != 0u || g.n % Cfg::MacroN != 0u || g.k % Cfg::MacroK != 0u
+               || g.k < (Cfg::Stages - 1u) * Cfg::MacroK)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            // a stage's copies address their source inside a 2 GiB window from the stage origin
+            {
+                const uint64_t spanA = static_cast<uint64_t>(g.lda) * sizeof(typename Cfg::InT)
+                                       * (Cfg::AKMajor ? Cfg::MacroM : Cfg::MacroK);
+                const uint64_t spanB = static_cast<uint64_t>(g.ldb) * sizeof(typename Cfg::InT)
+                                       * (Cfg::BKMajor ? Cfg::MacroN : Cfg::MacroK);
+                if(spanA >= 0x7FFF0000ull || spanB >= 0x7FFF0000ull)
+                    return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            }
             auto kernel = gemmBlockedKernel<Cfg>;
             // more than 64 KiB of dynamic LDS needs an explicit opt-in (idempotent, no allocation)
             if(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
