@@ -2,6 +2,7 @@
 #ifndef ROCWMMA_AMD_CSRC_COMMON_HPP
 #define ROCWMMA_AMD_CSRC_COMMON_HPP
 
+#include <atomic>
 #include <cstdint>
 #include <hip/hip_runtime.h>
 
@@ -40,6 +41,24 @@ namespace rocwmma_amd
         default:
             return 0;
         }
+    }
+
+    // Compute units of the current device (immutable per device, so remembered per ordinal).
+    inline uint32_t computeUnits()
+    {
+        constexpr int             kMaxDevices = 64;
+        static std::atomic<int>   known[kMaxDevices];
+        int                       dev = 0;
+        if(hipGetDevice(&dev) != hipSuccess)
+            return 256u;
+        if(dev >= 0 && dev < kMaxDevices && known[dev].load(std::memory_order_relaxed) > 0)
+            return static_cast<uint32_t>(known[dev].load(std::memory_order_relaxed));
+        int cus = 0;
+        if(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            return 256u;
+        if(dev >= 0 && dev < kMaxDevices)
+            known[dev].store(cus, std::memory_order_relaxed);
+        return static_cast<uint32_t>(cus);
     }
 
     inline int launchStatus()

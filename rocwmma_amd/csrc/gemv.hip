@@ -7,9 +7,14 @@
 // past its buffers; its CPU twin sgemv_cpu_h (samples/simple_sgemv.cpp:46-66) defines the
 // semantics kept here.
 //
-// Work split: one wave owns RowsPerWave consecutive rows and walks K in steps of 512 elements
-// (64 lanes x 8 halves = 1 KiB contiguous per row per step); the four waves of a workgroup
-// walk K together on neighbouring rows so the X chunk they share stays in the CU's L1.
+// Two kernels, picked by the number of right-hand sides:
+//   * split kernel (1 column): a workgroup of four waves owns two rows and splits K four ways;
+//     every wave keeps four 1 KiB row segments in flight, partial sums meet in LDS.  Many
+//     short waves keep all HBM channels busy.
+//   * staged kernel (2..8 columns): X (ncols x K halves, at most 128 KiB) is copied into LDS
+//     once per workgroup; persistent waves then stream rows of A, one row per wave at a time,
+//     reading X from LDS so the extra columns cost no L1/L2 traffic.
+//   If X does not fit the LDS the split kernel reads X through the caches instead.
 #include "common.hpp"
 
 namespace rocwmma_amd
@@ -41,31 +46,38 @@ namespace rocwmma_amd
             return v;
         }
 
-        template <uint32_t NCols, uint32_t RowsPerWave>
-        __global__ void __launch_bounds__(256) gemvKernel(uint32_t        m,
-                                                          uint32_t        k,
-                                                          const _Float16* a,
-                                                          uint32_t        lda,
-                                                          const _Float16* x,
-                                                          uint32_t        ldx,
-                                                          float*          y,
-                                                          uint32_t        ldy,
-                                                          float           alpha,
-                                                          float           beta)
+        // Split kernel: workgroup = 4 waves = (4 / KSplit) row groups x KSplit slices of K.
+        template <uint32_t NCols, uint32_t RowsPerWave, uint32_t KSplit>
+        __global__ void __launch_bounds__(256) gemvSplitKernel(uint32_t        m,
+                                                               uint32_t        k,
+                                                               const _Float16* a,
+                                                               uint32_t        lda,
+                                                               const _Float16* x,
+                                                               uint32_t        ldx,
+                                                               float*          y,
+                                                               uint32_t        ldy,
+                                                               float           alpha,
+                                                               float           beta)
         {
-            const uint32_t lane = threadIdx.x & 63u;
-            const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-            const uint32_t row0 = wave * RowsPerWave;
-            if(row0 >= m)
-                return;
+            __shared__ float partial[4][RowsPerWave * NCols];
+            const uint32_t   lane     = threadIdx.x & 63u;
+            const uint32_t   wave     = threadIdx.x >> 6;
+            const uint32_t   rowGroup = (blockIdx.x * 4u + wave) / KSplit;
+            const uint32_t   slice    = wave % KSplit;
+            const uint32_t   row0     = rowGroup * RowsPerWave;
+            // K slices in whole 16-byte chunks; the last slice takes the remainder
+            const uint32_t chunks   = k / 8u;
+            const uint32_t perSlice = (chunks + KSplit - 1u) / KSplit;
+            const uint32_t cBeg     = slice * perSlice;
+            const uint32_t cEnd     = (cBeg + perSlice < chunks) ? cBeg + perSlice : chunks;
 
             // rows past the end are clamped for loads and dropped at the store
-            const _Float16* aRow[RowsPerWave];
+            const u32x4_t* aRow[RowsPerWave];
 #pragma unroll
             for(uint32_t r = 0; r < RowsPerWave; ++r)
             {
                 const uint32_t row = (row0 + r < m) ? row0 + r : m - 1u;
-                aRow[r]            = a + static_cast<size_t>(row) * lda;
+                aRow[r]            = reinterpret_cast<const u32x4_t*>(a + static_cast<size_t>(row) * lda);
             }
 
             float acc[RowsPerWave][NCols];
@@ -75,17 +87,17 @@ namespace rocwmma_amd
                 for(uint32_t c = 0; c < NCols; ++c)
                     acc[r][c] = 0.0f;
 
-#pragma unroll 2
-            for(uint32_t k0 = lane * 8u; k0 < k; k0 += 512u)
+#pragma unroll 4
+            for(uint32_t ch = cBeg + lane; ch < cEnd; ch += 64u)
             {
                 u32x4_t av[RowsPerWave];
                 u32x4_t xv[NCols];
 #pragma unroll
                 for(uint32_t r = 0; r < RowsPerWave; ++r)
-                    av[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(aRow[r] + k0));
+                    av[r] = __builtin_nontemporal_load(aRow[r] + ch);
 #pragma unroll
                 for(uint32_t c = 0; c < NCols; ++c)
-                    xv[c] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(c) * ldx + k0);
+                    xv[c] = reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(c) * ldx)[ch];
 #pragma unroll
                 for(uint32_t r = 0; r < RowsPerWave; ++r)
 #pragma unroll
@@ -99,6 +111,30 @@ namespace rocwmma_amd
                 for(uint32_t c = 0; c < NCols; ++c)
                     acc[r][c] = waveSum(acc[r][c]);
 
+            if constexpr(KSplit > 1u)
+            {
+                if(lane == 0u)
+                {
+#pragma unroll
+                    for(uint32_t r = 0; r < RowsPerWave; ++r)
+#pragma unroll
+                        for(uint32_t c = 0; c < NCols; ++c)
+                            partial[wave][r * NCols + c] = acc[r][c];
+                }
+                __syncthreads();
+                if(slice == 0u)
+                {
+#pragma unroll
+                    for(uint32_t r = 0; r < RowsPerWave; ++r)
+#pragma unroll
+                        for(uint32_t c = 0; c < NCols; ++c)
+#pragma unroll
+                            for(uint32_t j = 1; j < KSplit; ++j)
+                                acc[r][c] += partial[wave + j][r * NCols + c];
+                }
+            }
+            if(slice != 0u)
+                return;
             // lane (r * NCols + c) writes result (r, c)
 #pragma unroll
             for(uint32_t r = 0; r < RowsPerWave; ++r)
@@ -114,46 +150,123 @@ namespace rocwmma_amd
                 }
         }
 
-        template <uint32_t NCols>
-        int launch(uint32_t m, uint32_t k, const void* a, uint32_t lda, const void* x, uint32_t ldx, float* y,
-                   uint32_t ldy, float alpha, float beta, hipStream_t stream)
+        // Staged kernel: X in LDS, persistent waves, one row per wave at a time.
+        template <uint32_t NCols, uint32_t Waves>
+        __global__ void __launch_bounds__(Waves * 64u) gemvStagedKernel(uint32_t        m,
+                                                                        uint32_t        k,
+                                                                        const _Float16* a,
+                                                                        uint32_t        lda,
+                                                                        const _Float16* x,
+                                                                        uint32_t        ldx,
+                                                                        float*          y,
+                                                                        uint32_t        ldy,
+                                                                        float           alpha,
+                                                                        float           beta)
         {
-            constexpr uint32_t rowsPerWave = NCols >= 8 ? 4u : 4u;
-            constexpr uint32_t wavesPerWg  = 4u;
-            const uint32_t     waves       = (m + rowsPerWave - 1u) / rowsPerWave;
-            const uint32_t     grid        = (waves + wavesPerWg - 1u) / wavesPerWg;
-            hipLaunchKernelGGL((gemvKernel<NCols, rowsPerWave>),
-                               dim3(grid),
-                               dim3(64u * wavesPerWg),
-                               0,
-                               stream,
-                               m,
-                               k,
-                               static_cast<const _Float16*>(a),
-                               lda,
-                               static_cast<const _Float16*>(x),
-                               ldx,
-                               y,
-                               ldy,
-                               alpha,
-                               beta);
+            extern __shared__ __attribute__((aligned(16))) char ldsRaw[];
+            u32x4_t*       xs     = reinterpret_cast<u32x4_t*>(ldsRaw); // [NCols][k / 8] 16-byte chunks
+            const uint32_t chunks = k / 8u;
+#pragma unroll
+            for(uint32_t c = 0; c < NCols; ++c)
+                for(uint32_t i = threadIdx.x; i < chunks; i += Waves * 64u)
+                    xs[c * chunks + i] = reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(c) * ldx)[i];
+            __syncthreads();
+
+            const uint32_t lane   = threadIdx.x & 63u;
+            const uint32_t gwave  = blockIdx.x * Waves + (threadIdx.x >> 6);
+            const uint32_t nwaves = gridDim.x * Waves;
+            for(uint32_t row = gwave; row < m; row += nwaves)
+            {
+                const u32x4_t* aRow = reinterpret_cast<const u32x4_t*>(a + static_cast<size_t>(row) * lda);
+                float          acc[NCols];
+#pragma unroll
+                for(uint32_t c = 0; c < NCols; ++c)
+                    acc[c] = 0.0f;
+#pragma unroll 4
+                for(uint32_t ch = lane; ch < chunks; ch += 64u)
+                {
+                    const u32x4_t av = __builtin_nontemporal_load(aRow + ch);
+#pragma unroll
+                    for(uint32_t c = 0; c < NCols; ++c)
+                        acc[c] = dot8(av, xs[c * chunks + ch], acc[c]);
+                }
+#pragma unroll
+                for(uint32_t c = 0; c < NCols; ++c)
+                    acc[c] = waveSum(acc[c]);
+#pragma unroll
+                for(uint32_t c = 0; c < NCols; ++c)
+                {
+                    if(lane == c)
+                    {
+                        float*      dst = y + static_cast<size_t>(c) * ldy + row;
+                        const float v   = alpha * acc[c];
+                        *dst            = (beta != 0.0f) ? v + beta * *dst : v;
+                    }
+                }
+            }
+        }
+
+        struct GemvArgs
+        {
+            uint32_t    m, k;
+            const void* a;
+            uint32_t    lda;
+            const void* x;
+            uint32_t    ldx;
+            float*      y;
+            uint32_t    ldy;
+            float       alpha, beta;
+        };
+
+        template <uint32_t NCols, uint32_t RowsPerWave, uint32_t KSplit>
+        int launchSplit(GemvArgs const& g, hipStream_t stream)
+        {
+            const uint32_t groups = (g.m + RowsPerWave - 1u) / RowsPerWave;
+            const uint32_t waves  = groups * KSplit;
+            hipLaunchKernelGGL((gemvSplitKernel<NCols, RowsPerWave, KSplit>), dim3((waves + 3u) / 4u), dim3(256), 0, stream,
+                               g.m, g.k, static_cast<const _Float16*>(g.a), g.lda, static_cast<const _Float16*>(g.x), g.ldx,
+                               g.y, g.ldy, g.alpha, g.beta);
             return launchStatus();
         }
+
+        template <uint32_t NCols, uint32_t Waves>
+        int launchStaged(GemvArgs const& g, uint32_t workgroups, hipStream_t stream)
+        {
+            const uint32_t ldsBytes = NCols * g.k * 2u;
+            auto           kernel   = gemvStagedKernel<NCols, Waves>;
+            if(ldsBytes > 65536u
+               && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(ldsBytes))
+                      != hipSuccess)
+                return ROCWMMA_AMD_LAUNCH_FAILED;
+            const uint32_t needed = (g.m + Waves - 1u) / Waves;
+            hipLaunchKernelGGL(kernel, dim3(needed < workgroups ? needed : workgroups), dim3(Waves * 64u), ldsBytes, stream,
+                               g.m, g.k, static_cast<const _Float16*>(g.a), g.lda, static_cast<const _Float16*>(g.x), g.ldx,
+                               g.y, g.ldy, g.alpha, g.beta);
+            return launchStatus();
+        }
+
+        constexpr uint32_t kStagedLdsLimit = 131072u; // X must leave room in the 160 KiB LDS
     } // namespace
 
     int launchGemv(uint32_t m, uint32_t k, uint32_t ncols, const void* a, uint32_t lda, const void* x, uint32_t ldx,
                    float* y, uint32_t ldy, float alpha, float beta, hipStream_t stream)
     {
+        const GemvArgs g{m, k, a, lda, x, ldx, y, ldy, alpha, beta};
+        const uint32_t cus    = computeUnits();
+        const bool     staged = ncols * k * 2u <= kStagedLdsLimit;
         switch(ncols)
         {
         case 1:
-            return launch<1>(m, k, a, lda, x, ldx, y, ldy, alpha, beta, stream);
+            return launchSplit<1, 2, 4>(g, stream);
         case 2:
-            return launch<2>(m, k, a, lda, x, ldx, y, ldy, alpha, beta, stream);
+            return staged ? launchStaged<2, 8>(g, 2u * cus, stream) : launchSplit<2, 2, 4>(g, stream);
         case 4:
-            return launch<4>(m, k, a, lda, x, ldx, y, ldy, alpha, beta, stream);
+            // two 512-thread workgroups per CU while X is at most 64 KiB, else one
+            return staged ? launchStaged<4, 8>(g, (4u * k * 2u <= 65536u ? 2u : 1u) * cus, stream)
+                          : launchSplit<4, 4, 2>(g, stream);
         case 8:
-            return launch<8>(m, k, a, lda, x, ldx, y, ldy, alpha, beta, stream);
+            return staged ? launchStaged<8, 16>(g, cus, stream) : launchSplit<8, 4, 2>(g, stream);
         default:
             return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
         }

@@ -33,7 +33,9 @@ def test_config4_full_shapes(m, k, ncols, beta):
     run(m, k, ncols, 1.0, beta, 0x5EED0004 + ncols)
 
 
-@pytest.mark.parametrize("m,k,ncols", [(1, 8, 1), (3, 520, 2), (37, 1000, 4), (130, 72, 8), (255, 4104, 1)])
+@pytest.mark.parametrize("m,k,ncols", [(1, 8, 1), (3, 520, 2), (37, 1000, 4), (130, 72, 8), (255, 4104, 1),
+                                       (2, 16, 1), (5, 24, 1), (64, 16384, 8), (100, 32776, 4), (9, 65536, 2),
+                                       (1000, 8, 8), (4100, 264, 2)])
 def test_ragged_shapes(m, k, ncols):
     run(m, k, ncols, 2.1, 2.1, 99)
 
