@@ -36,6 +36,8 @@ def parse_args():
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the headline GEMM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain 1 GiB device copy (known traffic) for counter calibration")
     ap.add_argument("--only", default=None,
                     help="run one headline case only, e.g. f16_rc (dtype_{r|c}{r|c} = A,B layout): for profiling")
     return ap.parse_args()
@@ -75,6 +77,15 @@ def main():
     RM, CM = rw.ROW_MAJOR, rw.COL_MAJOR
     S = args.size
     gen = torch.Generator(device=dev).manual_seed(0x5EED0002)
+
+    if args.calibrate_copy:
+        # reads 1 GiB, writes 1 GiB: the reference point FETCH_SIZE / WRITE_SIZE are scaled by
+        src = torch.ones(1 << 28, device=dev, dtype=torch.float32)
+        dst = torch.empty_like(src)
+        ms = event_ms(lambda: dst.copy_(src), 5, torch)
+        print(json.dumps({"calibrate_copy_bytes_each_way": src.numel() * 4, "ms": round(ms, 4),
+                          "gbs": round(2 * src.numel() * 4 / ms / 1e6, 1)}))
+        return
 
     def rand(count, dtype):
         return (torch.rand(count, device=dev, generator=gen) * 2 - 1).to(dtype)
