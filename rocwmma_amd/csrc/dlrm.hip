@@ -9,8 +9,9 @@
 //   * one wave owns a whole sample: the m <= 32 feature rows are one 32-row MFMA operand, so
 //     Z = F F^T is K/16 v_mfma_f32_32x32x16_f16 with the SAME registers as both multiplicands
 //     (applyTranspose of the A fragment is the B fragment);
-//   * a workgroup of 4 waves owns 8 consecutive samples, whose outputs are contiguous in
-//     memory: results are assembled in LDS and leave as 16-byte coalesced stores;
+//   * a workgroup of 8 waves owns 8 consecutive samples, whose inputs and outputs are
+//     contiguous in memory: features arrive as whole-wave 1 KiB direct-to-LDS copies, results
+//     are assembled in LDS and leave as 16-byte coalesced stores;
 //   * backward rebuilds the symmetric matrix G in registers from the LDS-staged upstream
 //     gradient (no global m x m scratch, no second launch), reads F^T operands with the
 //     transposing LDS load, and writes grad through LDS the same way.
@@ -27,13 +28,12 @@ namespace rocwmma_amd
 {
     namespace
     {
-        constexpr uint32_t kSamplesPerWg   = 8;
-        constexpr uint32_t kWavesPerWg     = 4;
-        constexpr uint32_t kSamplesPerWave = kSamplesPerWg / kWavesPerWg;
-        constexpr uint32_t kMaxM           = 32;
+        constexpr uint32_t kSamplesPerWg = 8; // = waves per workgroup: one sample per wave
+        constexpr uint32_t kWavesPerWg   = 8;
+        constexpr uint32_t kMaxM         = 32;
 
         typedef uint32_t u32x4_t __attribute__((ext_vector_type(4), may_alias));
-        typedef uint16_t u16_alias __attribute__((may_alias));
+        typedef short    s16x4_t __attribute__((ext_vector_type(4)));
 
         ROCWMMA_DEVICE inline uint32_t trilIndex(uint32_t row, uint32_t col) // row > col
         {
@@ -60,45 +60,95 @@ namespace rocwmma_amd
                 ldsDst[i] = src[i];
         }
 
+        // The feature rows of a workgroup's samples are contiguous in global memory
+        // (samples x m rows of K halves).  They are copied into LDS as one matrix of
+        // RowBytes-wide rows with whole-wave 1 KiB direct copies; inside a row the 16-byte
+        // chunks (forward) or 32-byte segments (backward) are XOR-swizzled by the row index so
+        // that the MFMA operand reads are bank-conflict free.  The swizzle is applied to the
+        // source address of each lane's 16 bytes.
+        template <uint32_t K>
+        struct FeatureTile
+        {
+            static constexpr uint32_t rowBytes  = K * 2u;
+            static constexpr uint32_t chunks    = rowBytes / 16u;
+            static constexpr uint32_t segments  = rowBytes / 32u;
+            static constexpr uint32_t rowsPer256 = rowBytes >= 256u ? 1u : 256u / rowBytes;
+
+            // forward: 16 consecutive rows reading the same logical chunk hit 16 distinct banks groups
+            ROCWMMA_DEVICE static inline uint32_t chunkSwizzle(uint32_t row)
+            {
+                return (row / rowsPer256) & ((chunks < 16u ? chunks : 16u) - 1u);
+            }
+            // backward: the 4 rows x 2 segments of one transposing read hit 8 distinct bank groups
+            ROCWMMA_DEVICE static inline uint32_t segmentSwizzle(uint32_t row)
+            {
+                return ((row & 3u) << 1) & (segments - 1u);
+            }
+
+            // Issues this wave's share of the copies of `bytes` (multiple of 16) from `src` into
+            // `ldsTile`.  Lanes past `bytes` read nothing (buffer bounds) and store zeros.
+            template <bool BySegment>
+            ROCWMMA_DEVICE static inline void
+                asyncLoad(char* ldsTile, const void* src, uint32_t bytes, uint32_t wave, uint32_t waves, uint32_t lane)
+            {
+                const lds::BufferRsrc rsrc   = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(src), 0, static_cast<int>(bytes), 0x00020000);
+                const uint32_t        copies = (bytes + 1023u) / 1024u;
+                for(uint32_t copy = wave; copy < copies; copy += waves)
+                {
+                    const uint32_t o   = copy * 1024u + lane * 16u; // LDS byte offset of this lane's 16 bytes
+                    const uint32_t row = o / rowBytes;
+                    const uint32_t pos = (o % rowBytes) / 16u;
+                    uint32_t       srcOff;
+                    if constexpr(BySegment)
+                        srcOff = row * rowBytes + ((((pos >> 1) ^ segmentSwizzle(row)) << 5) | ((pos & 1u) << 4));
+                    else
+                        srcOff = row * rowBytes + ((pos ^ chunkSwizzle(row)) << 4);
+                    lds::asyncCopy16(ldsTile + copy * 1024u, rsrc, srcOff, 0u);
+                }
+            }
+        };
+
         // ------------------------------------------------------------------ forward
         template <uint32_t K>
         __global__ void __launch_bounds__(64 * kWavesPerWg)
             dlrmFwdKernel(const float16_t* __restrict__ input, float16_t* __restrict__ output, uint32_t m, uint32_t batch)
         {
             constexpr uint32_t KSteps = K / 16u;
+            using Tile                = FeatureTile<K>;
             using FragA               = fragment<matrix_a, 32, 32, 16, float16_t, row_major>;
             using FragAcc             = fragment<accumulator, 32, 32, 16, float32_t>;
             using AccMap              = detail::AccMap<32, 32, 32>;
 
-            extern __shared__ __attribute__((aligned(16))) char ldsRaw[];
-            float16_t* ldsOut = reinterpret_cast<float16_t*>(ldsRaw);
+            extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
+            const uint32_t width     = K + (m * (m - 1u)) / 2u;
+            const uint32_t tileBytes = (((kSamplesPerWg - 1u) * m + kMaxM) * Tile::rowBytes + 1023u) & ~1023u;
+            char*          ldsIn     = ldsRaw;
+            float16_t*     ldsOut    = reinterpret_cast<float16_t*>(ldsRaw + tileBytes);
 
-            const uint32_t width   = K + (m * (m - 1u)) / 2u;
             const uint32_t lane    = threadIdx.x & 63u;
-            const uint32_t wave    = threadIdx.x >> 6;
+            const uint32_t wave    = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
             const uint32_t sample0 = blockIdx.x * kSamplesPerWg;
             const uint32_t nHere   = min(kSamplesPerWg, batch - sample0);
-            const uint32_t row     = lane & 31u;
-            const uint32_t kGroup  = lane >> 5;
 
-#pragma unroll
-            for(uint32_t s = 0; s < kSamplesPerWave; ++s)
+            // all feature rows of the workgroup's samples: one contiguous block
+            Tile::template asyncLoad<false>(ldsIn, input + static_cast<size_t>(sample0) * m * K, nHere * m * Tile::rowBytes,
+                                            wave, kWavesPerWg, lane);
+            lds::waitCopiesAndReads<0>();
+            __syncthreads();
+
+            if(wave < nHere)
             {
-                const uint32_t local = wave * kSamplesPerWave + s;
-                if(local >= nHere)
-                    break;
-                const float16_t* F = input + static_cast<size_t>(sample0 + local) * m * K;
-
-                // operand registers: row `row`, k = ks*16 + kGroup*8 .. +7 ; rows >= m are zero
-                FragA fa[KSteps];
+                // operand: matrix row = lane % 32 (rows >= m belong to the next sample or are
+                // stale LDS: they only reach Gram entries with an index >= m, which are dropped)
+                const uint32_t row    = lane & 31u;
+                const uint32_t kGroup = lane >> 5;
+                const uint32_t R      = wave * m + row;
+                const uint32_t swz    = Tile::chunkSwizzle(R);
+                FragA          fa[KSteps];
 #pragma unroll
                 for(uint32_t ks = 0; ks < KSteps; ++ks)
-                {
-                    u32x4_t v = {0u, 0u, 0u, 0u};
-                    if(row < m)
-                        v = *reinterpret_cast<const u32x4_t*>(F + row * K + ks * 16u + kGroup * 8u);
-                    *reinterpret_cast<u32x4_t*>(fa[ks].x) = v;
-                }
+                    *reinterpret_cast<u32x4_t*>(fa[ks].x)
+                        = *reinterpret_cast<const u32x4_t*>(ldsIn + R * Tile::rowBytes + (((ks * 2u + kGroup) ^ swz) << 4));
 
                 FragAcc acc;
                 fill_fragment(acc, 0.0f);
@@ -106,7 +156,7 @@ namespace rocwmma_amd
                 for(uint32_t ks = 0; ks < KSteps; ++ks)
                     mma_sync(acc, fa[ks], applyTranspose(fa[ks]), acc);
 
-                float16_t* out = ldsOut + local * width;
+                float16_t* out = ldsOut + wave * width;
                 // bottom-MLP row: the lanes holding row 0 copy their operand registers
                 if(row == 0u)
                 {
@@ -140,58 +190,42 @@ namespace rocwmma_amd
                                                                            uint32_t batch)
         {
             constexpr uint32_t NBlocks = K / 32u; // 32-column blocks of the m x K result
+            using Tile                 = FeatureTile<K>;
             using FragG                = fragment<matrix_a, 32, 32, 16, float16_t, row_major>;
             using FragF                = fragment<matrix_b, 32, 32, 16, float16_t, row_major>;
             using FragAcc              = fragment<accumulator, 32, 32, 16, float32_t>;
             using AccMap               = detail::AccMap<32, 32, 32>;
-            using FTile                = lds::DimMajorTile<(K < 128u ? 128u : K)>; // [feature row][K] with swizzled segments
 
-            // LDS: per workgroup the contiguous upstream rows of its samples, then one
-            // 32 x K feature tile per sample (rows m..31 stay zero).
-            constexpr uint32_t tileBytes = kMaxM * FTile::rowBytes;
-            extern __shared__ __attribute__((aligned(16))) char ldsRaw[];
-
-            const uint32_t width    = K + (m * (m - 1u)) / 2u;
-            const uint32_t upBytes  = ((kSamplesPerWg * width * 2u + 15u) / 16u) * 16u;
-            float16_t*     ldsUp    = reinterpret_cast<float16_t*>(ldsRaw);
-            char*          ldsTiles = ldsRaw + upBytes;
+            extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
+            const uint32_t width     = K + (m * (m - 1u)) / 2u;
+            const uint32_t tileBytes = (((kSamplesPerWg - 1u) * m + kMaxM) * Tile::rowBytes + 1023u) & ~1023u;
+            char*          ldsF      = ldsRaw; // features in, gradients out
+            float16_t*     ldsUp     = reinterpret_cast<float16_t*>(ldsRaw + tileBytes);
 
             const uint32_t lane    = threadIdx.x & 63u;
-            const uint32_t wave    = threadIdx.x >> 6;
+            const uint32_t wave    = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
             const uint32_t sample0 = blockIdx.x * kSamplesPerWg;
             const uint32_t nHere   = min(kSamplesPerWg, batch - sample0);
 
-            // stage upstream gradients (contiguous for the workgroup's samples)
+            // Rows past the last sample are read as contraction rows >= m (multiplied by the zero
+            // columns of G): they must hold finite values, so clear everything behind the features
+            // first (the tail of the last partial copy is out of the buffer's bounds and reads zeros).
+            const uint32_t featBytes = nHere * m * Tile::rowBytes;
+            for(uint32_t i = featBytes / 16u + threadIdx.x; i < tileBytes / 16u; i += blockDim.x)
+                reinterpret_cast<u32x4_t*>(ldsF)[i] = u32x4_t{0u, 0u, 0u, 0u};
+            // features: direct copies, segment-swizzled for the transposing reads
+            Tile::template asyncLoad<true>(ldsF, input + static_cast<size_t>(sample0) * m * K, featBytes, wave, kWavesPerWg, lane);
+            // upstream gradients (contiguous for the workgroup's samples)
             copyIn(ldsUp, upstream + static_cast<size_t>(sample0) * width, nHere * width);
-
-            // stage features: 16-byte chunks, segment-swizzled rows; zero the padding rows
-            constexpr uint32_t chunksPerRow = K / 8u;
-            for(uint32_t s = 0; s < nHere; ++s)
-            {
-                const float16_t* F    = input + static_cast<size_t>(sample0 + s) * m * K;
-                char*            tile = ldsTiles + s * tileBytes;
-                for(uint32_t i = threadIdx.x; i < kMaxM * chunksPerRow; i += blockDim.x)
-                {
-                    const uint32_t r     = i / chunksPerRow;
-                    const uint32_t chunk = i % chunksPerRow;
-                    u32x4_t        v     = {0u, 0u, 0u, 0u};
-                    if(r < m)
-                        v = *reinterpret_cast<const u32x4_t*>(F + r * K + chunk * 8u);
-                    *reinterpret_cast<u32x4_t*>(tile + FTile::offset(r, chunk >> 1) + ((chunk & 1u) << 4)) = v;
-                }
-            }
+            lds::waitCopiesAndReads<0>();
             __syncthreads();
 
-            const uint32_t row    = lane & 31u;
-            const uint32_t kGroup = lane >> 5;
-#pragma unroll
-            for(uint32_t s = 0; s < kSamplesPerWave; ++s)
+            FragAcc acc[NBlocks];
+            if(wave < nHere)
             {
-                const uint32_t local = wave * kSamplesPerWave + s;
-                if(local >= nHere)
-                    break;
-                const float16_t* up   = ldsUp + local * width;
-                char*            tile = ldsTiles + local * tileBytes;
+                const uint32_t   row    = lane & 31u;
+                const uint32_t   kGroup = lane >> 5;
+                const float16_t* up     = ldsUp + wave * width;
 
                 // G operand: row `row`, columns ks*16 + kGroup*8 + j, rebuilt from the packed triangle
                 FragG fg[2];
@@ -209,25 +243,45 @@ namespace rocwmma_amd
                         fg[ks].x[j] = g;
                     }
 
-                FragAcc acc[NBlocks];
+                // F operands: transposing reads, lane l gets column nb*32 + l%32 and contraction
+                // rows ks*16 + (l/32)*8 + 0..7 of this sample
+                const uint32_t group   = lane >> 4;
+                const uint32_t s16     = lane & 15u;
+                const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds::LdsPtr)ldsF));
+                FragF          ff[NBlocks][2];
+#pragma unroll
+                for(uint32_t nb = 0; nb < NBlocks; ++nb)
+#pragma unroll
+                    for(uint32_t ks = 0; ks < 2u; ++ks)
+#pragma unroll
+                        for(uint32_t kk = 0; kk < 2u; ++kk)
+                        {
+                            const uint32_t c    = ks * 16u + (group >> 1) * 8u + kk * 4u + (s16 >> 2);
+                            const uint32_t R    = wave * m + c;
+                            const uint32_t seg  = nb * 2u + (group & 1u);
+                            const uint32_t addr = ldsBase + R * Tile::rowBytes + ((seg ^ Tile::segmentSwizzle(R)) << 5)
+                                                  + ((s16 & 3u) << 3);
+                            s16x4_t v;
+                            asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+                            reinterpret_cast<s16x4_t*>(ff[nb][ks].x)[kk] = v;
+                        }
+                lds::waitReads();
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for(uint32_t nb = 0; nb < NBlocks; ++nb)
                 {
                     fill_fragment(acc[nb], 0.0f);
 #pragma unroll
                     for(uint32_t ks = 0; ks < 2u; ++ks)
-                    {
-                        FragF ff;
-                        FTile::readBlock32(ff.x, tile, nb * 32u, ks, lane);
-                        lds::waitReads();
-                        __builtin_amdgcn_sched_barrier(0);
-                        mma_sync(acc[nb], fg[ks], ff, acc[nb]);
-                    }
+                        mma_sync(acc[nb], fg[ks], ff[nb][ks], acc[nb]);
                 }
+            }
+            __syncthreads(); // every wave is done reading features (its own and its neighbour's rows)
 
-                // all of this wave's reads of the tile are done (same wave, in order): reuse it,
-                // un-swizzled, as the staging buffer of grad[sample] (m x K, row-major)
-                float16_t* stage = reinterpret_cast<float16_t*>(tile);
+            if(wave < nHere)
+            {
+                // this sample's feature rows become the staging buffer of its gradient (m x K, row-major)
+                float16_t* stage = reinterpret_cast<float16_t*>(ldsF) + wave * m * K;
 #pragma unroll
                 for(uint32_t nb = 0; nb < NBlocks; ++nb)
 #pragma unroll
@@ -247,34 +301,49 @@ namespace rocwmma_amd
             }
             __syncthreads();
 
-            // coalesced write-out: grad (m*K halves per sample) and the bottom-MLP gradient
-            for(uint32_t s = 0; s < nHere; ++s)
+            // coalesced write-out: gradients of all samples are one contiguous block
+            copyOut(grad + static_cast<size_t>(sample0) * m * K, reinterpret_cast<const float16_t*>(ldsF), nHere * m * K);
+            for(uint32_t i = threadIdx.x; i < nHere * (K / 8u); i += blockDim.x)
             {
-                copyOut(grad + static_cast<size_t>(sample0 + s) * m * K,
-                        reinterpret_cast<const float16_t*>(ldsTiles + s * tileBytes),
-                        m * K);
-                const float16_t* up  = ldsUp + s * width;
-                float16_t*       dst = mlpGrad + static_cast<size_t>(sample0 + s) * K;
-                for(uint32_t i = threadIdx.x; i < K; i += blockDim.x)
-                    dst[i] = up[i];
+                const uint32_t   s   = i / (K / 8u);
+                const uint32_t   c8  = i % (K / 8u);
+                const float16_t* src = ldsUp + s * width + c8 * 8u; // only 2-byte aligned in general
+                float16_t        tmp[8];
+#pragma unroll
+                for(uint32_t j = 0; j < 8u; ++j)
+                    tmp[j] = src[j];
+                reinterpret_cast<u32x4_t*>(mlpGrad + static_cast<size_t>(sample0 + s) * K)[c8] = *reinterpret_cast<u32x4_t*>(tmp);
             }
+        }
+
+        template <uint32_t K>
+        uint32_t tileBytesFor(uint32_t m)
+        {
+            return (((kSamplesPerWg - 1u) * m + kMaxM) * K * 2u + 1023u) & ~1023u;
+        }
+
+        template <typename Kernel>
+        int optInLds(Kernel kernel, uint32_t lds)
+        {
+            if(lds > 65536u
+               && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(lds))
+                      != hipSuccess)
+                return ROCWMMA_AMD_LAUNCH_FAILED;
+            return ROCWMMA_AMD_OK;
         }
 
         template <uint32_t K>
         int launchFwd(const void* input, void* output, uint32_t m, uint32_t batch, hipStream_t stream)
         {
-            const uint32_t width = K + (m * (m - 1u)) / 2u;
-            const uint32_t lds   = kSamplesPerWg * width * 2u;
-            const uint32_t grid  = (batch + kSamplesPerWg - 1u) / kSamplesPerWg;
-            hipLaunchKernelGGL((dlrmFwdKernel<K>),
-                               dim3(grid),
-                               dim3(64u * kWavesPerWg),
-                               lds,
-                               stream,
-                               static_cast<const float16_t*>(input),
-                               static_cast<float16_t*>(output),
-                               m,
-                               batch);
+            const uint32_t width  = K + (m * (m - 1u)) / 2u;
+            const uint32_t lds    = tileBytesFor<K>(m) + ((kSamplesPerWg * width * 2u + 15u) & ~15u);
+            const uint32_t grid   = (batch + kSamplesPerWg - 1u) / kSamplesPerWg;
+            auto           kernel = dlrmFwdKernel<K>;
+            if(int rc = optInLds(kernel, lds))
+                return rc;
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(64u * kWavesPerWg), lds, stream, static_cast<const float16_t*>(input),
+                               static_cast<float16_t*>(output), m, batch);
             return launchStatus();
         }
 
@@ -282,29 +351,15 @@ namespace rocwmma_amd
         int launchBwd(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t batch,
                       hipStream_t stream)
         {
-            using FTile           = lds::DimMajorTile<(K < 128u ? 128u : K)>;
             const uint32_t width  = K + (m * (m - 1u)) / 2u;
-            const uint32_t upB    = ((kSamplesPerWg * width * 2u + 15u) / 16u) * 16u;
-            const uint32_t lds    = upB + kSamplesPerWg * kMaxM * FTile::rowBytes;
+            const uint32_t lds    = tileBytesFor<K>(m) + ((kSamplesPerWg * width * 2u + 15u) & ~15u);
             const uint32_t grid   = (batch + kSamplesPerWg - 1u) / kSamplesPerWg;
             auto           kernel = dlrmBwdKernel<K>;
-            if(lds > 65536u
-               && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      static_cast<int>(lds))
-                      != hipSuccess)
-                return ROCWMMA_AMD_LAUNCH_FAILED;
-            hipLaunchKernelGGL(kernel,
-                               dim3(grid),
-                               dim3(64u * kWavesPerWg),
-                               lds,
-                               stream,
-                               static_cast<const float16_t*>(input),
-                               static_cast<const float16_t*>(upstream),
-                               static_cast<float16_t*>(grad),
-                               static_cast<float16_t*>(mlpGrad),
-                               m,
-                               batch);
+            if(int rc = optInLds(kernel, lds))
+                return rc;
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(64u * kWavesPerWg), lds, stream, static_cast<const float16_t*>(input),
+                               static_cast<const float16_t*>(upstream), static_cast<float16_t*>(grad),
+                               static_cast<float16_t*>(mlpGrad), m, batch);
             return launchStatus();
         }
     } // namespace
