@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "librocwmma_amd.so")
 
-SOURCES = ["api.hip", "gemm_wave_tile.hip", "gemm_blocked.hip", "gemv.hip", "dlrm.hip", "selftest.hip"]
+SOURCES = ["api.hip", "gemm_wave_tile.hip", "gemm_blocked.hip", "gemm_skinny.hip", "gemv.hip", "dlrm.hip", "selftest.hip"]
 
 # -packed-fp32-ops off: packed FP32 instructions are not generated for this target build.
 HIPCC_FLAGS = [

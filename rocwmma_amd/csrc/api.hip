@@ -175,6 +175,13 @@ int rocwmma_amd_gemm_ex(int         algo,
         return ROCWMMA_AMD_NO_DEVICE;
 
     GemmArgs args{m, n, k, a, b, c, d, lda, ldb, c ? ldc : ldd, ldd, alpha, beta, layout_c};
+    if(algo == ROCWMMA_AMD_GEMM_AUTO && m <= 32u)
+    {
+        // few token rows against a wide 8-bit weight matrix: the weight-streaming kernel
+        rc = launchGemmSkinny(dtype_in, dtype_out, layout_a, layout_b, args, asStream(stream));
+        if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE && rc != ROCWMMA_AMD_UNSUPPORTED_TYPE)
+            return rc;
+    }
     if(algo != ROCWMMA_AMD_GEMM_WAVE_TILE)
     {
         // The blocked kernel writes row-major C/D; a column-major result is the row-major

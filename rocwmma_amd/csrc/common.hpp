@@ -84,6 +84,7 @@ namespace rocwmma_amd
     // ROCWMMA_AMD_UNSUPPORTED_SHAPE / _TYPE mean "this family has no kernel for it".
     int launchGemmWaveTile(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
     int launchGemmBlocked(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
+    int launchGemmSkinny(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
 
 } // namespace rocwmma_amd
 

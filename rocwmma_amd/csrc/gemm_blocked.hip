@@ -205,7 +205,9 @@ namespace rocwmma_amd
 
             // A stage is copied in two halves (the A operand, then the B operand) so that each
             // MFMA phase of an iteration carries half of the copy instructions.
-            auto issueA = [&](uint32_t slot) {
+            // advance == false leaves the source on the stage just copied (used to re-copy the last
+            // stage instead of running past the end of the operand)
+            auto issueA = [&](uint32_t slot, bool advance = true) {
                 char*                 ldsA = ldsRaw + slot * Cfg::StageBytes;
                 const lds::BufferRsrc src  = lds::makeSource(aSrc);
 #pragma unroll
@@ -214,9 +216,9 @@ namespace rocwmma_amd
                     const uint32_t copy = i * Cfg::Waves + wave;
                     lds::asyncCopy16(ldsA + copy * 1024u, src, aLaneOff, TileA::copySourceOffset(copy, ldaB));
                 }
-                aSrc += aStep;
+                aSrc += advance ? aStep : size_t{0};
             };
-            auto issueB = [&](uint32_t slot) {
+            auto issueB = [&](uint32_t slot, bool advance = true) {
                 char*                 ldsB = ldsRaw + slot * Cfg::StageBytes + Cfg::BytesA;
                 const lds::BufferRsrc src  = lds::makeSource(bSrc);
 #pragma unroll
@@ -225,11 +227,11 @@ namespace rocwmma_amd
                     const uint32_t copy = i * Cfg::Waves + wave;
                     lds::asyncCopy16(ldsB + copy * 1024u, src, bLaneOff, TileB::copySourceOffset(copy, ldbB));
                 }
-                bSrc += bStep;
+                bSrc += advance ? bStep : size_t{0};
             };
-            auto issueStage = [&](uint32_t slot) {
-                issueA(slot);
-                issueB(slot);
+            auto issueStage = [&](uint32_t slot, bool advance = true) {
+                issueA(slot, advance);
+                issueB(slot, advance);
             };
 
             struct Frags
@@ -267,26 +269,26 @@ namespace rocwmma_amd
             constexpr uint32_t S      = Cfg::Stages;
             const uint32_t     stages = k / Cfg::MacroK; // >= S - 1 (checked by the host)
 
-            // Prologue
-#pragma unroll
-            for(uint32_t s = 0; s < S - 1u; ++s)
-                issueStage(s);
-            lds::waitCopiesAndReads<(S - 2u) * Cfg::Copies>();
-            lds::barrier();
-            Frags f0, f1;
-            readFrags(f0, 0u, 0u);
-
-            // Steady state: a new stage is issued every iteration
-            uint32_t i = 0;
-            for(; i + (S - 1u) < stages; ++i)
+            if constexpr(Cfg::KSteps == 2u)
             {
-                if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
+                // Prologue
+#pragma unroll
+                for(uint32_t s = 0; s < S - 1u; ++s)
+                    issueStage(s);
+                lds::waitCopiesAndReads<(S - 2u) * Cfg::Copies>();
+                lds::barrier();
+                Frags f0, f1;
+                readFrags(f0, 0u, 0u);
+
+                // Steady state: a new stage is issued every iteration
+                uint32_t i = 0;
+                for(; i + (S - 1u) < stages; ++i)
                 {
-                    lds::waitReads(); // fragments read during the previous phase
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                if constexpr(Cfg::KSteps == 2u)
-                {
+                    if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
+                    {
+                        lds::waitReads(); // fragments read during the previous phase
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                     issueA((i + S - 1u) % S);
                     readFrags(f1, i % S, 1u);
                     multiply(f0);
@@ -304,52 +306,69 @@ namespace rocwmma_amd
                     multiply(f1);
                     scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                     scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::CopiesB>();
-                }
-                else
-                {
-                    issueStage((i + S - 1u) % S);
-                    __builtin_amdgcn_sched_barrier(0);
-                    lds::waitCopiesAndReads<(S - 2u) * Cfg::Copies>();
-                    lds::barrier();
-                    __builtin_amdgcn_sched_barrier(0);
-                    readFrags(f1, (i + 1u) % S, 0u);
-                    multiply(f0);
-                    scheduleInterleaved<Cfg::MfmasPerStep, Cfg::ReadsPerStep, 0u>();
-                    f0 = f1;
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // Drain: nothing left to issue; the remaining stages are already in flight
-            for(; i < stages; ++i)
-            {
-                const bool more = i + 1u < stages;
-                if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
-                {
-                    lds::waitReads();
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if constexpr(Cfg::KSteps == 2u)
+                // Drain: nothing left to issue; the remaining stages are already in flight
+                for(; i < stages; ++i)
                 {
+                    const bool more = i + 1u < stages;
+                    if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
+                    {
+                        lds::waitReads();
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                     readFrags(f1, i % S, 1u);
                     multiply(f0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                lds::waitCopiesAndReads<0u>();
-                lds::barrier();
-                __builtin_amdgcn_sched_barrier(0);
-                if constexpr(Cfg::KSteps == 2u)
-                {
+                    __builtin_amdgcn_sched_barrier(0);
+                    lds::waitCopiesAndReads<0u>();
+                    lds::barrier();
+                    __builtin_amdgcn_sched_barrier(0);
                     if(more)
                         readFrags(f0, (i + 1u) % S, 0u);
                     multiply(f1);
                 }
-                else
+            }
+            else
+            {
+                // One MFMA step per stage (wide fp8): a phase multiplies stage s (fragments read
+                // during the previous phase) while it reads the fragments of stage s+1 and issues
+                // the copies of stage s+3; the wait + barrier closing the phase makes stage s+2
+                // visible.  Two phases per loop trip so the fragment sets swap without copies.
+                // Every phase issues a stage, so the loop body and its wait counts are uniform:
+                // past the end of K the last stage is copied again into a ring slot nobody reads.
+                static_assert(Cfg::KSteps == 1u && Cfg::AKMajor && Cfg::BKMajor, "one-step stages are K-major only");
+                Frags f0, f1;
+#define ROCWMMA_AMD_PHASE(STAGE, CUR, NXT, READ)                                                         \
+    do                                                                                                  \
+    {                                                                                                   \
+        issueStage(((STAGE) + S - 1u) % S, (STAGE) + S < stages);                                       \
+        if(READ)                                                                                        \
+            readFrags(NXT, ((STAGE) + 1u) % S, 0u);                                                     \
+        multiply(CUR);                                                                                  \
+        scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();                           \
+        scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::Copies>();             \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+        lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies>();                                              \
+        lds::barrier();                                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+    } while(0)
+
+#pragma unroll
+                for(uint32_t s = 0; s < S - 1u; ++s)
+                    issueStage(s, s + 1u < stages);
+                lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies>(); // stages 0 and 1 have landed
+                lds::barrier();
+                readFrags(f0, 0u, 0u);
+                uint32_t s = 0;
+                for(; s + 1u < stages; s += 2u)
                 {
-                    if(more)
-                        readFrags(f1, (i + 1u) % S, 0u);
-                    multiply(f0);
-                    f0 = f1;
+                    ROCWMMA_AMD_PHASE(s, f0, f1, true);
+                    ROCWMMA_AMD_PHASE(s + 1u, f1, f0, s + 2u < stages);
                 }
+                if(s < stages)
+                    multiply(f0);
+                lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
+#undef ROCWMMA_AMD_PHASE
             }
 
             // Epilogue: D = alpha * acc + beta * C, block by block (16-byte accesses per lane)
@@ -426,17 +445,30 @@ namespace rocwmma_amd
             return launchStatus();
         }
 
-        // Tile ladder: the 256 x 256 macro tile when the problem fills it, else 128 x 128.
+        // Tile ladder: the 256 x 256 macro tile when the problem fills it, else 128 x 128; when even
+        // that leaves compute units without a tile (few token rows against a wide weight matrix),
+        // 128 x 64 tiles double the number of workgroups.
         template <typename InT, typename OutT, typename CompT, bool AK, bool BK>
         int pickTile(GemmArgs const& g, hipStream_t stream)
         {
-            using Big   = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 4, 4>;
-            using Small = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2>;
+            using Big    = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 4, 4>;
+            using Small  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2>;
             if(g.m % Big::MacroM == 0u && g.n % Big::MacroN == 0u)
             {
                 int rc = launchCfg<Big>(g, stream);
                 if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
                     return rc;
+            }
+            if constexpr(AK && BK)
+            {
+                using Narrow = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1>;
+                if(g.m % Small::MacroM == 0u && g.n % Small::MacroN == 0u
+                   && (g.m / Small::MacroM) * (g.n / Small::MacroN) < computeUnits())
+                {
+                    int rc = launchCfg<Narrow>(g, stream);
+                    if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                        return rc;
+                }
             }
             return launchCfg<Small>(g, stream);
         }

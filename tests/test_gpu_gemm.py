@@ -159,6 +159,27 @@ def test_leading_dimensions_larger_than_extent():
         assert np.all(got[:, n:] == 777.0)
 
 
+@pytest.mark.parametrize("m", [16, 32, 48, 80, 112, 128])
+@pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3, orc.E5M2])
+def test_skinny_weight_streaming_kernel(dtype_in, m):
+    """M <= 128 token rows, 8-bit, A row / B col: served by the K-split weight-streaming kernel
+    (AUTO).  int8 must be bit-exact; the wave-tile kernel gives the same answer."""
+    n, k = 352, 1536
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(71, orc.I8, m * k), uniform_bits(72, orc.I8, k * n)
+        c = uniform_bits(73, orc.I32, m * n)
+    else:
+        a, b = normal_fp8_bits(71, dtype_in, m * k), normal_fp8_bits(72, dtype_in, k * n)
+        c = np.random.default_rng(73).uniform(-1, 1, m * n).astype(np.float32)
+    out = OUT_OF[dtype_in]
+    for alpha, beta in [(1.0, 0.0), (2.0, -3.0)]:
+        got = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, c, alpha, beta, rw.GEMM_AUTO)
+        want = orc.gemm(dtype_in, out, RM, CM, RM, RM, m, n, k, a, b, c, alpha, beta)
+        check(dtype_in, out, got, want, tol_for(dtype_in))
+        ref = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, c, alpha, beta, rw.GEMM_WAVE_TILE)
+        check(dtype_in, out, ref, want, tol_for(dtype_in))
+
+
 # ---------------------------------------------------------------- config 3: quantised shapes
 @pytest.mark.parametrize("m", [16, 128, 4096])
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3])
