@@ -38,6 +38,13 @@ namespace rocwmma
             __builtin_amdgcn_global_load_lds((GlobalPtr)src, (LdsPtr)ldsBase, 16, 0, 0);
         }
 
+        // The same copy marked non-temporal: for data that is read once (it should not displace
+        // operand panels other workgroups are about to re-read from the caches).
+        ROCWMMA_DEVICE ROCWMMA_INLINE void asyncCopy16Streaming(void* ldsBase, const void* src)
+        {
+            __builtin_amdgcn_global_load_lds((GlobalPtr)src, (LdsPtr)ldsBase, 16, 0, 2 /* nt */);
+        }
+
         // The same copy with buffer addressing: source address = resource base + waveOffset
         // (scalar) + laneOffset (one VGPR).  Nothing but scalar arithmetic is needed per copy,
         // which keeps the vector ALU and the VGPR file out of the copy path.

@@ -6,13 +6,17 @@
 // re-plumbed for CDNA4:
 //
 //   reference (gfx9 params)                      this kernel
-//   macro tile 128 x 128 x 16, 4 waves           256 x 256 x (64 bytes of K) x 4-stage LDS ring, 4 waves
-//   wave tile 2 x 2 blocks of 32x32x16 (2 MFMA)  4 x 4 blocks of 32x32, one wide-K MFMA per step
+//   macro tile 128 x 128 x 16, 4 waves           256 x 256 x (64 bytes of K) x 4-stage LDS ring, 8 waves
+//                                                (two per SIMD: one keeps the matrix pipe fed
+//                                                while the other waits at a barrier)
+//   wave tile 2 x 2 blocks of 32x32x16 (2 MFMA)  2 x 4 blocks of 32x32, one wide-K MFMA per step
 //   global -> VGPR -> shuffle -> LDS             global -> LDS directly (global_load_lds_dwordx4)
 //   LDS -> VGPR -> shuffle (AOS<->SOA)           swizzled ds_read_b128, or ds_read_b64_tr_b16
 //                                                for operands whose K is not contiguous
 //   2 LDS buffers, wait + barrier per step       copies 3 stages ahead, one bare barrier per stage
-//   8 MFMA between barriers                      32 MFMA (256 passes) between barriers
+//   8 MFMA between barriers                      16 MFMA (128 passes) per wave between barriers
+//   C read / D written in fragment layout       C staged through LDS (full-row non-temporal
+//                                                copies), D written with non-temporal stores
 //   grid (m/128, n/128)                          1-D grid, tiles dealt to XCDs in L2-friendly patches
 //
 // Column-major C/D is handled by the caller as the transposed problem (D^T = B^T A^T).
@@ -88,6 +92,13 @@ namespace rocwmma_amd
             static constexpr uint32_t ReadsB       = BlocksN * (BKMajor ? KPackBytes / 16u : 2u);
             static constexpr uint32_t ReadsPerStep = ReadsA + ReadsB;
             static constexpr uint32_t MfmasPerStep = BlocksM * BlocksN;
+            // beta * C operand staged through LDS in the epilogue, in groups of 32 rows by
+            // GroupBlocks blocks (256- or 512-byte rows), two group buffers per wave
+            static constexpr uint32_t GroupBlocks
+                = (BlocksN == 4u && 2u * 32u * 128u * sizeof(OutT) * Waves <= LdsBytes) ? 4u : 2u;
+            static constexpr bool StagedC = sizeof(OutT) == 4u && BlocksN % 2u == 0u
+                                            && BlocksM * (BlocksN / GroupBlocks) >= 2u
+                                            && 2u * 32u * GroupBlocks * Block * sizeof(OutT) * Waves <= LdsBytes;
 
             static_assert(AKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
             static_assert(BKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
@@ -368,35 +379,169 @@ namespace rocwmma_amd
                 if(s < stages)
                     multiply(f0);
                 lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
+                lds::barrier();
 #undef ROCWMMA_AMD_PHASE
             }
 
-            // Epilogue: D = alpha * acc + beta * C, block by block (16-byte accesses per lane)
-            const uint32_t wRow = row0 + waveM * Cfg::WaveM;
-            const uint32_t wCol = col0 + waveN * Cfg::WaveN;
+            // Epilogue: D = alpha * acc + beta * C, one row of blocks (BlocksN blocks) at a time,
+            // 16-byte accesses per lane.  Every block of a group has registers of its own, so
+            // the stores of a group issue back to back (a store whose data registers are about
+            // to be overwritten holds up the instruction stream until it has read them), and
+            // the C blocks of the next two groups are in flight while a group is finished.
+            const uint32_t wRow        = row0 + waveM * Cfg::WaveM;
+            const uint32_t wCol        = col0 + waveN * Cfg::WaveN;
+            // D is written once and not read again by this kernel: non-temporal stores
+            auto storeBlock = [&](OutT* dst, typename Cfg::FragC const& f, uint32_t ld) {
+                typedef uint32_t Words __attribute__((ext_vector_type(sizeof(OutT))));
 #pragma unroll
-            for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+                for(uint32_t r = 0; r < 4u; ++r)
+                {
+                    Words v;
+                    __builtin_memcpy(&v, f.x + 4u * r, sizeof(v));
+                    __builtin_nontemporal_store(
+                        v, reinterpret_cast<Words*>(dst + static_cast<size_t>(lane & 31u) * ld + 8u * r + 4u * (lane >> 5)));
+                }
+            };
+            auto           blockOffset = [&](uint32_t bi, uint32_t bj, uint32_t ld) {
+                return static_cast<size_t>(wRow + bi * Cfg::Block) * ld + wCol + bj * Cfg::Block;
+            };
+            if(beta != static_cast<CompT>(0))
+            {
+                if constexpr(Cfg::StagedC)
+                {
+                    // C reaches the accumulator layout through LDS: whole-wave direct copies
+                    // fetch full rows of a 32-row group of GroupBlocks blocks (read in the
+                    // accumulator layout straight from global memory, an instruction would touch
+                    // 32 rows for 32 bytes each, at half the rate).  Row r is stored with its
+                    // 16-byte chunks XOR-swizzled by r % 16 so that the 16 rows a quarter-wave
+                    // reads at one chunk position fall into distinct bank groups.  The main-loop
+                    // ring is free by now and every wave owns two group buffers in it.
+                    constexpr uint32_t GB          = Cfg::GroupBlocks;
+                    constexpr uint32_t RowBytes    = GB * Cfg::Block * sizeof(OutT); // 256 or 512
+                    constexpr uint32_t GroupBytes  = 32u * RowBytes;
+                    constexpr uint32_t RowChunks   = RowBytes / 16u;
+                    constexpr uint32_t RowsPerCopy = 1024u / RowBytes;
+                    constexpr uint32_t CopiesC     = GroupBytes / 1024u;
+                    constexpr uint32_t StoresD     = GB * 4u; // 16-byte stores per group
+                    constexpr uint32_t GroupsPerRow = Cfg::BlocksN / GB;
+                    constexpr uint32_t NG          = Cfg::BlocksM * GroupsPerRow;
+                    static_assert((RowBytes == 256u || RowBytes == 512u) && 2u * GroupBytes * Cfg::Waves <= Cfg::LdsBytes
+                                      && NG >= 2u,
+                                  "C staging geometry");
+                    char*          myLds  = ldsRaw + wave * (2u * GroupBytes);
+                    const char*    cWave  = reinterpret_cast<const char*>(c + static_cast<size_t>(wRow) * ldc + wCol);
+                    const size_t   ldcB   = static_cast<size_t>(ldc) * sizeof(OutT);
+                    const uint32_t half   = lane >> 5;
+                    const uint32_t cpRow  = lane / RowChunks; // row inside a copy
+                    const uint32_t chunk  = lane % RowChunks; // chunk position inside the LDS row
+                    auto           copyGroup = [&](uint32_t gi) {
+                        const uint32_t bi = gi / GroupsPerRow, bj0 = (gi % GroupsPerRow) * GB;
+#pragma unroll
+                        for(uint32_t i = 0; i < CopiesC; ++i)
+                        {
+                            const uint32_t r = RowsPerCopy * i + cpRow;
+                            lds::asyncCopy16Streaming(myLds + (gi % 2u) * GroupBytes + i * 1024u,
+                                                      cWave + (bi * 32u + r) * ldcB + bj0 * Cfg::Block * sizeof(OutT)
+                                                          + ((chunk ^ (r & 15u)) << 4));
+                        }
+                    };
+                    const uint32_t rdRow  = lane & 31u;
+                    const uint32_t rdBase = rdRow * RowBytes;
+                    copyGroup(0u);
+                    copyGroup(1u);
+#pragma unroll
+                    for(uint32_t gi = 0; gi < NG; ++gi)
+                    {
+                        const uint32_t bi = gi / GroupsPerRow, bj0 = (gi % GroupsPerRow) * GB;
+                        // vector-memory operations younger than this group's copies: the next
+                        // group's copies and the stores of the two previous groups
+                        if(gi == 0u)
+                            lds::waitCopiesAndReads<CopiesC>();
+                        else if(gi == 1u)
+                            lds::waitCopiesAndReads<(NG > 2u ? CopiesC : 0u) + StoresD>();
+                        else if(gi + 1u < NG)
+                            lds::waitCopiesAndReads<CopiesC + 2u * StoresD>();
+                        else
+                            lds::waitCopiesAndReads<2u * StoresD>();
+                        asm volatile("" ::: "memory");
+                        typename Cfg::FragC io[GB];
+#pragma unroll
+                        for(uint32_t bj = 0; bj < GB; ++bj)
+#pragma unroll
+                            for(uint32_t r = 0; r < 4u; ++r)
+                            {
+                                const uint32_t g = bj * 8u + 2u * r + half; // logical chunk of this run
+                                detail::copyBytes<16u>(io[bj].x + 4u * r,
+                                                       myLds + (gi % 2u) * GroupBytes + rdBase + ((g ^ (rdRow & 15u)) << 4));
+                            }
+                        if(gi + 2u < NG)
+                        {
+                            lds::waitReads(); // the buffer is overwritten next
+                            asm volatile("" ::: "memory");
+                            copyGroup(gi + 2u);
+                        }
+#pragma unroll
+                        for(uint32_t bj = 0; bj < GB; ++bj)
+                        {
+#pragma unroll
+                            for(uint32_t e = 0; e < io[bj].num_elements; ++e)
+                                io[bj].x[e] = static_cast<OutT>(alpha * acc[bi][bj0 + bj].x[e]
+                                                                + beta * static_cast<CompT>(io[bj].x[e]));
+                        }
+#pragma unroll
+                        for(uint32_t bj = 0; bj < GB; ++bj)
+                            storeBlock(d + blockOffset(bi, bj0 + bj, ldd), io[bj], ldd);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                else
+                {
+                typename Cfg::FragC fc[2][Cfg::BlocksN];
+                auto                loadGroup = [&](uint32_t bi) {
+#pragma unroll
+                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                        load_matrix_sync(fc[bi % 2u][bj], c + blockOffset(bi, bj, ldc), ldc);
+                };
+                loadGroup(0u);
+                if constexpr(Cfg::BlocksM > 1u)
+                    loadGroup(1u);
+#pragma unroll
+                for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+                {
+#pragma unroll
+                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                    {
+                        auto& io = fc[bi % 2u][bj];
+#pragma unroll
+                        for(uint32_t e = 0; e < io.num_elements; ++e)
+                            io.x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e] + beta * static_cast<CompT>(io.x[e]));
+                    }
+#pragma unroll
+                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                        storeBlock(d + blockOffset(bi, bj, ldd), fc[bi % 2u][bj], ldd);
+                    if(bi + 2u < Cfg::BlocksM)
+                        loadGroup(bi + 2u);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                }
+            }
+            else
             {
 #pragma unroll
-                for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
                 {
-                    const size_t rr = wRow + bi * Cfg::Block;
-                    const size_t cc = wCol + bj * Cfg::Block;
-                    typename Cfg::FragC fc;
-                    if(beta != static_cast<CompT>(0))
-                    {
-                        load_matrix_sync(fc, c + rr * ldc + cc, ldc);
+                    typename Cfg::FragC fd[Cfg::BlocksN];
 #pragma unroll
-                        for(uint32_t e = 0; e < fc.num_elements; ++e)
-                            fc.x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e] + beta * static_cast<CompT>(fc.x[e]));
-                    }
-                    else
+                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
                     {
 #pragma unroll
-                        for(uint32_t e = 0; e < fc.num_elements; ++e)
-                            fc.x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e]);
+                        for(uint32_t e = 0; e < fd[bj].num_elements; ++e)
+                            fd[bj].x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e]);
                     }
-                    store_matrix_sync(d + rr * ldd + cc, fc, ldd);
+#pragma unroll
+                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                        storeBlock(d + blockOffset(bi, bj, ldd), fd[bj], ldd);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
@@ -451,7 +596,7 @@ namespace rocwmma_amd
         template <typename InT, typename OutT, typename CompT, bool AK, bool BK>
         int pickTile(GemmArgs const& g, hipStream_t stream)
         {
-            using Big    = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 4, 4>;
+            using Big    = BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 2, 4, 4, 2>;
             using Small  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2>;
             if(g.m % Big::MacroM == 0u && g.n % Big::MacroN == 0u)
             {
