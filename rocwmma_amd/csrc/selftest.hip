@@ -76,17 +76,48 @@ namespace rocwmma_amd
             return launchStatus();
         }
 
+        // Block sizes follow the reference's unit-test matrix (test/unit/unit_test_params.hpp:89-141):
+        // BlockM/N 16..256 against BlockK 8..256, thinned for the largest blocks to bound the
+        // number of kernels.
+        constexpr bool roundtripShape(uint32_t block, uint32_t blockk)
+        {
+            if(block == 16u)
+                return blockk == 16u || blockk == 32u || blockk == 64u || blockk == 128u || blockk == 256u;
+            if(block == 32u || block == 64u)
+                return blockk == 8u || blockk == 16u || blockk == 32u || blockk == 64u || blockk == 128u;
+            if(block == 128u || block == 256u)
+                return blockk == 8u || blockk == 32u;
+            return false;
+        }
+
+        template <typename MatrixT, typename T, typename Layout, uint32_t B, uint32_t K>
+        int launchShape(int coop, uint32_t rows, uint32_t cols, const void* in, void* out, uint32_t ld, hipStream_t s)
+        {
+            // accumulator blocks above 64 x 64 would not fit a wave's registers
+            constexpr bool tooBig = std::is_same<MatrixT, accumulator>::value && B > 64u;
+            if constexpr(roundtripShape(B, K) && !tooBig)
+                return launchRoundtrip<fragment<MatrixT, B, B, K, T, Layout>>(coop, rows, cols, in, out, ld, s);
+            else
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+        }
+
         template <typename MatrixT, typename T, typename Layout, uint32_t B>
         int pickBlockK(int blockk, int coop, uint32_t rows, uint32_t cols, const void* in, void* out, uint32_t ld, hipStream_t s)
         {
             switch(blockk)
             {
+            case 8:
+                return launchShape<MatrixT, T, Layout, B, 8>(coop, rows, cols, in, out, ld, s);
             case 16:
-                return launchRoundtrip<fragment<MatrixT, B, B, 16, T, Layout>>(coop, rows, cols, in, out, ld, s);
+                return launchShape<MatrixT, T, Layout, B, 16>(coop, rows, cols, in, out, ld, s);
+            case 32:
+                return launchShape<MatrixT, T, Layout, B, 32>(coop, rows, cols, in, out, ld, s);
             case 64:
-                return launchRoundtrip<fragment<MatrixT, B, B, 64, T, Layout>>(coop, rows, cols, in, out, ld, s);
+                return launchShape<MatrixT, T, Layout, B, 64>(coop, rows, cols, in, out, ld, s);
             case 128:
-                return launchRoundtrip<fragment<MatrixT, B, B, 128, T, Layout>>(coop, rows, cols, in, out, ld, s);
+                return launchShape<MatrixT, T, Layout, B, 128>(coop, rows, cols, in, out, ld, s);
+            case 256:
+                return launchShape<MatrixT, T, Layout, B, 256>(coop, rows, cols, in, out, ld, s);
             default:
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             }
@@ -103,6 +134,10 @@ namespace rocwmma_amd
                 return pickBlockK<MatrixT, T, Layout, 32>(blockk, coop, rows, cols, in, out, ld, s);
             case 64:
                 return pickBlockK<MatrixT, T, Layout, 64>(blockk, coop, rows, cols, in, out, ld, s);
+            case 128:
+                return pickBlockK<MatrixT, T, Layout, 128>(blockk, coop, rows, cols, in, out, ld, s);
+            case 256:
+                return pickBlockK<MatrixT, T, Layout, 256>(blockk, coop, rows, cols, in, out, ld, s);
             default:
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             }

@@ -31,15 +31,22 @@ def _shape(context, block, blockk):
     (rw.F16, 16, 16), (rw.F16, 32, 16), (rw.F16, 16, 64), (rw.F16, 32, 64), (rw.F16, 64, 16),
     (rw.I8, 16, 64), (rw.I8, 32, 64), (rw.I8, 32, 128), (rw.I8, 16, 16),
     (rw.F32, 16, 16), (rw.F32, 32, 16), (rw.F32, 64, 64),
+    # the rest of the reference's unit-test matrix (test/unit/unit_test_params.hpp:89-141):
+    # BlockK 8 .. 256 and blocks up to 256
+    (rw.F16, 32, 8), (rw.F16, 64, 32), (rw.F16, 16, 256), (rw.F16, 128, 8), (rw.F16, 128, 32), (rw.F16, 256, 8),
+    (rw.F16, 256, 32), (rw.I8, 64, 8), (rw.I8, 16, 256), (rw.I8, 128, 32), (rw.I8, 256, 8),
+    (rw.F32, 32, 8), (rw.F32, 16, 128), (rw.F32, 128, 8), (rw.F32, 256, 32),
 ])
 def test_load_store_identity_and_no_contamination(dtype, block, blockk, context, layout, coop):
     import torch
 
+    if context == 2 and block > 64:
+        pytest.skip("an accumulator block above 64 x 64 does not fit a wave's registers")
     h, w = _shape(context, block, blockk)
     tiles_r, tiles_c = 3, 2
     rows, cols = tiles_r * h, tiles_c * w
     pad = 16  # elements of padding in the leading dimension: must stay untouched
-    ld = (cols if layout == RM else rows) + pad
+    ld = -(-(cols if layout == RM else rows) // 16) * 16 + pad  # multiple of 16 elements (alignment rule of the ABI)
     outer = rows if layout == RM else cols
     np_t = NP[dtype]
     if dtype == rw.F32:
