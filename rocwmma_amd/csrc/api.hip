@@ -65,6 +65,8 @@ namespace rocwmma_amd
                                  || dtypeIn == ROCWMMA_AMD_E5M2;
             const bool okTypes = (floatIn && dtypeOut == ROCWMMA_AMD_F32)
                                  || (dtypeIn == ROCWMMA_AMD_F16 && dtypeOut == ROCWMMA_AMD_F16)
+                                 || (dtypeIn == ROCWMMA_AMD_BF16 && dtypeOut == ROCWMMA_AMD_BF16)
+                                 || (dtypeIn == ROCWMMA_AMD_F32 && dtypeOut == ROCWMMA_AMD_F32)
                                  || (dtypeIn == ROCWMMA_AMD_I8 && dtypeOut == ROCWMMA_AMD_I32);
             if(!okTypes)
                 return ROCWMMA_AMD_UNSUPPORTED_TYPE;

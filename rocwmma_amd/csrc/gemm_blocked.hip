@@ -652,6 +652,8 @@ namespace rocwmma_amd
             return pickLayout16<bfloat16_t, float32_t, float32_t>(layoutA, layoutB, g, stream);
         if(dtypeIn == ROCWMMA_AMD_F16 && dtypeOut == ROCWMMA_AMD_F16)
             return pickLayout16<float16_t, float16_t, float32_t>(layoutA, layoutB, g, stream);
+        if(dtypeIn == ROCWMMA_AMD_BF16 && dtypeOut == ROCWMMA_AMD_BF16)
+            return pickLayout16<bfloat16_t, bfloat16_t, float32_t>(layoutA, layoutB, g, stream);
         if(dtypeIn == ROCWMMA_AMD_I8 && dtypeOut == ROCWMMA_AMD_I32)
             return pickLayout8<int8_t, int32_t, int32_t>(layoutA, layoutB, g, stream);
         if(dtypeIn == ROCWMMA_AMD_E4M3 && dtypeOut == ROCWMMA_AMD_F32)

@@ -161,6 +161,10 @@ namespace rocwmma_amd
             return pickLayout<float16_t, float16_t, float32_t, 32, 16>(layoutA, layoutB, g, stream);
         if(dtypeIn == ROCWMMA_AMD_BF16 && dtypeOut == ROCWMMA_AMD_F32)
             return pickLayout<bfloat16_t, float32_t, float32_t, 32, 16>(layoutA, layoutB, g, stream);
+        if(dtypeIn == ROCWMMA_AMD_BF16 && dtypeOut == ROCWMMA_AMD_BF16)
+            return pickLayout<bfloat16_t, bfloat16_t, float32_t, 32, 16>(layoutA, layoutB, g, stream);
+        if(dtypeIn == ROCWMMA_AMD_F32 && dtypeOut == ROCWMMA_AMD_F32)
+            return pickLayout<float32_t, float32_t, float32_t, 4, 2>(layoutA, layoutB, g, stream);
         if(dtypeIn == ROCWMMA_AMD_E4M3 && dtypeOut == ROCWMMA_AMD_F32)
             return pickLayout<float8_t, float32_t, float32_t, 128, 64>(layoutA, layoutB, g, stream);
         if(dtypeIn == ROCWMMA_AMD_E5M2 && dtypeOut == ROCWMMA_AMD_F32)

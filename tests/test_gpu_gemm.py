@@ -42,6 +42,28 @@ def check(dtype_in, dtype_out, got, want, tol):
     return err
 
 
+# ------------------------------------------------ type combinations of the reference's GEMM tests
+@pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED])
+@pytest.mark.parametrize("la,lb", [(RM, CM), (CM, RM), (RM, RM), (CM, CM)])
+@pytest.mark.parametrize("dtype_in,dtype_out,tol", [
+    (orc.F16, orc.F16, 1e-3),    # <f16, f16, f32>
+    (orc.BF16, orc.BF16, 4e-3),  # <bf16, bf16, f32>: one bf16 ulp (2^-8) of a value v costs v/(2v+1) * 2^-8 <= 2e-3
+    (orc.F32, orc.F32, 1e-5),    # <f32, f32, f32> (wave-tile kernel only)
+])
+def test_narrow_output_and_f32_type_combinations(dtype_in, dtype_out, tol, la, lb, algo):
+    """Input/Output/Compute triples of test/gemm/gemm_common_test_params.hpp:51-111 beyond the
+    f32-output ones: C and D in the input type, f32 compute."""
+    if dtype_in == orc.F32 and algo == rw.GEMM_BLOCKED:
+        pytest.skip("f32 inputs run on the wave-tile kernel only")
+    m, n, k = 256, 384, 192
+    a = uniform_bits(51, dtype_in, m * k)
+    b = uniform_bits(52, dtype_in, k * n)
+    c = uniform_bits(53, dtype_out, m * n)
+    got = run_gemm(dtype_in, dtype_out, la, lb, RM, m, n, k, a, b, c, 1.5, -0.5, algo)
+    want = orc.gemm(dtype_in, dtype_out, la, lb, RM, RM, m, n, k, a, b, c, 1.5, -0.5)
+    check(dtype_in, dtype_out, got, want, tol)
+
+
 # ---------------------------------------------------------------- config 1: simple_hgemm workload
 @pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED, rw.GEMM_AUTO])
 def test_config1_256_cubed_f16_alpha_beta_2(algo):
