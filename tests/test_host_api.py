@@ -53,7 +53,8 @@ def test_gemm_argument_validation(lib):
     assert _gemm(lib, m=0) == 1
     assert _gemm(lib, la=7) == 1
     assert _gemm(lib, c=None, beta=1.0) == 1
-    assert _gemm(lib, dtype_in=rw.F32) == 2
+    assert _gemm(lib, dtype_in=rw.I32) == 2
+    assert _gemm(lib, dtype_in=rw.BF16, dtype_out=rw.F16) == 2
     assert _gemm(lib, dtype_in=rw.I8, dtype_out=rw.F32) == 2
     assert _gemm(lib, dtype_in=rw.I8, dtype_out=rw.I32, alpha=0.5) == 1
     assert _gemm(lib, m=24) == 3
