@@ -9,7 +9,7 @@
 //   * one wave owns a whole sample: the m <= 32 feature rows are one 32-row MFMA operand, so
 //     Z = F F^T is K/16 v_mfma_f32_32x32x16_f16 with the SAME registers as both multiplicands
 //     (applyTranspose of the A fragment is the B fragment);
-//   * a workgroup of 8 waves owns 8 consecutive samples, whose inputs and outputs are
+//   * a workgroup of 2, 4 or 8 waves owns as many consecutive samples, whose inputs and outputs are
 //     contiguous in memory: features arrive as whole-wave 1 KiB direct-to-LDS copies, results
 //     are assembled in LDS and leave as 16-byte coalesced stores;
 //   * backward rebuilds the symmetric matrix G in registers from the LDS-staged upstream
@@ -28,8 +28,9 @@ namespace rocwmma_amd
 {
     namespace
     {
-        constexpr uint32_t kSamplesPerWg = 8; // = waves per workgroup: one sample per wave
-        constexpr uint32_t kWavesPerWg   = 8;
+        // A workgroup owns `Samples` consecutive samples, one per wave: 8 for large batches (longest
+        // contiguous stores), 4 or 2 when the batch would otherwise not give every compute unit
+        // several workgroups (batch 2048: 7 us with 4 samples per workgroup against 19 us with 8).
         constexpr uint32_t kMaxM         = 32;
 
         typedef uint32_t u32x4_t __attribute__((ext_vector_type(4), may_alias));
@@ -109,8 +110,8 @@ namespace rocwmma_amd
         };
 
         // ------------------------------------------------------------------ forward
-        template <uint32_t K>
-        __global__ void __launch_bounds__(64 * kWavesPerWg)
+        template <uint32_t K, uint32_t Samples>
+        __global__ void __launch_bounds__(64 * Samples)
             dlrmFwdKernel(const float16_t* __restrict__ input, float16_t* __restrict__ output, uint32_t m, uint32_t batch)
         {
             constexpr uint32_t KSteps = K / 16u;
@@ -121,18 +122,18 @@ namespace rocwmma_amd
 
             extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
             const uint32_t width     = K + (m * (m - 1u)) / 2u;
-            const uint32_t tileBytes = (((kSamplesPerWg - 1u) * m + kMaxM) * Tile::rowBytes + 1023u) & ~1023u;
+            const uint32_t tileBytes = (((Samples - 1u) * m + kMaxM) * Tile::rowBytes + 1023u) & ~1023u;
             char*          ldsIn     = ldsRaw;
             float16_t*     ldsOut    = reinterpret_cast<float16_t*>(ldsRaw + tileBytes);
 
             const uint32_t lane    = threadIdx.x & 63u;
             const uint32_t wave    = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-            const uint32_t sample0 = blockIdx.x * kSamplesPerWg;
-            const uint32_t nHere   = min(kSamplesPerWg, batch - sample0);
+            const uint32_t sample0 = blockIdx.x * Samples;
+            const uint32_t nHere   = min(Samples, batch - sample0);
 
             // all feature rows of the workgroup's samples: one contiguous block
             Tile::template asyncLoad<false>(ldsIn, input + static_cast<size_t>(sample0) * m * K, nHere * m * Tile::rowBytes,
-                                            wave, kWavesPerWg, lane);
+                                            wave, Samples, lane);
             lds::waitCopiesAndReads<0>();
             __syncthreads();
 
@@ -181,8 +182,8 @@ namespace rocwmma_amd
         }
 
         // ------------------------------------------------------------------ backward
-        template <uint32_t K>
-        __global__ void __launch_bounds__(64 * kWavesPerWg) dlrmBwdKernel(const float16_t* __restrict__ input,
+        template <uint32_t K, uint32_t Samples>
+        __global__ void __launch_bounds__(64 * Samples) dlrmBwdKernel(const float16_t* __restrict__ input,
                                                                            const float16_t* __restrict__ upstream,
                                                                            float16_t* __restrict__ grad,
                                                                            float16_t* __restrict__ mlpGrad,
@@ -198,14 +199,14 @@ namespace rocwmma_amd
 
             extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
             const uint32_t width     = K + (m * (m - 1u)) / 2u;
-            const uint32_t tileBytes = (((kSamplesPerWg - 1u) * m + kMaxM) * Tile::rowBytes + 1023u) & ~1023u;
+            const uint32_t tileBytes = (((Samples - 1u) * m + kMaxM) * Tile::rowBytes + 1023u) & ~1023u;
             char*          ldsF      = ldsRaw; // features in, gradients out
             float16_t*     ldsUp     = reinterpret_cast<float16_t*>(ldsRaw + tileBytes);
 
             const uint32_t lane    = threadIdx.x & 63u;
             const uint32_t wave    = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-            const uint32_t sample0 = blockIdx.x * kSamplesPerWg;
-            const uint32_t nHere   = min(kSamplesPerWg, batch - sample0);
+            const uint32_t sample0 = blockIdx.x * Samples;
+            const uint32_t nHere   = min(Samples, batch - sample0);
 
             // Rows past the last sample are read as contraction rows >= m (multiplied by the zero
             // columns of G): they must hold finite values, so clear everything behind the features
@@ -214,7 +215,7 @@ namespace rocwmma_amd
             for(uint32_t i = featBytes / 16u + threadIdx.x; i < tileBytes / 16u; i += blockDim.x)
                 reinterpret_cast<u32x4_t*>(ldsF)[i] = u32x4_t{0u, 0u, 0u, 0u};
             // features: direct copies, segment-swizzled for the transposing reads
-            Tile::template asyncLoad<true>(ldsF, input + static_cast<size_t>(sample0) * m * K, featBytes, wave, kWavesPerWg, lane);
+            Tile::template asyncLoad<true>(ldsF, input + static_cast<size_t>(sample0) * m * K, featBytes, wave, Samples, lane);
             // upstream gradients (contiguous for the workgroup's samples)
             copyIn(ldsUp, upstream + static_cast<size_t>(sample0) * width, nHere * width);
             lds::waitCopiesAndReads<0>();
@@ -316,10 +317,10 @@ namespace rocwmma_amd
             }
         }
 
-        template <uint32_t K>
+        template <uint32_t K, uint32_t Samples>
         uint32_t tileBytesFor(uint32_t m)
         {
-            return (((kSamplesPerWg - 1u) * m + kMaxM) * K * 2u + 1023u) & ~1023u;
+            return (((Samples - 1u) * m + kMaxM) * K * 2u + 1023u) & ~1023u;
         }
 
         template <typename Kernel>
@@ -333,34 +334,71 @@ namespace rocwmma_amd
             return ROCWMMA_AMD_OK;
         }
 
+        template <uint32_t K, uint32_t Samples>
+        int launchFwdS(const void* input, void* output, uint32_t m, uint32_t batch, hipStream_t stream)
+        {
+            const uint32_t width  = K + (m * (m - 1u)) / 2u;
+            const uint32_t lds    = tileBytesFor<K, Samples>(m) + ((Samples * width * 2u + 15u) & ~15u);
+            const uint32_t grid   = (batch + Samples - 1u) / Samples;
+            auto           kernel = dlrmFwdKernel<K, Samples>;
+            if(int rc = optInLds(kernel, lds))
+                return rc;
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(64u * Samples), lds, stream, static_cast<const float16_t*>(input),
+                               static_cast<float16_t*>(output), m, batch);
+            return launchStatus();
+        }
+
+        template <uint32_t K, uint32_t Samples>
+        int launchBwdS(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t batch,
+                       hipStream_t stream)
+        {
+            const uint32_t width  = K + (m * (m - 1u)) / 2u;
+            const uint32_t lds    = tileBytesFor<K, Samples>(m) + ((Samples * width * 2u + 15u) & ~15u);
+            const uint32_t grid   = (batch + Samples - 1u) / Samples;
+            auto           kernel = dlrmBwdKernel<K, Samples>;
+            if(int rc = optInLds(kernel, lds))
+                return rc;
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(64u * Samples), lds, stream, static_cast<const float16_t*>(input),
+                               static_cast<const float16_t*>(upstream), static_cast<float16_t*>(grad),
+                               static_cast<float16_t*>(mlpGrad), m, batch);
+            return launchStatus();
+        }
+        // samples per workgroup for a batch: 8 once that still leaves >= 8 workgroups per compute unit
+        inline uint32_t samplesFor(uint32_t batch)
+        {
+            const uint32_t cus = computeUnits();
+            if(batch >= 64u * cus)
+                return 8u;
+            return batch >= 8u * cus ? 4u : 2u;
+        }
+
         template <uint32_t K>
         int launchFwd(const void* input, void* output, uint32_t m, uint32_t batch, hipStream_t stream)
         {
-            const uint32_t width  = K + (m * (m - 1u)) / 2u;
-            const uint32_t lds    = tileBytesFor<K>(m) + ((kSamplesPerWg * width * 2u + 15u) & ~15u);
-            const uint32_t grid   = (batch + kSamplesPerWg - 1u) / kSamplesPerWg;
-            auto           kernel = dlrmFwdKernel<K>;
-            if(int rc = optInLds(kernel, lds))
-                return rc;
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(64u * kWavesPerWg), lds, stream, static_cast<const float16_t*>(input),
-                               static_cast<float16_t*>(output), m, batch);
-            return launchStatus();
+            switch(samplesFor(batch))
+            {
+            case 8:
+                return launchFwdS<K, 8>(input, output, m, batch, stream);
+            case 4:
+                return launchFwdS<K, 4>(input, output, m, batch, stream);
+            default:
+                return launchFwdS<K, 2>(input, output, m, batch, stream);
+            }
         }
 
         template <uint32_t K>
         int launchBwd(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t batch,
                       hipStream_t stream)
         {
-            const uint32_t width  = K + (m * (m - 1u)) / 2u;
-            const uint32_t lds    = tileBytesFor<K>(m) + ((kSamplesPerWg * width * 2u + 15u) & ~15u);
-            const uint32_t grid   = (batch + kSamplesPerWg - 1u) / kSamplesPerWg;
-            auto           kernel = dlrmBwdKernel<K>;
-            if(int rc = optInLds(kernel, lds))
-                return rc;
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(64u * kWavesPerWg), lds, stream, static_cast<const float16_t*>(input),
-                               static_cast<const float16_t*>(upstream), static_cast<float16_t*>(grad),
-                               static_cast<float16_t*>(mlpGrad), m, batch);
-            return launchStatus();
+            switch(samplesFor(batch))
+            {
+            case 8:
+                return launchBwdS<K, 8>(input, upstream, grad, mlpGrad, m, batch, stream);
+            case 4:
+                return launchBwdS<K, 4>(input, upstream, grad, mlpGrad, m, batch, stream);
+            default:
+                return launchBwdS<K, 2>(input, upstream, grad, mlpGrad, m, batch, stream);
+            }
         }
     } // namespace
 
