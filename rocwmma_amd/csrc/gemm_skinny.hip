@@ -3,15 +3,19 @@
 //
 // At these shapes (the reference's GEMM kernels, samples/perf_hgemm.cpp:518-714, need whole
 // 128-wide macro tiles in M and would leave most of the chip idle) the job is streaming the
-// weights from HBM exactly once, so the kernel is built for memory-level parallelism, written
-// with the public fragment API only:
-//   * a workgroup of four waves owns 16*NBlocks weight rows and ALL token rows;
-//   * the four waves split K; each wave walks its quarter in 128-byte steps with
-//     16 x 16 x 128 fragments (one v_mfma_f32_16x16x128_f8f6f4, or two v_mfma_i32_16x16x64_i8),
-//     so a weight row is read as whole 128-byte lines and many lines are in flight per wave;
-//   * the four partial accumulators meet in LDS; the sum is formed in a fixed order, so the
-//     result is deterministic (and bit-exact for int8).
+// weights from HBM exactly once, so the kernel is built for memory-level parallelism:
+//   * a workgroup of 16 waves = 4 blocks of 16 weight rows x 4 slices of K; every wave walks
+//     its K slice of its weight rows in 128-byte steps with 16 x 16 x 128 fragments loaded
+//     straight from global memory (one v_mfma_f32_16x16x128_f8f6f4, or two
+//     v_mfma_i32_16x16x64_i8, per step), several steps in flight;
+//   * the token matrix A is copied into LDS once per workgroup (direct-to-LDS copies, 16-byte
+//     chunks XOR-swizzled by row so the operand reads are bank-conflict free) and read from
+//     there: fetched from the L2 by every wave, the same few KiB of A cost as much time as
+//     the whole weight stream (17 us against 9 us at M = 16, N = 14336, K = 4096);
+//   * the four K-slice partial accumulators of a block meet in LDS; the sum is formed in a
+//     fixed order, so the result is deterministic (and bit-exact for int8).
 #include "common.hpp"
+#include <rocwmma/rocwmma_lds.hpp>
 
 using namespace rocwmma;
 
@@ -19,10 +23,13 @@ namespace rocwmma_amd
 {
     namespace
     {
-        constexpr uint32_t kSkinnyWaves = 4;
-        constexpr uint32_t kSkinnyK     = 128; // K elements (= bytes) per fragment step
+        constexpr uint32_t kSkinnySlices = 4;   // K slices per block of weight rows
+        constexpr uint32_t kSkinnyBlocks = 4;   // blocks of 16 weight rows per workgroup
+        constexpr uint32_t kSkinnyWaves  = kSkinnySlices * kSkinnyBlocks;
+        constexpr uint32_t kSkinnyK      = 128; // K elements (= bytes) per fragment step
+        constexpr uint32_t kSkinnyMaxA   = 131072; // bytes of LDS the token matrix may take
 
-        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t NBlocks>
+        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t Ahead>
         __global__ void __launch_bounds__(64 * kSkinnyWaves) gemmSkinnyKernel(uint32_t    m,
                                                                               uint32_t    n,
                                                                               uint32_t    k,
@@ -41,116 +48,162 @@ namespace rocwmma_amd
             using FragB   = fragment<matrix_b, 16, 16, kSkinnyK, InT, col_major>;
             using FragAcc = fragment<accumulator, 16, 16, kSkinnyK, CompT>;
             using FragC   = fragment<accumulator, 16, 16, kSkinnyK, OutT, row_major>;
-            constexpr uint32_t Blocks = MBlocks * NBlocks;
+            using MapA    = detail::InputMap<16, kSkinnyK, 16, detail::packClassOf<InT>()>;
+            static_assert(sizeof(InT) == 1, "8-bit operands");
 
-            extern __shared__ __attribute__((aligned(16))) char ldsRaw[];
-            // partial[wave][block][lane] : the 4 accumulator registers of a lane as one 16-byte unit
+            extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
+            char* aTile = ldsRaw; // [m][k] bytes, chunk c of row r at chunk position c ^ (r % 16)
+            // partial[wave][mblock][lane] : the 4 accumulator registers of a lane as one 16-byte unit
             using Quad    = CompT __attribute__((ext_vector_type(4)));
-            Quad* partial = reinterpret_cast<Quad*>(ldsRaw);
+            Quad* partial = reinterpret_cast<Quad*>(ldsRaw + m * k);
 
-            const uint32_t lane = threadIdx.x & 63u;
-            const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-            const uint32_t n0   = blockIdx.x * NBlocks * 16u;
-            const uint32_t kLen = k / kSkinnyWaves;
-            const uint32_t kBeg = wave * kLen;
+            const uint32_t lane   = threadIdx.x & 63u;
+            const uint32_t wave   = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            const uint32_t slice  = wave % kSkinnySlices;
+            const uint32_t blk    = wave / kSkinnySlices;
+            const uint32_t nBlock = blockIdx.x * kSkinnyBlocks + blk; // block of 16 weight rows
+            const bool     live   = nBlock * 16u < n;
+            const uint32_t n0     = (live ? nBlock : 0u) * 16u; // idle waves shadow block 0, store nothing
+            const uint32_t kLen   = k / kSkinnySlices;
+            const uint32_t kBeg   = slice * kLen;
 
-            FragAcc acc[MBlocks][NBlocks];
+            // A -> LDS: whole-wave 1 KiB copies, k / 1024 per row
+            {
+                const uint32_t perRow = k / 1024u;
+                const uint32_t copies = m * perRow;
+                for(uint32_t j = wave; j < copies; j += kSkinnyWaves)
+                {
+                    const uint32_t r   = j / perRow;
+                    const uint32_t pos = (j % perRow) * 64u + lane; // chunk position inside the LDS row
+                    lds::asyncCopy16(aTile + r * k + (j % perRow) * 1024u,
+                                     reinterpret_cast<const char*>(a) + static_cast<size_t>(r) * lda + ((pos ^ (r & 15u)) << 4));
+                }
+            }
+
+            FragAcc acc[MBlocks];
 #pragma unroll
             for(uint32_t i = 0; i < MBlocks; ++i)
-#pragma unroll
-                for(uint32_t j = 0; j < NBlocks; ++j)
-                    fill_fragment(acc[i][j], static_cast<CompT>(0));
+                fill_fragment(acc[i], static_cast<CompT>(0));
 
-            const InT* bPtr = b + static_cast<size_t>(n0) * ldb + kBeg;
-            const InT* aPtr = a + kBeg;
-#pragma unroll 8
-            for(uint32_t kk = 0; kk < kLen; kk += kSkinnyK)
+            // this lane's A operand rows in LDS and its swizzle
+            const uint32_t aRow = lane & 15u;
+            const InT*     bPtr = b + static_cast<size_t>(n0) * ldb + kBeg;
+
+            auto loadB = [&](FragB(&fb)[Ahead], uint32_t kk) {
+#pragma unroll
+                for(uint32_t u = 0; u < Ahead; ++u)
+                    load_matrix_sync(fb[u], bPtr + kk + u * kSkinnyK, ldb);
+            };
+            auto multiply = [&](FragB(&fb)[Ahead], uint32_t kk) {
+#pragma unroll
+                for(uint32_t u = 0; u < Ahead; ++u)
+#pragma unroll
+                    for(uint32_t i = 0; i < MBlocks; ++i)
+                    {
+                        FragA          fa;
+                        const uint32_t row = i * 16u + aRow;
+#pragma unroll
+                        for(uint32_t ch = 0; ch < MapA::nchunks; ++ch)
+#pragma unroll
+                            for(uint32_t piece = 0; piece < MapA::kpack / 16u; ++piece)
+                            {
+                                const uint32_t kByte = kBeg + kk + u * kSkinnyK + MapA::chunkK(ch, lane) + piece * 16u;
+                                detail::copyBytes<16u>(fa.x + ch * MapA::kpack + piece * 16u,
+                                                       aTile + row * k + (((kByte >> 4) ^ (row & 15u)) << 4));
+                            }
+                        mma_sync(acc[i], fa, fb[u], acc[i]);
+                    }
+            };
+
+            // the first batch of weight fragments is requested before waiting for A
+            FragB fb[Ahead];
+            loadB(fb, 0u);
+            lds::waitCopiesAndReads<0>();
+            __syncthreads();
+            multiply(fb, 0u);
+            for(uint32_t kk = Ahead * kSkinnyK; kk < kLen; kk += Ahead * kSkinnyK)
             {
-                FragB fb[NBlocks];
-#pragma unroll
-                for(uint32_t j = 0; j < NBlocks; ++j)
-                    load_matrix_sync(fb[j], bPtr + static_cast<size_t>(j * 16u) * ldb + kk, ldb);
-#pragma unroll
-                for(uint32_t i = 0; i < MBlocks; ++i)
-                {
-                    FragA fa;
-                    load_matrix_sync(fa, aPtr + static_cast<size_t>(i * 16u) * lda + kk, lda);
-#pragma unroll
-                    for(uint32_t j = 0; j < NBlocks; ++j)
-                        mma_sync(acc[i][j], fa, fb[j], acc[i][j]);
-                }
+                loadB(fb, kk);
+                multiply(fb, kk);
             }
 
             // meet in LDS
 #pragma unroll
             for(uint32_t i = 0; i < MBlocks; ++i)
-#pragma unroll
-                for(uint32_t j = 0; j < NBlocks; ++j)
-                    partial[(wave * Blocks + i * NBlocks + j) * 64u + lane] = *reinterpret_cast<Quad*>(acc[i][j].x);
+                partial[(wave * MBlocks + i) * 64u + lane] = *reinterpret_cast<Quad*>(acc[i].x);
             __syncthreads();
 
-            // block q is finished by wave q % 4: fixed summation order wave 0, 1, 2, 3
+            // token block i of a weight block is finished by the wave of slice i % 4: fixed
+            // summation order slice 0, 1, 2, 3
 #pragma unroll
             for(uint32_t i = 0; i < MBlocks; ++i)
+            {
+                if(i % kSkinnySlices != slice || !live)
+                    continue;
+                const uint32_t first = blk * kSkinnySlices;
+                Quad           sum   = partial[((first + 0u) * MBlocks + i) * 64u + lane];
 #pragma unroll
-                for(uint32_t j = 0; j < NBlocks; ++j)
+                for(uint32_t w = 1; w < kSkinnySlices; ++w)
+                    sum += partial[((first + w) * MBlocks + i) * 64u + lane];
+                const size_t row = i * 16u;
+                const size_t col = n0;
+                FragC        fc;
+                if(beta != static_cast<CompT>(0))
                 {
-                    const uint32_t q = i * NBlocks + j;
-                    if(q % kSkinnyWaves != wave)
-                        continue;
-                    Quad sum = partial[(0u * Blocks + q) * 64u + lane];
+                    load_matrix_sync(fc, c + row * ldc + col, ldc);
 #pragma unroll
-                    for(uint32_t w = 1; w < kSkinnyWaves; ++w)
-                        sum += partial[(w * Blocks + q) * 64u + lane];
-                    const size_t row = i * 16u;
-                    const size_t col = n0 + j * 16u;
-                    FragC        fc;
-                    if(beta != static_cast<CompT>(0))
-                    {
-                        load_matrix_sync(fc, c + row * ldc + col, ldc);
-#pragma unroll
-                        for(uint32_t e = 0; e < 4u; ++e)
-                            fc.x[e] = static_cast<OutT>(alpha * sum[e] + beta * static_cast<CompT>(fc.x[e]));
-                    }
-                    else
-                    {
-#pragma unroll
-                        for(uint32_t e = 0; e < 4u; ++e)
-                            fc.x[e] = static_cast<OutT>(alpha * sum[e]);
-                    }
-                    store_matrix_sync(d + row * ldd + col, fc, ldd);
+                    for(uint32_t e = 0; e < 4u; ++e)
+                        fc.x[e] = static_cast<OutT>(alpha * sum[e] + beta * static_cast<CompT>(fc.x[e]));
                 }
+                else
+                {
+#pragma unroll
+                    for(uint32_t e = 0; e < 4u; ++e)
+                        fc.x[e] = static_cast<OutT>(alpha * sum[e]);
+                }
+                store_matrix_sync(d + row * ldd + col, fc, ldd);
+            }
         }
 
-        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t NBlocks>
+        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t Ahead>
         int launchOne(GemmArgs const& g, hipStream_t stream)
         {
-            constexpr uint32_t lds    = kSkinnyWaves * MBlocks * NBlocks * 1024u;
-            auto               kernel = gemmSkinnyKernel<InT, OutT, CompT, MBlocks, NBlocks>;
+            const uint32_t lds    = g.m * g.k + kSkinnyWaves * MBlocks * 1024u;
+            auto           kernel = gemmSkinnyKernel<InT, OutT, CompT, MBlocks, Ahead>;
             if(lds > 65536u
                && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(lds))
                       != hipSuccess)
                 return ROCWMMA_AMD_LAUNCH_FAILED;
-            hipLaunchKernelGGL(kernel, dim3(g.n / (NBlocks * 16u)), dim3(64u * kSkinnyWaves), lds, stream, g.m, g.n, g.k,
-                               static_cast<InT const*>(g.a), static_cast<InT const*>(g.b), static_cast<OutT const*>(g.c),
-                               static_cast<OutT*>(g.d), g.lda, g.ldb, g.ldc, g.ldd, static_cast<CompT>(g.alpha),
-                               static_cast<CompT>(g.beta));
+            const uint32_t nBlocks = g.n / 16u;
+            hipLaunchKernelGGL(kernel, dim3((nBlocks + kSkinnyBlocks - 1u) / kSkinnyBlocks), dim3(64u * kSkinnyWaves), lds,
+                               stream, g.m, g.n, g.k, static_cast<InT const*>(g.a), static_cast<InT const*>(g.b),
+                               static_cast<OutT const*>(g.c), static_cast<OutT*>(g.d), g.lda, g.ldb, g.ldc, g.ldd,
+                               static_cast<CompT>(g.alpha), static_cast<CompT>(g.beta));
             return launchStatus();
         }
 
         template <typename InT, typename OutT, typename CompT>
         int pickShape(GemmArgs const& g, hipStream_t stream)
         {
-            if(g.m % 16u != 0u || g.m > 32u || g.k % (kSkinnyWaves * kSkinnyK) != 0u)
+            // whole 1 KiB copies per row of A, whole fragment steps per K slice, A resident in LDS
+            if(g.m % 16u != 0u || g.m > 32u || g.n % 16u != 0u || g.k % 1024u != 0u || g.m * g.k > kSkinnyMaxA)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-            const uint32_t mBlocks = g.m / 16u;
-            // 16 weight rows per workgroup: the most workgroups and the most loads in flight
-            if(g.n % 16u != 0u)
-                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-            if(mBlocks == 1u)
-                return launchOne<InT, OutT, CompT, 1, 1>(g, stream);
-            return launchOne<InT, OutT, CompT, 2, 1>(g, stream);
+            // K steps of a wave's slice fetched together: as many as divide the slice, up to 8
+            const uint32_t steps = g.k / (kSkinnySlices * kSkinnyK);
+            if(g.m == 16u)
+            {
+                if(steps % 8u == 0u)
+                    return launchOne<InT, OutT, CompT, 1, 8>(g, stream);
+                if(steps % 4u == 0u)
+                    return launchOne<InT, OutT, CompT, 1, 4>(g, stream);
+                return launchOne<InT, OutT, CompT, 1, 2>(g, stream);
+            }
+            if(steps % 8u == 0u)
+                return launchOne<InT, OutT, CompT, 2, 8>(g, stream);
+            if(steps % 4u == 0u)
+                return launchOne<InT, OutT, CompT, 2, 4>(g, stream);
+            return launchOne<InT, OutT, CompT, 2, 2>(g, stream);
         }
     } // namespace
 

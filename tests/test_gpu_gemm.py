@@ -181,12 +181,13 @@ def test_leading_dimensions_larger_than_extent():
         assert np.all(got[:, n:] == 777.0)
 
 
-@pytest.mark.parametrize("m", [16, 32, 48, 80, 112, 128])
+@pytest.mark.parametrize("m,k", [(16, 1536), (32, 1536), (48, 1536), (80, 1536), (112, 1536), (128, 1536),
+                                 (16, 1024), (32, 1024), (16, 2048), (32, 2048), (16, 4096), (32, 4096)])
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3, orc.E5M2])
-def test_skinny_weight_streaming_kernel(dtype_in, m):
+def test_skinny_weight_streaming_kernel(dtype_in, m, k):
     """M <= 128 token rows, 8-bit, A row / B col: served by the K-split weight-streaming kernel
     (AUTO).  int8 must be bit-exact; the wave-tile kernel gives the same answer."""
-    n, k = 352, 1536
+    n = 352  # k: 3, 2, 4 and 8 fragment steps per wave (the kernel fetches 1, 2, 4 or 8 at a time)
     if dtype_in == orc.I8:
         a, b = uniform_bits(71, orc.I8, m * k), uniform_bits(72, orc.I8, k * n)
         c = uniform_bits(73, orc.I32, m * n)
