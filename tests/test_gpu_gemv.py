@@ -35,13 +35,16 @@ def test_config4_full_shapes(m, k, ncols, beta):
 
 @pytest.mark.parametrize("m,k,ncols", [(1, 8, 1), (3, 520, 2), (37, 1000, 4), (130, 72, 8), (255, 4104, 1),
                                        (2, 16, 1), (5, 24, 1), (64, 16384, 8), (100, 32776, 4), (9, 65536, 2),
-                                       (1000, 8, 8), (4100, 264, 2)])
+                                       (1000, 8, 8), (4100, 264, 2),
+                                       # m a multiple of 16 and k a multiple of 4096
+                                       (48, 4096, 4), (16, 8192, 8), (2064, 4096, 8), (80, 8192, 4)])
 def test_ragged_shapes(m, k, ncols):
     run(m, k, ncols, 2.1, 2.1, 99)
 
 
 def test_padded_leading_dimension():
     run(64, 512, 4, 1.0, 0.0, 5, lda=640)
+    run(64, 4096, 8, 1.0, 0.5, 6, lda=4096 + 64)
 
 
 def test_equals_gemm_with_n_columns():
