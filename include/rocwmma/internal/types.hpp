@@ -37,6 +37,17 @@ namespace rocwmma
     using float8_t  = __hip_fp8_e4m3;
     using bfloat8_t = __hip_fp8_e5m2;
 
+    // Names of element types of other devices, kept so that code which only *mentions* them
+    // (type lists, std::is_same tests; e.g. the reference's test/gemm/gemm_test_traits.hpp:115-185)
+    // still compiles.  gfx950's matrix cores have neither the fnuz fp8 formats nor xf32: these
+    // types cannot be the element type of a fragment here.
+    using float8_fnuz_t  = __hip_fp8_e4m3_fnuz;
+    using bfloat8_fnuz_t = __hip_fp8_e5m2_fnuz;
+    struct xfloat32_t
+    {
+        float data;
+    };
+
     namespace detail
     {
         // Matrix-core operand class of an element type.

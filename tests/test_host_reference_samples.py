@@ -50,3 +50,70 @@ def test_reference_sample_compiles_against_these_headers(sample, tmp_path):
     assert ours in deps, "the sample did not pick up this repository's rocwmma.hpp"
     assert os.path.join(REFERENCE, "library") not in deps
     assert "/opt/rocm/include/rocwmma" not in deps
+
+
+# The reference's own test kernels (device side only; their GTest hosts are not involved).  They
+# gate their bodies on the architecture identifiers they know, so the device pass is told to report
+# gfx942's identifier (ROCWMMA_AMD_REPORT_ARCH_ID); nothing else is changed.
+TEST_KERNEL_UNITS = {
+    "unit_load_store_fill_contamination_coop": """
+#include <hip/hip_runtime.h>
+#include "load_store_matrix_sync_test/device/load_store_matrix_sync.hpp"
+#include "fill_fragment_test/device/fill_fragment.hpp"
+#include "contamination_test/device/load_contamination.hpp"
+#include "contamination_test/device/store_contamination.hpp"
+#include "load_store_matrix_coop_sync_test/device/load_store_matrix_coop_sync.hpp"
+namespace rocwmma {
+template __global__ void LoadStoreMatrixSyncA<32, 16, float16_t, row_major>(uint32_t, uint32_t, float16_t const*, float16_t*, uint32_t, float16_t, float16_t);
+template __global__ void LoadStoreMatrixSyncA<256, 8, float32_t, col_major>(uint32_t, uint32_t, float32_t const*, float32_t*, uint32_t, float32_t, float32_t);
+template __global__ void LoadStoreMatrixSyncB<64, 32, int8_t, col_major>(uint32_t, uint32_t, int8_t const*, int8_t*, uint32_t, int8_t, int8_t);
+template __global__ void LoadStoreMatrixSyncAcc<32, 32, float32_t, row_major>(uint32_t, uint32_t, float32_t const*, float32_t*, uint32_t, float32_t, float32_t);
+}
+""",
+    "dlrm_test_kernels": """
+#include <hip/hip_runtime.h>
+#include <rocwmma/rocwmma.hpp>
+#include "dlrm/device/dlrm_dot_fwd.hpp"
+#include "dlrm/device/dlrm_dot_bwd.hpp"
+namespace rocwmma {
+template __global__ void dlrmDotFwd<float16_t, 16>(const float16_t* __restrict, float16_t* __restrict, float*, uint, uint, uint, uint, uint, uint);
+template __global__ void trilReconstruct<float16_t>(const float16_t* __restrict, float16_t* __restrict, uint, uint, uint, uint, uint);
+template __global__ void dlrmDotBwd<float16_t, 16>(const float16_t* __restrict, const float16_t* __restrict, float16_t* __restrict, float16_t* __restrict, float16_t* __restrict, uint, uint, uint, uint, uint, uint);
+}
+""",
+    "gemm_single_block_test_kernel": """
+#include <hip/hip_runtime.h>
+#include <iostream>
+#include <rocwmma/rocwmma.hpp>
+#include "gemm/gemm_PGR0_LB0_MP0_SB_NC/device/kernel_device_func.hpp"
+namespace rocwmma {
+template __global__ void gemm_PGR0_LB0_MP0_SB_NC<32, 32, 16, float16_t, float32_t, float32_t, row_major, col_major, row_major, row_major, 128, 2, 64, 0x942>(uint32_t, uint32_t, uint32_t, float16_t const*, float16_t const*, float32_t const*, float32_t*, uint32_t, uint32_t, uint32_t, uint32_t, float32_t, float32_t);
+template __global__ void gemm_PGR0_LB0_MP0_SB_NC<16, 16, 64, int8_t, int32_t, int32_t, col_major, row_major, row_major, row_major, 64, 4, 64, 0x942>(uint32_t, uint32_t, uint32_t, int8_t const*, int8_t const*, int32_t const*, int32_t*, uint32_t, uint32_t, uint32_t, uint32_t, int32_t, int32_t);
+}
+""",
+}
+
+
+@pytest.mark.parametrize("unit", sorted(TEST_KERNEL_UNITS))
+def test_reference_test_kernels_compile_against_these_headers(unit, tmp_path):
+    tests_dir = os.path.join(REFERENCE, "test")
+    hipcc = _hipcc()
+    if not os.path.isdir(tests_dir):
+        pytest.skip("reference checkout not present")
+    if hipcc is None:
+        pytest.skip("hipcc not present")
+    src = tmp_path / (unit + ".cpp")
+    src.write_text(TEST_KERNEL_UNITS[unit])
+    obj = tmp_path / (unit + ".o")
+    dep = tmp_path / (unit + ".d")
+    cmd = [hipcc, "--offload-arch=gfx950", "-std=c++17", "-O1", "-DROCWMMA_AMD_REPORT_ARCH_ID=0x942",
+           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(tests_dir, "unit"), "-I" + tests_dir,
+           "-I" + os.path.join(tests_dir, "gemm"),
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+           "-MD", "-MF", str(dep), "-c", str(src), "-o", str(obj)]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert res.returncode == 0, res.stdout[-3000:]
+    deps = " ".join(p.read_text() for p in tmp_path.glob("*.d"))
+    assert os.path.join(ROOT, "include", "rocwmma", "rocwmma.hpp") in deps
+    assert os.path.join(REFERENCE, "library") not in deps
+    assert "/opt/rocm/include/rocwmma" not in deps
