@@ -16,6 +16,7 @@
 //     reading X from LDS so the extra columns cost no L1/L2 traffic.
 //   If X does not fit the LDS the split kernel reads X through the caches instead.
 #include "common.hpp"
+#include <rocwmma/rocwmma_lds.hpp>
 
 namespace rocwmma_amd
 {
@@ -206,6 +207,144 @@ namespace rocwmma_amd
             }
         }
 
+        // Quad kernel for 4 and 8 right-hand sides: the dot products run on the matrix core's
+        // small-block instruction v_mfma_f32_4x4x4_16B_f16 (16 independent 4 x 4 x 4 blocks per
+        // wave), which fits a row stream: a lane fetches 16 bytes, lanes 4b..4b+3 hold the same
+        // 16-byte K chunk of 4 consecutive rows of A (block b of the instruction), so one load
+        // instruction reads 4 rows x 256 contiguous bytes and feeds two instructions per group of 4
+        // columns.  Against the v_dot2 kernels this is 8x fewer arithmetic instructions, 4x fewer
+        // LDS reads of X and 6x fewer cross-lane reduction steps (8192 x 8192, 8 columns:
+        // 30 -> 24.6 us; 14336 x 4096: 30 -> 20.9 us).
+        //   * workgroup = 16 waves = 4 row-quad lanes x 4 slices of K; X is copied into LDS once
+        //     (direct-to-LDS, the chunks of column c XOR-swizzled by (c % 4) * 4 so the 16 lanes
+        //     of a quarter-wave, 4 chunks x 4 columns, read 16 distinct bank groups);
+        //   * a wave walks its K slice of its 4 rows, `Unroll` 1 KiB loads in flight;
+        //   * block b accumulates the products of its own K chunks; at the end of a row quad the
+        //     16 blocks are summed with 4 cross-lane steps, the K-slice partial sums meet in LDS
+        //     and are added in slice order (deterministic).
+        constexpr uint32_t kQuadWaves = 16, kQuadSlices = 4;
+
+        template <uint32_t NCols, uint32_t Unroll>
+        __global__ void __launch_bounds__(kQuadWaves * 64u) gemvQuadKernel(uint32_t        m,
+                                                                           uint32_t        k,
+                                                                           const _Float16* a,
+                                                                           uint32_t        lda,
+                                                                           const _Float16* x,
+                                                                           uint32_t        ldx,
+                                                                           float*          y,
+                                                                           uint32_t        ldy,
+                                                                           float           alpha,
+                                                                           float           beta,
+                                                                           uint32_t        quadsPerWg)
+        {
+            typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+            typedef float    float4_t __attribute__((ext_vector_type(4)));
+            typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+            constexpr uint32_t Groups = NCols / 4u;
+
+            extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
+            const uint32_t chunks  = k / 8u; // 16-byte chunks per row of A / column of X
+            u32x4_t*       xs      = reinterpret_cast<u32x4_t*>(ldsRaw); // [NCols][chunks]
+            float*         partial = reinterpret_cast<float*>(ldsRaw + static_cast<size_t>(NCols) * k * 2u);
+            // partial[row quad of the workgroup][K slice][row in quad][column]
+
+            const uint32_t lane = threadIdx.x & 63u;
+            const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            {
+                const uint32_t perCol = chunks / 64u;
+                for(uint32_t j = wave; j < NCols * perCol; j += kQuadWaves)
+                {
+                    const uint32_t c   = j / perCol;
+                    const uint32_t pos = (j % perCol) * 64u + lane;
+                    rocwmma::lds::asyncCopy16(xs + c * chunks + (j % perCol) * 64u,
+                                              reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(c) * ldx)
+                                                  + (pos ^ ((c & 3u) << 2)));
+                }
+                rocwmma::lds::waitCopiesAndReads<0>();
+            }
+            __syncthreads();
+
+            const uint32_t r4     = lane & 3u; // row of the quad (A operand) = column of the group (X operand)
+            const uint32_t blk    = lane >> 2; // block of the instruction = K chunk within a step
+            const uint32_t slice  = wave % kQuadSlices;
+            const uint32_t qLane  = wave / kQuadSlices;
+            const uint32_t quads  = m / 4u;
+            const uint32_t q0     = blockIdx.x * quadsPerWg;
+            const uint32_t sliceChunks = chunks / kQuadSlices;
+            const uint32_t cBeg   = slice * sliceChunks;
+            const uint32_t steps  = sliceChunks / 16u; // a multiple of Unroll (checked by the host)
+
+            for(uint32_t ql = qLane; ql < quadsPerWg && q0 + ql < quads; ql += kQuadWaves / kQuadSlices)
+            {
+                const uint32_t  row  = (q0 + ql) * 4u + r4;
+                const u32x4_t*  aRow = reinterpret_cast<const u32x4_t*>(a + static_cast<size_t>(row) * lda) + cBeg + blk;
+                float4_t        acc[Groups];
+#pragma unroll
+                for(uint32_t g = 0; g < Groups; ++g)
+                    acc[g] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                for(uint32_t s0 = 0; s0 < steps; s0 += Unroll)
+                {
+                    u32x4_t av[Unroll];
+#pragma unroll
+                    for(uint32_t u = 0; u < Unroll; ++u)
+                        av[u] = __builtin_nontemporal_load(aRow + 16u * (s0 + u));
+#pragma unroll
+                    for(uint32_t u = 0; u < Unroll; ++u)
+                    {
+                        const uint32_t ch  = cBeg + blk + 16u * (s0 + u);
+                        const u32x2_t  alo = {av[u][0], av[u][1]}, ahi = {av[u][2], av[u][3]};
+#pragma unroll
+                        for(uint32_t g = 0; g < Groups; ++g)
+                        {
+                            const u32x4_t xv  = xs[(g * 4u + r4) * chunks + (ch ^ (r4 << 2))];
+                            const u32x2_t xlo = {xv[0], xv[1]}, xhi = {xv[2], xv[3]};
+                            // D[i][j] += sum_k X[column i][k] * A[row j][k]
+                            acc[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, xlo),
+                                                                        __builtin_bit_cast(half4_t, alo), acc[g], 0, 0, 0);
+                            acc[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, xhi),
+                                                                        __builtin_bit_cast(half4_t, ahi), acc[g], 0, 0, 0);
+                        }
+                    }
+                }
+                // lane (b, j) holds D[0..3][j] of block b: sum the 16 blocks
+#pragma unroll
+                for(uint32_t g = 0; g < Groups; ++g)
+#pragma unroll
+                    for(uint32_t i = 0; i < 4u; ++i)
+                    {
+                        float v = acc[g][i];
+                        v += __shfl_xor(v, 4, 64);
+                        v += __shfl_xor(v, 8, 64);
+                        v += __shfl_xor(v, 16, 64);
+                        v += __shfl_xor(v, 32, 64);
+                        acc[g][i] = v;
+                    }
+                if(blk == 0u)
+                {
+#pragma unroll
+                    for(uint32_t g = 0; g < Groups; ++g)
+#pragma unroll
+                        for(uint32_t i = 0; i < 4u; ++i)
+                            partial[((ql * kQuadSlices + slice) * 4u + r4) * NCols + g * 4u + i] = acc[g][i];
+                }
+            }
+            __syncthreads();
+            const uint32_t quadsHere = q0 < quads ? (quads - q0 < quadsPerWg ? quads - q0 : quadsPerWg) : 0u;
+            const uint32_t rowsHere  = quadsHere * 4u;
+            for(uint32_t i = threadIdx.x; i < rowsHere * NCols; i += kQuadWaves * 64u)
+            {
+                const uint32_t r = i % rowsHere, c = i / rowsHere; // consecutive threads: consecutive rows of a column of Y
+                const float*   p = partial + ((r / 4u) * kQuadSlices * 4u + (r & 3u)) * NCols + c;
+                float          sum = p[0];
+#pragma unroll
+                for(uint32_t h = 1; h < kQuadSlices; ++h)
+                    sum += p[h * 4u * NCols];
+                float*      dst = y + static_cast<size_t>(c) * ldy + q0 * 4u + r;
+                const float v   = alpha * sum;
+                *dst            = (beta != 0.0f) ? v + beta * *dst : v;
+            }
+        }
+
         struct GemvArgs
         {
             uint32_t    m, k;
@@ -246,6 +385,40 @@ namespace rocwmma_amd
             return launchStatus();
         }
 
+        template <uint32_t NCols, uint32_t Unroll>
+        int launchQuadU(GemvArgs const& g, uint32_t workgroups, uint32_t quadsPerWg, uint32_t ldsBytes, hipStream_t stream)
+        {
+            auto kernel = gemvQuadKernel<NCols, Unroll>;
+            if(ldsBytes > 65536u
+               && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(ldsBytes))
+                      != hipSuccess)
+                return ROCWMMA_AMD_LAUNCH_FAILED;
+            hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(kQuadWaves * 64u), ldsBytes, stream, g.m, g.k,
+                               static_cast<const _Float16*>(g.a), g.lda, static_cast<const _Float16*>(g.x), g.ldx, g.y, g.ldy,
+                               g.alpha, g.beta, quadsPerWg);
+            return launchStatus();
+        }
+
+        template <uint32_t NCols>
+        int launchQuad(GemvArgs const& g, hipStream_t stream)
+        {
+            // whole row quads; whole 1 KiB copies per column of X; whole steps of 16 chunks per K slice
+            if(g.m % 4u != 0u || g.k % (8u * 16u * kQuadSlices * 2u) != 0u)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            const uint32_t quads      = g.m / 4u;
+            const uint32_t cus        = computeUnits();
+            const uint32_t workgroups = quads < cus ? quads : cus;
+            const uint32_t quadsPerWg = (quads + workgroups - 1u) / workgroups;
+            const uint32_t ldsBytes   = NCols * g.k * 2u + quadsPerWg * kQuadSlices * 4u * NCols * 4u;
+            if(ldsBytes > 160u * 1024u)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            const uint32_t steps = g.k / (8u * 16u * kQuadSlices);
+            if(steps % 8u == 0u)
+                return launchQuadU<NCols, 8>(g, workgroups, quadsPerWg, ldsBytes, stream);
+            return launchQuadU<NCols, 2>(g, workgroups, quadsPerWg, ldsBytes, stream);
+        }
+
         constexpr uint32_t kStagedLdsLimit = 131072u; // X must leave room in the 160 KiB LDS
     } // namespace
 
@@ -255,6 +428,14 @@ namespace rocwmma_amd
         const GemvArgs g{m, k, a, lda, x, ldx, y, ldy, alpha, beta};
         const uint32_t cus    = computeUnits();
         const bool     staged = ncols * k * 2u <= kStagedLdsLimit;
+        // 8 columns: the quad kernel where the shape allows it (with 4 columns it only ties with
+        // the staged kernel)
+        if(ncols == 8u)
+        {
+            const int rc = launchQuad<8>(g, stream);
+            if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                return rc;
+        }
         switch(ncols)
         {
         case 1:
