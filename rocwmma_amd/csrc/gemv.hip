@@ -414,6 +414,8 @@ namespace rocwmma_amd
             if(ldsBytes > 160u * 1024u)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             const uint32_t steps = g.k / (8u * 16u * kQuadSlices);
+            if(steps % 16u == 0u)
+                return launchQuadU<NCols, 16>(g, workgroups, quadsPerWg, ldsBytes, stream);
             if(steps % 8u == 0u)
                 return launchQuadU<NCols, 8>(g, workgroups, quadsPerWg, ldsBytes, stream);
             return launchQuadU<NCols, 2>(g, workgroups, quadsPerWg, ldsBytes, stream);
@@ -428,11 +430,10 @@ namespace rocwmma_amd
         const GemvArgs g{m, k, a, lda, x, ldx, y, ldy, alpha, beta};
         const uint32_t cus    = computeUnits();
         const bool     staged = ncols * k * 2u <= kStagedLdsLimit;
-        // 8 columns: the quad kernel where the shape allows it (with 4 columns it only ties with
-        // the staged kernel)
-        if(ncols == 8u)
+        // 4 and 8 columns: the quad kernel where the shape allows it
+        if(ncols == 4u || ncols == 8u)
         {
-            const int rc = launchQuad<8>(g, stream);
+            const int rc = ncols == 4u ? launchQuad<4>(g, stream) : launchQuad<8>(g, stream);
             if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
                 return rc;
         }

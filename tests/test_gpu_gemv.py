@@ -39,7 +39,7 @@ def test_config4_full_shapes(m, k, ncols, beta):
                                        # m a multiple of 16 and k a multiple of 4096
                                        (48, 4096, 4), (16, 8192, 8), (2064, 4096, 8), (80, 8192, 4),
                                        # 8 columns, m % 4 == 0, k % 1024 == 0 but not % 4096; one row quad
-                                       (100, 3072, 8), (4, 1024, 8), (1028, 2048, 8)])
+                                       (100, 3072, 8), (4, 1024, 8), (1028, 2048, 8), (100, 3072, 4), (12, 1024, 4)])
 def test_ragged_shapes(m, k, ncols):
     run(m, k, ncols, 2.1, 2.1, 99)
 
