@@ -62,6 +62,14 @@ namespace rocwmma
                 src, (LdsPtr)ldsBase, 16, static_cast<int>(laneOffset), static_cast<int>(waveOffset), 0, 0);
         }
 
+        // The buffer-addressed copy marked non-temporal (data that is read once).
+        ROCWMMA_DEVICE ROCWMMA_INLINE void
+            asyncCopy16Streaming(void* ldsBase, BufferRsrc src, uint32_t laneOffset, uint32_t waveOffset)
+        {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                src, (LdsPtr)ldsBase, 16, static_cast<int>(laneOffset), static_cast<int>(waveOffset), 0, 2 /* nt */);
+        }
+
         // s_waitcnt with "at most MaxLoads vector-memory operations still in flight" and all of
         // this wave's LDS reads returned.  Direct-to-LDS copies complete in issue order, so
         // leaving the newest MaxLoads outstanding means every older copy has landed.

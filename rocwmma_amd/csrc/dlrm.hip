@@ -104,7 +104,7 @@ namespace rocwmma_amd
                         srcOff = row * rowBytes + ((((pos >> 1) ^ segmentSwizzle(row)) << 5) | ((pos & 1u) << 4));
                     else
                         srcOff = row * rowBytes + ((pos ^ chunkSwizzle(row)) << 4);
-                    lds::asyncCopy16(ldsTile + copy * 1024u, rsrc, srcOff, 0u);
+                    lds::asyncCopy16Streaming(ldsTile + copy * 1024u, rsrc, srcOff, 0u);
                 }
             }
         };
