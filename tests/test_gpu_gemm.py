@@ -181,6 +181,52 @@ def test_leading_dimensions_larger_than_extent():
         assert np.all(got[:, n:] == 777.0)
 
 
+@pytest.mark.parametrize("dtype_in,dtype_out", [(orc.F16, orc.F32), (orc.F16, orc.F16), (orc.I8, orc.I32)])
+def test_c_may_alias_d(dtype_in, dtype_out):
+    """In-place update (the same buffer as C and D), as the header allows: every element is read
+    before it is written, by the same lane (blocked kernel: C staged through LDS for 32-bit outputs,
+    through registers for 16-bit outputs)."""
+    import torch
+
+    m, n, k = 512, 768, 256
+    a = uniform_bits(81, dtype_in, m * k)
+    b = uniform_bits(82, dtype_in, k * n)
+    c = uniform_bits(83, dtype_out, m * n)
+    alpha, beta = (1.0, 1.0) if dtype_in == orc.I8 else (0.5, 1.5)
+    want = orc.gemm(dtype_in, dtype_out, RM, CM, RM, RM, m, n, k, a, b, c, alpha, beta)
+    for algo in (rw.GEMM_BLOCKED, rw.GEMM_WAVE_TILE):
+        cd = to_device(c.copy())
+        rw.gemm(dtype_in, dtype_out, RM, CM, RM, m, n, k, to_device(a), to_device(b), cd, cd, alpha, beta, algo=algo)
+        torch.cuda.synchronize()
+        check(dtype_in, dtype_out, to_host(cd, orc.storage_dtype(dtype_out)), want, tol_for(dtype_in))
+
+
+@pytest.mark.parametrize("la,lb", [(RM, CM), (CM, RM), (RM, RM), (CM, CM)])
+def test_padded_leading_dimensions_every_layout_many_tiles(la, lb):
+    """Padded lda / ldb / ldc / ldd with several macro tiles in both directions: the padding of D
+    must stay untouched, the window must match the oracle."""
+    import torch
+
+    m, n, k = 512, 768, 320
+    pad_a, pad_b, pad_c = 24, 40, 12
+    rng = np.random.default_rng(91)
+    a_rows, a_cols = (m, k) if la == RM else (k, m)
+    b_rows, b_cols = (k, n) if lb == RM else (n, k)
+    A = orc.encode(orc.F16, rng.uniform(-1, 1, (a_rows, a_cols + pad_a)).astype(np.float32))
+    B = orc.encode(orc.F16, rng.uniform(-1, 1, (b_rows, b_cols + pad_b)).astype(np.float32))
+    C = rng.uniform(-1, 1, (m, n + pad_c)).astype(np.float32)
+    want = orc.gemm(orc.F16, orc.F32, la, lb, RM, RM, m, n, k, np.ascontiguousarray(A[:, :a_cols]),
+                    np.ascontiguousarray(B[:, :b_cols]), np.ascontiguousarray(C[:, :n]), 1.0, -2.0)
+    for algo in (rw.GEMM_BLOCKED, rw.GEMM_WAVE_TILE):
+        d = torch.full((m, n + pad_c), 777.0, device="cuda")
+        rw.gemm(orc.F16, orc.F32, la, lb, RM, m, n, k, to_device(A), to_device(B), to_device(C), d, 1.0, -2.0,
+                lda=a_cols + pad_a, ldb=b_cols + pad_b, ldc=n + pad_c, ldd=n + pad_c, algo=algo)
+        torch.cuda.synchronize()
+        got = d.cpu().numpy()
+        check(orc.F16, orc.F32, np.ascontiguousarray(got[:, :n]).reshape(-1), want, 1e-3)
+        assert np.all(got[:, n:] == 777.0)
+
+
 @pytest.mark.parametrize("m,k", [(16, 1536), (32, 1536), (48, 1536), (80, 1536), (112, 1536), (128, 1536),
                                  (16, 1024), (32, 1024), (16, 2048), (32, 2048), (16, 4096), (32, 4096)])
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3, orc.E5M2])
