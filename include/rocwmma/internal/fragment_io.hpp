@@ -155,6 +155,7 @@ namespace rocwmma
         template <typename IO, typename DataT>
         struct FragmentMover
         {
+            static constexpr uint32_t Items = IO::Items; // work items of the whole fragment
             ROCWMMA_DEVICE static ROCWMMA_INLINE void load(DataT* x, const DataT* data, uint32_t ld)
             {
                 const uint32_t lane = threadIdx.x & (kWaveSize - 1u);

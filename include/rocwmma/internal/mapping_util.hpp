@@ -63,7 +63,8 @@ namespace rocwmma
             {
                 return make_coord2d(blockIdx.x, blockIdx.y);
             }
-            ROCWMMA_DEVICE static inline WorkgroupDimT workgroupDim()
+            // a constant expression when the thread-block shape is given at compile time
+            ROCWMMA_DEVICE constexpr static inline WorkgroupDimT workgroupDim()
             {
                 if constexpr(TBlockX > 0u && TBlockY > 0u)
                     return waveCount(make_coord2d(TBlockX, TBlockY));
@@ -114,6 +115,16 @@ namespace rocwmma
         template <>
         struct DataSpace<void>;
     } // namespace detail
+
+    // Names existing kernels use for the (row, col) -> element offset map of a row- or column-major
+    // array (reference: library/include/rocwmma/internal/layout/layout.hpp, namespace DataLayout).
+    namespace DataLayout
+    {
+        template <typename DataOrientation>
+        using Array1d = detail::DataSpace<DataOrientation>;
+        using RowMajor = Array1d<row_major>;
+        using ColMajor = Array1d<col_major>;
+    } // namespace DataLayout
 
     template <uint32_t BlockHeight, uint32_t BlockWidth, typename DataT, typename DataLayout>
     struct MappingUtil

@@ -22,12 +22,14 @@
 #include "internal/config.hpp"
 #include "internal/constants.hpp"
 #include "internal/coord.hpp"
+#include "internal/flow_control.hpp"
 #include "internal/fragment_io.hpp"
 #include "internal/fragment_map.hpp"
 #include "internal/mapping_util.hpp"
 #include "internal/mfma_gfx950.hpp"
 #include "internal/type_traits.hpp"
 #include "internal/types.hpp"
+#include "internal/utils.hpp"
 
 namespace rocwmma
 {

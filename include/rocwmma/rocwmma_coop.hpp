@@ -41,6 +41,38 @@ namespace rocwmma
         }
     } // namespace detail
 
+    // Cooperative I/O description of a fragment shared by WaveCount waves (reference:
+    // library/include/rocwmma/internal/accessors.hpp:55-59).  IOTraits::IOCount is the number of
+    // items one wave moves (at least 1); kernels use it only to derive the deprecated split
+    // counts, which the loads and stores below ignore.
+    template <typename FragT, uint32_t WaveCount>
+    struct GetCoopIOConfig;
+
+    template <uint32_t WaveCount,
+              typename MatrixT,
+              uint32_t BlockM,
+              uint32_t BlockN,
+              uint32_t BlockK,
+              typename DataT,
+              typename DataLayoutT>
+    struct GetCoopIOConfig<fragment<MatrixT, BlockM, BlockN, BlockK, DataT, DataLayoutT>, WaveCount>
+    {
+        struct type
+        {
+            using Mover = typename detail::CoopMover<MatrixT, BlockM, BlockN, BlockK, DataT, DataLayoutT>::type;
+            struct IOTraits
+            {
+                enum : uint32_t
+                {
+                    IOCount = (Mover::Items + WaveCount - 1u) / WaveCount
+                };
+            };
+        };
+    };
+
+    template <typename FragT, uint32_t WaveCount = 1u>
+    using GetCoopIOConfig_t = typename GetCoopIOConfig<std::decay_t<FragT>, WaveCount>::type;
+
     // ---- loads -----------------------------------------------------------------------------
     template <typename MatrixT, uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT, typename DataLayoutT>
     ROCWMMA_DEVICE ROCWMMA_INLINE void

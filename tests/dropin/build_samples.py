@@ -1,4 +1,5 @@
-"""Builds the reference's sample programs against this repository's headers (drop-in check).
+"""Builds the reference's sample programs and its cooperative GEMM test kernel against this
+repository's headers (drop-in check).
 
 The sample sources are compiled where they lie in the reference checkout (nothing is copied);
 the executables go to tests/dropin/_bin/, which is git-ignored and travels to the GPU box with
@@ -13,6 +14,14 @@ validates its own GPU result against its own CPU code and prints PASSED or FAILE
                               perf_hgemm at 1024^3 instead of 7168^3, whose CPU check takes minutes).
 
 Validation needs the samples' debug path (no -DNDEBUG).
+
+Kernel matrix: the reference's cooperative LDS double-buffered GEMM test kernel
+(test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp) is instantiated by
+tests/dropin/coop_gemm_matrix.cpp (host side only, written here) over the case list that
+coop_gemm_cases() enumerates: the axes of the reference's own test matrix
+(test/gemm/gemm_common_test_params.hpp:44-330, test/gemm/gemm_PGR1_LB2_MP0_MB_CP/test/*):
+element types, block sizes, A/B/C layouts, LDS layout, cooperation level and LDS mapping, blocks
+per wave, thread-block shape.  tests/test_gpu_reference_kernel_matrix.py runs the executables.
 """
 import os
 import shutil
@@ -63,6 +72,56 @@ def _hipcc():
     return None
 
 
+REFERENCE_TESTS = "/root/reference/test"
+MATRIX_UNITS = 8  # translation units (and executables) the case list is dealt over
+
+# (input, output, compute) -> block sizes (BlockM = BlockN, BlockK) a matrix instruction exists for
+_MATRIX_TYPES = [
+    (("f16", "f32", "f32"), [(16, 16), (16, 32), (16, 64), (32, 8), (32, 16), (32, 32)]),
+    (("f16", "f16", "f32"), [(16, 32), (32, 16)]),
+    (("bf16", "f32", "f32"), [(16, 16), (16, 32), (32, 8), (32, 16)]),
+    (("bf16", "bf16", "f32"), [(16, 32), (32, 16)]),
+    (("f32", "f32", "f32"), [(16, 4), (16, 8), (32, 2), (32, 4)]),
+    (("i8", "i32", "i32"), [(16, 32), (16, 64), (32, 16), (32, 32)]),
+    (("f8", "f32", "f32"), [(16, 32), (16, 64), (16, 128), (32, 16), (32, 64)]),
+    (("bf8", "f32", "f32"), [(16, 32), (16, 128), (32, 16), (32, 64)]),
+]
+_CONFIGS = ["Block::LdsNT", "Block::LdsTN", "Block::LdsRF", "Wave::LdsNT", "Wave::LdsTN", "Wg::LdsNT", "Wg::LdsTN"]
+_BLOCKS = [(1, 1), (2, 2), (1, 2), (2, 1), (4, 2), (2, 4), (4, 4), (1, 4)]
+_TBLOCKS = [(128, 2), (64, 1), (64, 4), (256, 1), (128, 1), (64, 2)]
+
+
+def coop_gemm_cases():
+    """The CASE(...) lines, deterministic.  f16 -> f32 gets the full product of block sizes x A/B
+    layouts x LDS layouts x configs; the other types walk the same axes diagonally.  Blocks per wave,
+    thread-block shape and the C/D layout rotate with the case index.  Cases the kernel's own guard
+    rejects (register budget, LdsRF with more than one wave) are reported as skipped at run time."""
+    cases = []
+
+    def add(types, size, la, lb, lds, cfg):
+        i = len(cases)
+        # (32-wide blocks: at most 2 x 2 per wave, more exceeds the kernel's register budget; the
+        # index is skewed so that the cases dealt to one translation unit differ in blocks per wave)
+        nblocks = 4 if size[0] == 32 else len(_BLOCKS)
+        bx, by = _BLOCKS[(i + i // MATRIX_UNITS) % nblocks]
+        tx, ty = (64, 1) if cfg.endswith("LdsRF") and i % 2 == 0 else _TBLOCKS[(i // 3) % len(_TBLOCKS)]
+        lc = "RC"[(i // 2) % 2]
+        cases.append(f"CASE({size[0]}, {size[0]}, {size[1]}, {types[0]}, {types[1]}, {types[2]}, "
+                     f"{la}, {lb}, {lc}, {lds}, {cfg}, {bx}, {by}, {tx}, {ty});")
+
+    for types, sizes in _MATRIX_TYPES:
+        full = types == ("f16", "f32", "f32")
+        n = 0
+        for size in sizes:
+            for cfg in _CONFIGS:
+                for la, lb in (("R", "C"), ("C", "R"), ("R", "R"), ("C", "C")):
+                    for lds in ("R", "C"):
+                        n += 1
+                        if full or n % 8 == (len(cases) // 5) % 8:
+                            add(types, size, la, lb, lds, cfg)
+    return cases
+
+
 def available():
     return os.path.isdir(REFERENCE_SAMPLES) and _hipcc() is not None
 
@@ -96,8 +155,41 @@ def build(verbose=False):
     return out
 
 
+def build_coop_gemm_matrix(verbose=False):
+    """Compiles the kernel-matrix executables (in parallel); returns their paths."""
+    if not (os.path.isdir(os.path.join(REFERENCE_TESTS, "gemm")) and _hipcc() is not None):
+        return []
+    os.makedirs(BIN, exist_ok=True)
+    cases = coop_gemm_cases()
+    procs = []
+    for unit in range(MATRIX_UNITS):
+        lst = os.path.join(BIN, f"coop_gemm_cases_{unit}.inc")
+        with open(lst, "w") as f:
+            f.write("\n".join(cases[unit::MATRIX_UNITS]) + "\n")
+        exe = os.path.join(BIN, f"coop_gemm_matrix_{unit}")
+        # the reference's test kernels are gated on the architecture ids they know: the device pass
+        # reports gfx942's
+        cmd = [_hipcc(), "--offload-arch=gfx950", "-std=c++17", "-O2", "-DROCWMMA_AMD_REPORT_ARCH_ID=0x942",
+               f'-DCASE_LIST="{lst}"',
+               "-I" + os.path.join(ROOT, "include"), "-I" + REFERENCE_TESTS, "-I" + os.path.join(REFERENCE_TESTS, "gemm"),
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+               os.path.join(HERE, "coop_gemm_matrix.cpp"), "-o", exe]
+        procs.append((exe, lst, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    out = []
+    for exe, lst, proc in procs:
+        log, _ = proc.communicate()
+        if proc.returncode != 0:
+            raise RuntimeError(f"{os.path.basename(exe)}: hipcc failed\n{log[-3000:]}")
+        os.remove(lst)
+        if verbose:
+            print(exe)
+        out.append(exe)
+    return out
+
+
 if __name__ == "__main__":
     if not available():
         print("reference checkout or hipcc not present: nothing built")
         sys.exit(0)
     build(verbose=True)
+    build_coop_gemm_matrix(verbose=True)

@@ -1,0 +1,44 @@
+"""Drop-in check on the GPU: the reference's cooperative, LDS double-buffered multi-block GEMM test
+kernel (test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp in the reference tree),
+compiled unchanged against this repository's headers, over a matrix of element types, block sizes,
+A/B/C layouts, LDS layouts, cooperation levels (block / wave / workgroup), LDS mappings
+(NT / TN / register file), blocks per wave and thread-block shapes.
+
+Operands are small integers, so every case must match a plain CPU loop bit for bit whatever the
+accumulation order.  tests/dropin/build_samples.py enumerates the cases and builds the executables
+on the development machine (where the reference checkout is); they travel with the tree.  Where
+they are absent the tests are skipped."""
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "dropin"))
+import build_samples  # noqa: E402
+
+BIN = os.path.join(HERE, "dropin", "_bin")
+
+
+@pytest.mark.parametrize("unit", range(build_samples.MATRIX_UNITS))
+def test_reference_cooperative_gemm_kernel_matrix(unit):
+    exe = os.path.join(BIN, f"coop_gemm_matrix_{unit}")
+    if not os.path.exists(exe):
+        pytest.skip("kernel-matrix executables not built on this machine (tests/dropin/build_samples.py)")
+    expected = len(build_samples.coop_gemm_cases()[unit::build_samples.MATRIX_UNITS])
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+    tail = res.stdout[-2000:]
+    failed = [line for line in res.stdout.splitlines() if line.startswith("FAILED")]
+    assert not failed, "\n".join(failed[:10])
+    assert res.returncode == 0, tail
+    summary = re.search(r"SUMMARY: (\d+) passed, (\d+) failed, (\d+) skipped", res.stdout)
+    assert summary, tail
+    passed, nfailed, skipped = map(int, summary.groups())
+    assert nfailed == 0 and passed + skipped == expected, tail
+    # the kernel's own guard rejects some cases (register budget; the register-file LDS mapping
+    # needs a single wave): most of the matrix must run
+    assert passed >= 0.6 * expected, tail

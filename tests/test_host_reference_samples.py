@@ -91,6 +91,28 @@ template __global__ void gemm_PGR0_LB0_MP0_SB_NC<32, 32, 16, float16_t, float32_
 template __global__ void gemm_PGR0_LB0_MP0_SB_NC<16, 16, 64, int8_t, int32_t, int32_t, col_major, row_major, row_major, row_major, 64, 4, 64, 0x942>(uint32_t, uint32_t, uint32_t, int8_t const*, int8_t const*, int32_t const*, int32_t*, uint32_t, uint32_t, uint32_t, uint32_t, int32_t, int32_t);
 }
 """,
+    "gemm_cooperative_lds_test_kernel": """
+#include <hip/hip_runtime.h>
+#include <iostream>
+#include <rocwmma/rocwmma.hpp>
+#include <rocwmma/rocwmma_coop.hpp>
+#include <rocwmma/rocwmma_transforms.hpp>
+#include "gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp"
+namespace rocwmma {
+template __global__ void gemm_PGR1_LB2_MP0_MB_CP<32, 32, 16, float16_t, float32_t, float32_t, row_major, col_major, row_major, row_major, col_major, CooperativeGemm::WorkgroupLevel::LdsNT, 2, 2, 128, 2, 64, 0x942>(uint32_t, uint32_t, uint32_t, float16_t const*, float16_t const*, float32_t const*, float32_t*, uint32_t, uint32_t, uint32_t, uint32_t, float32_t, float32_t);
+template __global__ void gemm_PGR1_LB2_MP0_MB_CP<16, 16, 64, int8_t, int32_t, int32_t, col_major, row_major, col_major, col_major, row_major, CooperativeGemm::BlockLevel::LdsTN, 2, 4, 64, 4, 64, 0x942>(uint32_t, uint32_t, uint32_t, int8_t const*, int8_t const*, int32_t const*, int32_t*, uint32_t, uint32_t, uint32_t, uint32_t, int32_t, int32_t);
+template __global__ void gemm_PGR1_LB2_MP0_MB_CP<16, 16, 128, float8_t, float32_t, float32_t, row_major, col_major, row_major, row_major, row_major, CooperativeGemm::WaveLevel::LdsNT, 2, 2, 128, 2, 64, 0x942>(uint32_t, uint32_t, uint32_t, float8_t const*, float8_t const*, float32_t const*, float32_t*, uint32_t, uint32_t, uint32_t, uint32_t, float32_t, float32_t);
+// pieces of the library surface that kernel's helpers lean on
+static_assert(Waitcnt<3, 2>::encoded == (3 | (2 << 8) | (7 << 4)), "s_waitcnt encoding");
+static_assert(std::is_same<WaitVmcnt<5>, Waitcnt<5, 0>>::value && std::is_same<WaitLgkmcnt<1>, Waitcnt<0, 1>>::value, "");
+static_assert(std::is_same<DataLayout::Array1d<col_major>, GetDataLayout_t<fragment<matrix_b, 16, 16, 16, float16_t, col_major>>>::value, "");
+static_assert(DataLayout::RowMajor::fromMatrixCoord(make_coord2d(3u, 5u), 100u) == 305u && DataLayout::ColMajor::fromMatrixCoord(make_coord2d(3u, 5u), 100u) == 503u, "");
+static_assert(GetCoopIOConfig_t<fragment<matrix_a, 128, 16, 16, float16_t, row_major>, 4>::IOTraits::IOCount * 4u == GetCoopIOConfig_t<fragment<matrix_a, 128, 16, 16, float16_t, row_major>>::IOTraits::IOCount, "");
+static_assert(detail::WaveSpace<128, 2>::workgroupDim() == make_coord2d(2u, 2u), "compile-time workgroup shape");
+constexpr bool sameText(const char* a, const char* b) { return *a == *b && (*a == 0 || sameText(a + 1, b + 1)); }
+static_assert(sameText(dataTypeToString<float16_t>(), "f16") && sameText(dataTypeToString<bfloat8_t>(), "bf8") && sameText(dataTypeToString<row_major>(), "T") && sameText(dataTypeToString<col_major>(), "N"), "");
+}
+""",
 }
 
 
