@@ -58,6 +58,19 @@ namespace rocwmma
             return (blockM % 32u == 0u && blockN % 32u == 0u) ? 32u : 16u;
         }
 
+        // Blocks with an edge of 8 have no matrix instruction; they exist for load / store / fill
+        // only (the reference's unit tests move 32..256 x 8 blocks, test/unit/unit_test_params.hpp:
+        // 104-141).  Inputs: the 64 lanes form 8 rows x 8 lane groups along K.  Accumulators:
+        // 32-row x 8-column tiles, one 4-column run per lane.
+        constexpr uint32_t inputTileDim(uint32_t blockM, uint32_t blockN, uint32_t blockDim)
+        {
+            return blockDim % 16u == 0u ? mmaTileDim(blockM, blockN) : 8u;
+        }
+        constexpr uint32_t accTileRows(uint32_t blockM, uint32_t blockN)
+        {
+            return blockN % 16u == 0u ? mmaTileDim(blockM, blockN) : 32u;
+        }
+
         // Largest per-lane K run (elements) for which an MFMA exists, given the class.
         constexpr uint32_t maxKPack(PackClass c)
         {
@@ -93,8 +106,8 @@ namespace rocwmma
         template <uint32_t BlockDim, uint32_t BlockK, uint32_t Tile, PackClass Class>
         struct InputMap
         {
-            static_assert(Tile == 16u || Tile == 32u, "MFMA tile edge is 16 or 32");
-            static_assert(BlockDim % Tile == 0u, "block dimension must be a multiple of the MFMA tile");
+            static_assert(Tile == 8u || Tile == 16u || Tile == 32u, "tile edge is 16 or 32 (8: load / store only)");
+            static_assert(BlockDim % Tile == 0u, "block dimension must be a multiple of the tile edge");
 
             static constexpr uint32_t tile    = Tile;
             static constexpr uint32_t groups  = kWaveSize / Tile;
@@ -142,18 +155,21 @@ namespace rocwmma
             }
         };
 
-        // Geometry of an accumulator fragment.
+        // Geometry of an accumulator fragment.  Tile = rows of a tile; a tile is Tile columns wide,
+        // or 8 columns for blocks whose width is not a multiple of 16 (load / store only).
         template <uint32_t BlockM, uint32_t BlockN, uint32_t Tile>
         struct AccMap
         {
             static_assert(Tile == 16u || Tile == 32u, "MFMA tile edge is 16 or 32");
-            static_assert(BlockM % Tile == 0u && BlockN % Tile == 0u,
-                          "accumulator block must be a multiple of the MFMA tile");
+            static constexpr uint32_t tile  = Tile;
+            static constexpr uint32_t tileN = BlockN % 16u == 0u ? Tile : 8u;
+            static_assert(tileN == Tile || Tile == 32u, "8-column tiles are 32 rows high");
+            static_assert(BlockM % Tile == 0u && BlockN % tileN == 0u,
+                          "accumulator block must be a multiple of the MFMA tile (or 32 x 8 for load / store)");
 
-            static constexpr uint32_t tile     = Tile;
             static constexpr uint32_t nbi      = BlockM / Tile;
-            static constexpr uint32_t nbj      = BlockN / Tile;
-            static constexpr uint32_t perBlock = Tile * Tile / kWaveSize; // 4 or 16
+            static constexpr uint32_t nbj      = BlockN / tileN;
+            static constexpr uint32_t perBlock = Tile * tileN / kWaveSize; // 4 or 16
             static constexpr uint32_t runs     = perBlock / 4u; // 4-column runs per block per lane
             static constexpr uint32_t nruns    = nbi * nbj * runs;
             static constexpr uint32_t size     = nbi * nbj * perBlock;
@@ -169,7 +185,7 @@ namespace rocwmma
             }
             static constexpr uint32_t runCol(uint32_t r, uint32_t lane)
             {
-                return ((r / runs) % nbj) * Tile + (Tile == 16u ? 0u : 8u * (r % runs))
+                return ((r / runs) % nbj) * tileN + (Tile == 16u ? 0u : 8u * (r % runs))
                        + (lane / Tile) * 4u;
             }
             static constexpr uint32_t rowOf(uint32_t e, uint32_t lane)

@@ -127,7 +127,7 @@ namespace rocwmma
         template <uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT>
         struct FragConfig<matrix_a, BlockM, BlockN, BlockK, DataT>
         {
-            using Map = InputMap<BlockM, BlockK, mmaTileDim(BlockM, BlockN), packClassOf<DataT>()>;
+            using Map = InputMap<BlockM, BlockK, inputTileDim(BlockM, BlockN, BlockM), packClassOf<DataT>()>;
             // K runs along a row of A
             template <typename Layout>
             using IO = InputIO<Map, DataT, std::is_same<Layout, row_major>::value>;
@@ -135,7 +135,7 @@ namespace rocwmma
         template <uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT>
         struct FragConfig<matrix_b, BlockM, BlockN, BlockK, DataT>
         {
-            using Map = InputMap<BlockN, BlockK, mmaTileDim(BlockM, BlockN), packClassOf<DataT>()>;
+            using Map = InputMap<BlockN, BlockK, inputTileDim(BlockM, BlockN, BlockN), packClassOf<DataT>()>;
             // K runs along a column of B
             template <typename Layout>
             using IO = InputIO<Map, DataT, std::is_same<Layout, col_major>::value>;
@@ -143,7 +143,7 @@ namespace rocwmma
         template <uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT>
         struct FragConfig<accumulator, BlockM, BlockN, BlockK, DataT>
         {
-            using Map = AccMap<BlockM, BlockN, mmaTileDim(BlockM, BlockN)>;
+            using Map = AccMap<BlockM, BlockN, accTileRows(BlockM, BlockN)>;
             template <typename Layout>
             using IO = AccIO<Map, DataT, std::is_same<Layout, row_major>::value>;
         };
@@ -341,6 +341,8 @@ namespace rocwmma
         using MapAcc = typename detail::FragConfig<accumulator, BlockM, BlockN, BlockK, ComputeT>::Map;
         static_assert(sizeof(InputTA) == sizeof(InputTB) && MapA::kpack == MapB::kpack,
                       "A and B fragments must use the same K packing");
+        static_assert(MapA::tile == MapAcc::tile && MapB::tile == MapAcc::tile && MapAcc::tileN == MapAcc::tile,
+                      "blocks with an edge of 8 can be loaded, stored and filled but not multiplied");
         // The accumulator is kept transposed: the instruction's row operand is B, its column
         // operand is A (see fragment_map.hpp).
         using Op = detail::Mfma<detail::TypeInfo<InputTB>::cls,

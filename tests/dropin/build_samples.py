@@ -122,6 +122,47 @@ def coop_gemm_cases():
     return cases
 
 
+# (BlockM, BlockN) of the reference's unit tests (test/unit/unit_test_params.hpp:89-141)
+_UNIT_SIZES = ([(16, k) for k in (16, 32, 64, 128, 256)]
+               + [(b, k) for b in (32, 64, 128, 256) for k in (8, 16, 32, 64, 128, 256)])
+_UNIT_TYPES = ["f16", "f32", "i8", "bf16", "f64", "f8", "i32", "bf8"]
+_UNIT_TBLOCKS = [(64, 1), (64, 2), (128, 1), (64, 4), (128, 2), (256, 1)]
+
+
+def unit_kernel_cases():
+    """The UNIT(...) lines for tests/dropin/unit_kernels.cpp, deterministic: every kernel x block
+    size x layout, with element type and thread-block shape rotating; the map kernels (which copy
+    their block element by element in every lane) on small blocks only."""
+    cases = []
+
+    def add(kind, kernel, size, layout, p1, p2):
+        i = len(cases)
+        t = _UNIT_TYPES[(i + i // len(_UNIT_TYPES)) % len(_UNIT_TYPES)]
+        tx, ty = _UNIT_TBLOCKS[(i // 2 + i // 7) % len(_UNIT_TBLOCKS)]
+        cases.append(f"UNIT({kind}, {kernel}, {size[0]}, {size[1]}, {t}, {layout}, {tx}, {ty}, {p1}, {p2});")
+
+    for size in _UNIT_SIZES:
+        for layout in "RC":
+            for op in ("A", "B", "Acc"):
+                n = len(cases)
+                add("IDENT", "LoadStoreMatrixSync" + op, size, layout, 0, 0)
+                # sharing dimension 0 / 1, index of the row / column of waves that does the work
+                add("IDENT", "LoadStoreMatrixCoopSync" + op, size, layout, n % 2, (n // 2) % 3)
+                add("FILL", "fillFragment" + op, size, layout, 5 - n % 11, 0)
+                pad = ((4, 8), (3, 1), (4, 1), (3, 8))[n % 4]  # the reference's frame widths
+                add("LOADC", "loadContamination" + op, size, layout, *pad)
+                add("STOREC", "storeContamination" + op, size, layout, *pad)
+    for size in ((16, 16), (32, 8), (16, 64), (32, 32), (64, 16)):
+        for layout in "RC":
+            for kernel in ("MapBlockToMatrix", "MapWaveToMatrix", "MapMatrixToData", "MapThreadToMatrix"):
+                add("IDENT", kernel, size, layout, 0, 0)
+            add("OVR_BLOCK_M", "MapBlockToMatrixOverrideM", size, layout, 1, 0)
+            add("OVR_BLOCK_N", "MapBlockToMatrixOverrideN", size, layout, 1, 0)
+            add("OVR_ELEM_M", "MapMatrixToDataOverrideM", size, layout, size[0] // 2, 0)
+            add("OVR_ELEM_N", "MapMatrixToDataOverrideN", size, layout, size[1] // 2, 0)
+    return cases
+
+
 def available():
     return os.path.isdir(REFERENCE_SAMPLES) and _hipcc() is not None
 
@@ -155,25 +196,22 @@ def build(verbose=False):
     return out
 
 
-def build_coop_gemm_matrix(verbose=False):
-    """Compiles the kernel-matrix executables (in parallel); returns their paths."""
-    if not (os.path.isdir(os.path.join(REFERENCE_TESTS, "gemm")) and _hipcc() is not None):
-        return []
+def _build_case_units(source, stem, cases, extra_includes, verbose):
+    """Deals `cases` over MATRIX_UNITS translation units of `source` and compiles them in parallel."""
     os.makedirs(BIN, exist_ok=True)
-    cases = coop_gemm_cases()
     procs = []
     for unit in range(MATRIX_UNITS):
-        lst = os.path.join(BIN, f"coop_gemm_cases_{unit}.inc")
+        lst = os.path.join(BIN, f"{stem}_cases_{unit}.inc")
         with open(lst, "w") as f:
             f.write("\n".join(cases[unit::MATRIX_UNITS]) + "\n")
-        exe = os.path.join(BIN, f"coop_gemm_matrix_{unit}")
+        exe = os.path.join(BIN, f"{stem}_{unit}")
         # the reference's test kernels are gated on the architecture ids they know: the device pass
         # reports gfx942's
         cmd = [_hipcc(), "--offload-arch=gfx950", "-std=c++17", "-O2", "-DROCWMMA_AMD_REPORT_ARCH_ID=0x942",
-               f'-DCASE_LIST="{lst}"',
-               "-I" + os.path.join(ROOT, "include"), "-I" + REFERENCE_TESTS, "-I" + os.path.join(REFERENCE_TESTS, "gemm"),
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
-               os.path.join(HERE, "coop_gemm_matrix.cpp"), "-o", exe]
+               f'-DCASE_LIST="{lst}"', "-I" + os.path.join(ROOT, "include")]
+        cmd += ["-I" + d for d in extra_includes]
+        cmd += ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+                os.path.join(HERE, source), "-o", exe]
         procs.append((exe, lst, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     out = []
     for exe, lst, proc in procs:
@@ -187,9 +225,26 @@ def build_coop_gemm_matrix(verbose=False):
     return out
 
 
+def build_coop_gemm_matrix(verbose=False):
+    """Compiles the cooperative-GEMM kernel-matrix executables; returns their paths."""
+    if not (os.path.isdir(os.path.join(REFERENCE_TESTS, "gemm")) and _hipcc() is not None):
+        return []
+    return _build_case_units("coop_gemm_matrix.cpp", "coop_gemm_matrix", coop_gemm_cases(),
+                             [REFERENCE_TESTS, os.path.join(REFERENCE_TESTS, "gemm")], verbose)
+
+
+def build_unit_kernels(verbose=False):
+    """Compiles the unit-test-kernel executables; returns their paths."""
+    if not (os.path.isdir(os.path.join(REFERENCE_TESTS, "unit")) and _hipcc() is not None):
+        return []
+    return _build_case_units("unit_kernels.cpp", "unit_kernels", unit_kernel_cases(),
+                             [REFERENCE_TESTS, os.path.join(REFERENCE_TESTS, "unit")], verbose)
+
+
 if __name__ == "__main__":
     if not available():
         print("reference checkout or hipcc not present: nothing built")
         sys.exit(0)
     build(verbose=True)
     build_coop_gemm_matrix(verbose=True)
+    build_unit_kernels(verbose=True)

@@ -104,9 +104,19 @@ int main()
     checkAcc<48, 16, 16>("acc 48x16");
     checkAcc<32, 64, 32>("acc 32x64");
     checkAcc<128, 128, 32>("acc 128x128");
+    // blocks with an edge of 8: load / store only
+    checkInput<8, 32, 8, PackClass::Bits16>("f16 8x32 t8", 4);
+    checkInput<8, 256, 8, PackClass::Bits16>("f16 8x256 t8", 8);
+    checkInput<8, 64, 8, PackClass::Int8>("i8 8x64 t8", 8);
+    checkInput<8, 32, 8, PackClass::Fp8>("f8 8x32 t8", 4);
+    checkInput<8, 128, 8, PackClass::Other>("f64 8x128 t8", 1);
+    checkAcc<32, 8, 32>("acc 32x8");
+    checkAcc<256, 8, 32>("acc 256x8");
 
     CHECK(mmaTileDim(32, 32) == 32 && mmaTileDim(64, 32) == 32 && mmaTileDim(32, 16) == 16 && mmaTileDim(16, 16) == 16
-              && mmaTileDim(128, 1) == 16,
+              && mmaTileDim(128, 1) == 16 && inputTileDim(1, 8, 8) == 8 && inputTileDim(32, 32, 32) == 32
+              && inputTileDim(64, 1, 64) == 16 && accTileRows(64, 8) == 32 && accTileRows(64, 32) == 32
+              && accTileRows(16, 32) == 16,
           "tile choice");
     if(failures)
     {

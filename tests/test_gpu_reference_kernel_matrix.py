@@ -1,11 +1,19 @@
-"""Drop-in check on the GPU: the reference's cooperative, LDS double-buffered multi-block GEMM test
+"""Drop-in checks on the GPU, part 1: the reference's cooperative, LDS double-buffered multi-block GEMM test
 kernel (test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp in the reference tree),
 compiled unchanged against this repository's headers, over a matrix of element types, block sizes,
 A/B/C layouts, LDS layouts, cooperation levels (block / wave / workgroup), LDS mappings
 (NT / TN / register file), blocks per wave and thread-block shapes.
 
 Operands are small integers, so every case must match a plain CPU loop bit for bit whatever the
-accumulation order.  tests/dropin/build_samples.py enumerates the cases and builds the executables
+accumulation order.
+
+Part 2: the device kernels of the reference's unit tests that use only the public API
+(test/unit/*/device/*.hpp: load / store, cooperative load / store, fill, load and store contamination,
+MappingUtil coordinate maps and their overrides), over the reference's block sizes
+(16..256 x 8..256, test/unit/unit_test_params.hpp:89-141), both layouts, eight element types and six
+thread-block shapes; each must move exactly the elements its contract says (tests/dropin/unit_kernels.cpp).
+
+tests/dropin/build_samples.py enumerates the cases and builds the executables
 on the development machine (where the reference checkout is); they travel with the tree.  Where
 they are absent the tests are skipped."""
 import os
@@ -42,3 +50,22 @@ def test_reference_cooperative_gemm_kernel_matrix(unit):
     # the kernel's own guard rejects some cases (register budget; the register-file LDS mapping
     # needs a single wave): most of the matrix must run
     assert passed >= 0.6 * expected, tail
+
+
+@pytest.mark.parametrize("unit", range(build_samples.MATRIX_UNITS))
+def test_reference_unit_test_kernels(unit):
+    exe = os.path.join(BIN, f"unit_kernels_{unit}")
+    if not os.path.exists(exe):
+        pytest.skip("unit-kernel executables not built on this machine (tests/dropin/build_samples.py)")
+    expected = len(build_samples.unit_kernel_cases()[unit::build_samples.MATRIX_UNITS])
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+    tail = res.stdout[-2000:]
+    failed = [line for line in res.stdout.splitlines() if line.startswith("FAILED")]
+    assert not failed, "\n".join(failed[:10])
+    assert res.returncode == 0, tail
+    summary = re.search(r"SUMMARY: (\d+) passed, (\d+) failed, (\d+) skipped", res.stdout)
+    assert summary, tail
+    passed, nfailed, skipped = map(int, summary.groups())
+    assert nfailed == 0 and passed + skipped == expected, tail
+    # the kernels' own guard rejects blocks that exceed a wave's register budget (e.g. 256 x 256 f64)
+    assert passed >= 0.8 * expected, tail
