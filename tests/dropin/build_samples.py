@@ -16,7 +16,8 @@ validates its own GPU result against its own CPU code and prints PASSED or FAILE
 Validation needs the samples' debug path (no -DNDEBUG).
 
 Kernel matrix: the reference's cooperative LDS double-buffered GEMM test kernel
-(test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp) is instantiated by
+(test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp) and its two GEMM test kernels
+without LDS (test/gemm/gemm_PGR0_LB0_MP0_{MB,SB}_NC/device/kernel_device_func.hpp) are instantiated by
 tests/dropin/coop_gemm_matrix.cpp (host side only, written here) over the case list that
 coop_gemm_cases() enumerates: the axes of the reference's own test matrix
 (test/gemm/gemm_common_test_params.hpp:44-330, test/gemm/gemm_PGR1_LB2_MP0_MB_CP/test/*):
@@ -119,6 +120,21 @@ def coop_gemm_cases():
                         n += 1
                         if full or n % 8 == (len(cases) // 5) % 8:
                             add(types, size, la, lb, lds, cfg)
+
+    # the two kernels without LDS (test/gemm/gemm_PGR0_LB0_MP0_{MB,SB}_NC): every type, block size
+    # and A/B layout pair
+    for types, sizes in _MATRIX_TYPES:
+        for size in sizes:
+            for la, lb in (("R", "C"), ("C", "R"), ("R", "R"), ("C", "C")):
+                i = len(cases)
+                nblocks = 4 if size[0] == 32 else len(_BLOCKS)
+                bx, by = _BLOCKS[1 + (i + i // MATRIX_UNITS) % (nblocks - 1)]  # more than one block
+                tx, ty = _TBLOCKS[(i // 3) % len(_TBLOCKS)]
+                lc = "RC"[(i // 2) % 2]
+                head = f"{size[0]}, {size[0]}, {size[1]}, {types[0]}, {types[1]}, {types[2]}, {la}, {lb}, {lc}"
+                cases.append(f"CASE_MB({head}, {bx}, {by}, {tx}, {ty});")
+                tx, ty = _TBLOCKS[(i // 3 + 2) % len(_TBLOCKS)]
+                cases.append(f"CASE_SB({head}, {tx}, {ty});")
     return cases
 
 
@@ -196,19 +212,35 @@ def build(verbose=False):
     return out
 
 
-def _build_case_units(source, stem, cases, extra_includes, verbose):
-    """Deals `cases` over MATRIX_UNITS translation units of `source` and compiles them in parallel."""
+def coop_gemm_units():
+    """The GEMM cases as dealt to the executables: (value of GEMM_KERNEL, cases) per unit.  The
+    reference's three kernel headers share their include guards, so a unit holds one kernel."""
+    cases = coop_gemm_cases()
+    coop = [c for c in cases if c.startswith("CASE(")]
+    ncoop = MATRIX_UNITS - 2
+    return ([(0, coop[u::ncoop]) for u in range(ncoop)]
+            + [(1, [c for c in cases if c.startswith("CASE_MB(")]),
+               (2, [c for c in cases if c.startswith("CASE_SB(")])])
+
+
+def unit_kernel_units():
+    cases = unit_kernel_cases()
+    return [(0, cases[u::MATRIX_UNITS]) for u in range(MATRIX_UNITS)]
+
+
+def _build_case_units(source, stem, units, family_macro, extra_includes, verbose):
+    """Compiles `source` once per unit (its case list passed as CASE_LIST), in parallel."""
     os.makedirs(BIN, exist_ok=True)
     procs = []
-    for unit in range(MATRIX_UNITS):
+    for unit, (family, cases) in enumerate(units):
         lst = os.path.join(BIN, f"{stem}_cases_{unit}.inc")
         with open(lst, "w") as f:
-            f.write("\n".join(cases[unit::MATRIX_UNITS]) + "\n")
+            f.write("\n".join(cases) + "\n")
         exe = os.path.join(BIN, f"{stem}_{unit}")
         # the reference's test kernels are gated on the architecture ids they know: the device pass
         # reports gfx942's
         cmd = [_hipcc(), "--offload-arch=gfx950", "-std=c++17", "-O2", "-DROCWMMA_AMD_REPORT_ARCH_ID=0x942",
-               f'-DCASE_LIST="{lst}"', "-I" + os.path.join(ROOT, "include")]
+               f'-DCASE_LIST="{lst}"', f"-D{family_macro}={family}", "-I" + os.path.join(ROOT, "include")]
         cmd += ["-I" + d for d in extra_includes]
         cmd += ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
                 os.path.join(HERE, source), "-o", exe]
@@ -226,10 +258,10 @@ def _build_case_units(source, stem, cases, extra_includes, verbose):
 
 
 def build_coop_gemm_matrix(verbose=False):
-    """Compiles the cooperative-GEMM kernel-matrix executables; returns their paths."""
+    """Compiles the GEMM kernel-matrix executables; returns their paths."""
     if not (os.path.isdir(os.path.join(REFERENCE_TESTS, "gemm")) and _hipcc() is not None):
         return []
-    return _build_case_units("coop_gemm_matrix.cpp", "coop_gemm_matrix", coop_gemm_cases(),
+    return _build_case_units("coop_gemm_matrix.cpp", "coop_gemm_matrix", coop_gemm_units(), "GEMM_KERNEL",
                              [REFERENCE_TESTS, os.path.join(REFERENCE_TESTS, "gemm")], verbose)
 
 
@@ -237,7 +269,7 @@ def build_unit_kernels(verbose=False):
     """Compiles the unit-test-kernel executables; returns their paths."""
     if not (os.path.isdir(os.path.join(REFERENCE_TESTS, "unit")) and _hipcc() is not None):
         return []
-    return _build_case_units("unit_kernels.cpp", "unit_kernels", unit_kernel_cases(),
+    return _build_case_units("unit_kernels.cpp", "unit_kernels", unit_kernel_units(), "UNIT_FAMILY",
                              [REFERENCE_TESTS, os.path.join(REFERENCE_TESTS, "unit")], verbose)
 
 

@@ -1,7 +1,8 @@
-// Drop-in check: the reference's cooperative, LDS double-buffered multi-block GEMM test kernel
-// (reference: test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:70-283, with its
-// mapping / scheduling / driver helpers test/gemm/gemm_{config,global_mapping,local_mapping,
-// coop_schedule,driver}.hpp) is compiled unchanged against this repository's headers and run over
+// Drop-in check: the reference's three GEMM test kernels, the cooperative, LDS double-buffered
+// multi-block one (reference: test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:70-283,
+// with its mapping / scheduling / driver helpers test/gemm/gemm_{config,global_mapping,local_mapping,
+// coop_schedule,driver}.hpp) and the two without LDS (test/gemm/gemm_PGR0_LB0_MP0_{MB,SB}_NC/device/
+// kernel_device_func.hpp), are compiled unchanged against this repository's headers and run over
 // a matrix of block sizes, element types, operand layouts, LDS layouts, cooperation levels,
 // blocks per wave and thread-block shapes.
 //
@@ -27,7 +28,18 @@
 #include <rocwmma/rocwmma_coop.hpp>
 #include <rocwmma/rocwmma_transforms.hpp>
 
+// The reference's three kernel headers share their include guards, so a translation unit holds one
+// of them: GEMM_KERNEL = 0 cooperative, 1 multi-block without LDS, 2 single-block without LDS.
+#ifndef GEMM_KERNEL
+#define GEMM_KERNEL 0
+#endif
+#if GEMM_KERNEL == 0
 #include "gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp"
+#elif GEMM_KERNEL == 1
+#include "gemm_PGR0_LB0_MP0_MB_NC/device/kernel_device_func.hpp"
+#else
+#include "gemm_PGR0_LB0_MP0_SB_NC/device/kernel_device_func.hpp"
+#endif
 
 #ifndef CASE_LIST
 #error "compile with -DCASE_LIST=\"file\" naming the list of CASE(...) lines (see tests/dropin/build_samples.py)"
@@ -91,40 +103,30 @@ namespace
         }                                                                                \
     } while(0)
 
-    template <uint32_t BlockM,
-              uint32_t BlockN,
-              uint32_t BlockK,
-              typename InputT,
-              typename OutputT,
-              typename ComputeT,
-              typename LayoutA,
-              typename LayoutB,
-              typename LayoutC,
-              typename LayoutLds,
-              typename GemmConfig,
-              uint32_t BlocksX,
-              uint32_t BlocksY,
-              uint32_t TBlockX,
-              uint32_t TBlockY>
-    void runCase(const char* name)
+    // Fills, launches, checks.  The three kernels share the argument list and the grid rule; they
+    // differ in the macro tile a workgroup covers and in their LDS need.
+    template <typename InputT, typename OutputT, typename ComputeT, typename LayoutA, typename LayoutB, typename LayoutC>
+    void runGemm(const char* name,
+                 void (*kernel)(uint32_t, uint32_t, uint32_t, InputT const*, InputT const*, OutputT const*, OutputT*,
+                                uint32_t, uint32_t, uint32_t, uint32_t, ComputeT, ComputeT),
+                 uint32_t macroM,
+                 uint32_t macroN,
+                 uint32_t blockK,
+                 uint32_t ldsBytes,
+                 uint32_t tx,
+                 uint32_t ty,
+                 bool     enabled)
     {
-        using Guard = gemm_PGR1_LB2_MP0_MB_CP_guard<BlockM, BlockN, BlockK, InputT, OutputT, ComputeT, LayoutA, LayoutB,
-                                                    LayoutC, LayoutC, LayoutLds, GemmConfig, BlocksX, BlocksY, TBlockX,
-                                                    TBlockY, 64u, kArch>;
-        // (enableBuild() also asks whether the *current compilation pass* targets that architecture,
-        // which the host pass never does; enableRun() is what the reference's harness asks)
-        if(!Guard::enableRun())
+        if(!enabled)
         {
             std::printf("SKIPPED %s (disabled by the kernel's own guard)\n", name);
             ++gSkipped;
             return;
         }
-        constexpr uint32_t macroM = BlockM * BlocksX * (TBlockX / 64u);
-        constexpr uint32_t macroN = BlockN * BlocksY * TBlockY;
-        const uint32_t     m = 2u * macroM, n = 3u * macroN, k = 5u * BlockK;
-        const uint32_t     lda = naturalLd<LayoutA>(m, k), ldb = naturalLd<LayoutB>(k, n);
-        const uint32_t     ldc = naturalLd<LayoutC>(m, n), ldd = ldc;
-        const int          alpha = 2, beta = 3;
+        const uint32_t m = 2u * macroM, n = 3u * macroN, k = 5u * blockK;
+        const uint32_t lda = naturalLd<LayoutA>(m, k), ldb = naturalLd<LayoutB>(k, n);
+        const uint32_t ldc = naturalLd<LayoutC>(m, n), ldd = ldc;
+        const int      alpha = 2, beta = 3;
 
         std::vector<InputT>  a(static_cast<size_t>(m) * k), b(static_cast<size_t>(k) * n);
         std::vector<OutputT> c(static_cast<size_t>(m) * n), d(static_cast<size_t>(m) * n), want(c.size());
@@ -170,11 +172,7 @@ namespace
         HIP_OK(hipMemcpy(dC, c.data(), c.size() * sizeof(OutputT), hipMemcpyHostToDevice));
         HIP_OK(hipMemset(dD, 0x7f, d.size() * sizeof(OutputT))); // a value no case produces
 
-        auto           kernel   = gemm_PGR1_LB2_MP0_MB_CP<BlockM, BlockN, BlockK, InputT, OutputT, ComputeT, LayoutA,
-                                              LayoutB, LayoutC, LayoutC, LayoutLds, GemmConfig, BlocksX, BlocksY,
-                                              TBlockX, TBlockY, 64u, kArch>;
-        const uint32_t ldsBytes = 2u * sizeof(InputT) * (macroM + macroN) * BlockK;
-        const dim3     grid((m + macroM - 1u) / macroM, (n + macroN - 1u) / macroN), block(TBlockX, TBlockY);
+        const dim3 grid((m + macroM - 1u) / macroM, (n + macroN - 1u) / macroN), block(tx, ty);
         hipLaunchKernelGGL(kernel, grid, block, ldsBytes, 0, m, n, k, dA, dB, dC, dD, lda, ldb, ldc, ldd,
                            static_cast<ComputeT>(alpha), static_cast<ComputeT>(beta));
         HIP_OK(hipGetLastError());
@@ -207,9 +205,11 @@ namespace
         std::fflush(stdout);
     }
 
+#if GEMM_KERNEL == 0
     namespace Block = CooperativeGemm::BlockLevel;
     namespace Wave  = CooperativeGemm::WaveLevel;
     namespace Wg    = CooperativeGemm::WorkgroupLevel;
+#endif
     using R         = row_major;
     using C         = col_major;
     using f16       = float16_t;
@@ -220,9 +220,39 @@ namespace
     using i8        = int8_t;
     using i32       = int32_t;
 
-#define CASE(BM, BN, BK, IN, OUT, COMP, LA, LB, LC, LLDS, CFG, BX, BY, TX, TY) \
-    runCase<BM, BN, BK, IN, OUT, COMP, LA, LB, LC, LLDS, CFG, BX, BY, TX, TY>( \
-        #BM "x" #BN "x" #BK " " #IN "->" #OUT " A:" #LA " B:" #LB " C:" #LC " lds:" #LLDS " " #CFG " " #BX "x" #BY " tb(" #TX "," #TY ")")
+// The guards' enableBuild() also asks whether the *current compilation pass* targets that
+// architecture, which the host pass never does; enableRun() is what the reference's harness asks.
+// Grid, block and LDS size as in the reference's harness (test/gemm/gemm_PGR1_LB2_MP0_MB_CP/detail/
+// kernel_impl.hpp:134-194 and its two siblings).
+
+// cooperative, LDS double-buffered, multi-block
+#define CASE(BM, BN, BK, IN, OUT, COMP, LA, LB, LC, LLDS, CFG, BX, BY, TX, TY)                                        \
+    runGemm<IN, OUT, COMP, LA, LB, LC>(                                                                               \
+        "coop " #BM "x" #BN "x" #BK " " #IN "->" #OUT " A:" #LA " B:" #LB " C:" #LC " lds:" #LLDS " " #CFG " " #BX    \
+        "x" #BY " tb(" #TX "," #TY ")",                                                                               \
+        gemm_PGR1_LB2_MP0_MB_CP<BM, BN, BK, IN, OUT, COMP, LA, LB, LC, LC, LLDS, CFG, BX, BY, TX, TY, 64u, kArch>,    \
+        BM * BX * (TX / 64u), BN * BY * TY, BK,                                                                      \
+        2u * sizeof(IN) * (BM * BX * (TX / 64u) + BN * BY * TY) * BK, TX, TY,                                        \
+        gemm_PGR1_LB2_MP0_MB_CP_guard<BM, BN, BK, IN, OUT, COMP, LA, LB, LC, LC, LLDS, CFG, BX, BY, TX, TY, 64u,      \
+                                      kArch>::enableRun())
+
+// no LDS, BX x BY blocks per wave
+#define CASE_MB(BM, BN, BK, IN, OUT, COMP, LA, LB, LC, BX, BY, TX, TY)                                            \
+    runGemm<IN, OUT, COMP, LA, LB, LC>(                                                                           \
+        "multi-block " #BM "x" #BN "x" #BK " " #IN "->" #OUT " A:" #LA " B:" #LB " C:" #LC " " #BX "x" #BY        \
+        " tb(" #TX "," #TY ")",                                                                                   \
+        gemm_PGR0_LB0_MP0_MB_NC<BM, BN, BK, IN, OUT, COMP, LA, LB, LC, LC, BX, BY, TX, TY, 64u, kArch>,           \
+        BM * BX * (TX / 64u), BN * BY * TY, BK, 0u, TX, TY,                                                       \
+        gemm_PGR0_LB0_MP0_MB_NC_guard<BM, BN, BK, IN, OUT, COMP, BX, BY, TX, TY, 64u, kArch>::enableRun())
+
+// no LDS, one block per wave
+#define CASE_SB(BM, BN, BK, IN, OUT, COMP, LA, LB, LC, TX, TY)                                             \
+    runGemm<IN, OUT, COMP, LA, LB, LC>(                                                                    \
+        "single-block " #BM "x" #BN "x" #BK " " #IN "->" #OUT " A:" #LA " B:" #LB " C:" #LC " tb(" #TX     \
+        "," #TY ")",                                                                                       \
+        gemm_PGR0_LB0_MP0_SB_NC<BM, BN, BK, IN, OUT, COMP, LA, LB, LC, LC, TX, TY, 64u, kArch>,            \
+        BM * (TX / 64u), BN * TY, BK, 0u, TX, TY,                                                          \
+        gemm_PGR0_LB0_MP0_SB_NC_guard<BM, BN, BK, IN, OUT, COMP, TX, TY, 64u, kArch>::enableRun())
 } // namespace
 
 int main()

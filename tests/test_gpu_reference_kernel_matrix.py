@@ -1,5 +1,6 @@
 """Drop-in checks on the GPU, part 1: the reference's cooperative, LDS double-buffered multi-block GEMM test
-kernel (test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp in the reference tree),
+kernel (test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp in the reference tree) and its
+two GEMM test kernels without LDS (test/gemm/gemm_PGR0_LB0_MP0_{MB,SB}_NC/device/kernel_device_func.hpp),
 compiled unchanged against this repository's headers, over a matrix of element types, block sizes,
 A/B/C layouts, LDS layouts, cooperation levels (block / wave / workgroup), LDS mappings
 (NT / TN / register file), blocks per wave and thread-block shapes.
@@ -37,7 +38,7 @@ def test_reference_cooperative_gemm_kernel_matrix(unit):
     exe = os.path.join(BIN, f"coop_gemm_matrix_{unit}")
     if not os.path.exists(exe):
         pytest.skip("kernel-matrix executables not built on this machine (tests/dropin/build_samples.py)")
-    expected = len(build_samples.coop_gemm_cases()[unit::build_samples.MATRIX_UNITS])
+    expected = len(build_samples.coop_gemm_units()[unit][1])
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
     tail = res.stdout[-2000:]
     failed = [line for line in res.stdout.splitlines() if line.startswith("FAILED")]
@@ -57,7 +58,7 @@ def test_reference_unit_test_kernels(unit):
     exe = os.path.join(BIN, f"unit_kernels_{unit}")
     if not os.path.exists(exe):
         pytest.skip("unit-kernel executables not built on this machine (tests/dropin/build_samples.py)")
-    expected = len(build_samples.unit_kernel_cases()[unit::build_samples.MATRIX_UNITS])
+    expected = len(build_samples.unit_kernel_units()[unit][1])
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
     tail = res.stdout[-2000:]
     failed = [line for line in res.stdout.splitlines() if line.startswith("FAILED")]
