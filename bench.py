@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-Headline workload (BASELINE.json configs[1]): D = A*B + C at M = N = K = 8192 with f16 and with
+Headline workload: D = A*B + C at M = N = K = 8192 with f16 and with
 bf16 inputs, f32 C/D, all four A/B layout combinations.  One "step" is one pass over those
 eight GEMMs; the reported value is total flops / total time in TFLOP/s (2*M*N*K per GEMM,
 reference formula test/performance.hpp:424-433).  Inputs are synthetic, uniform[-1, 1], already
