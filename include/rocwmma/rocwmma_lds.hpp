@@ -154,13 +154,28 @@ namespace rocwmma
                     reinterpret_cast<detail::u32x4*>(regs)[j]
                         = *reinterpret_cast<const detail::u32x4*>(ldsTile + offset(row, first + j));
             }
+
+            // Operand of one 16-wide MFMA block with 16 bytes of K per lane (16x16x32 f16 / bf16,
+            // 16x16x64 i8): rows [row0, row0+16), the whole 64 bytes of K of the stage; lane l
+            // holds row l % 16, chunk l / 16.  A quarter-wave reads 16 rows at one chunk index:
+            // 16 distinct bank groups by the choice of swz.
+            template <uint32_t KPackBytes>
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void
+                readBlock16(void* regs, const char* ldsTile, uint32_t row0, uint32_t /*ks*/, uint32_t lane)
+            {
+                static_assert(KPackBytes == 16u, "a 64-byte stage row feeds 16-wide blocks with 16 bytes per lane");
+                const uint32_t row = row0 + (lane & 15u);
+                *reinterpret_cast<detail::u32x4*>(regs)
+                    = *reinterpret_cast<const detail::u32x4*>(ldsTile + offset(row, lane >> 4));
+            }
         };
 
         // ---------------------------------------------------------------------------------
         // Dim-major stage (16-bit elements): 32 LDS rows (one per K index) of Dim elements.
         // Rows are cut into 32-byte segments (16 elements); segment s of K row k lives at
-        // segment position s ^ swz(k), which spreads the four K rows and two segments a
-        // half-wave touches in one transposing read over all banks.
+        // segment position s ^ swz(k).  A half-wave touches, in one transposing read, either four
+        // K rows of two neighbouring segments (32-wide blocks) or K rows k..k+3 and k+8..k+11 of
+        // one segment (16-wide blocks): swz puts both patterns on eight distinct 32-byte positions.
         // ---------------------------------------------------------------------------------
         template <uint32_t Dim>
         struct DimMajorTile
@@ -178,19 +193,19 @@ namespace rocwmma
 
             ROCWMMA_HOST_DEVICE static constexpr uint32_t swz(uint32_t k)
             {
-                return (k & 3u) << 1;
+                return ((k & 3u) << 1) | ((k >> 3) & 1u);
             }
             ROCWMMA_HOST_DEVICE static constexpr uint32_t offset(uint32_t k, uint32_t seg)
             {
                 return k * rowBytes + ((seg ^ swz(k)) << 5);
             }
             // Source byte offset of `lane` inside a copy issued by wave `wave` of a pool whose
-            // size times rowsPerCopy is a multiple of 4 (so k & 3 is the same for all its copies).
+            // size times rowsPerCopy is a multiple of 16 (so k & 15 is the same for all its copies).
             ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t laneSourceOffset(uint32_t lane, uint32_t wave, uint32_t ldBytes)
             {
                 const uint32_t kInCopy = lane / slotsPerRow;
                 const uint32_t pos     = lane % slotsPerRow;
-                const uint32_t k       = wave * rowsPerCopy + kInCopy; // only k & 3 matters
+                const uint32_t k       = wave * rowsPerCopy + kInCopy; // only k & 15 matters
                 const uint32_t seg     = (pos >> 1) ^ swz(k);
                 return kInCopy * ldBytes + (seg << 5) + ((pos & 1u) << 4);
             }
@@ -222,6 +237,32 @@ namespace rocwmma
                 const uint32_t seg   = (dim0 >> 4) + (group & 1u);
                 const uint32_t kBase = ks * 16u + (group >> 1) * 8u + (s >> 2);
                 const uint32_t inSeg = (s & 3u) << 3; // 4 elements = 8 bytes per source lane
+#pragma unroll
+                for(uint32_t kk = 0; kk < 2u; ++kk)
+                {
+                    const uint32_t k    = kBase + kk * 4u;
+                    const uint32_t addr = ldsBase + offset(k, seg) + inSeg;
+                    s16x4          v;
+                    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+                    reinterpret_cast<s16x4*>(regs)[kk] = v;
+                }
+            }
+
+            // Operand of one 16-wide MFMA block with 8 K values per lane (v_mfma_*_16x16x32):
+            // lane l ends up with dim = dim0 + l % 16 and k = (l/16)*8 + 0..7 (the stage's 32 K
+            // rows in one step).  Same remarks as for readBlock32.
+            template <uint32_t KPackBytes = 16u>
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void
+                readBlock16(void* regs, const char* ldsTile, uint32_t dim0, uint32_t /*ks*/, uint32_t lane)
+            {
+                static_assert(KPackBytes == 16u, "transposing reads feed the 8-halves-per-lane MFMA shapes");
+                typedef short s16x4 __attribute__((ext_vector_type(4)));
+                const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsPtr)ldsTile));
+                const uint32_t group   = lane >> 4;
+                const uint32_t s       = lane & 15u;
+                const uint32_t seg     = dim0 >> 4;
+                const uint32_t kBase   = group * 8u + (s >> 2);
+                const uint32_t inSeg   = (s & 3u) << 3;
 #pragma unroll
                 for(uint32_t kk = 0; kk < 2u; ++kk)
                 {

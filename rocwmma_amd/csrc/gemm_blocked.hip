@@ -42,7 +42,8 @@ namespace rocwmma_amd
                   uint32_t BlocksM_,
                   uint32_t BlocksN_,
                   uint32_t Stages_       = 4u, // LDS ring depth
-                  uint32_t WavesPerSimd_ = 1u> // resident waves per SIMD the register budget must allow
+                  uint32_t WavesPerSimd_ = 1u, // resident waves per SIMD the register budget must allow
+                  uint32_t BlockEdge_    = 32u> // MFMA block edge: 32 (32x32xK) or 16 (16x16x2K)
         struct BlockedConfig
         {
             using InT   = InT_;
@@ -57,7 +58,7 @@ namespace rocwmma_amd
             static constexpr uint32_t BlocksN = BlocksN_;
             static constexpr uint32_t Waves   = WavesM * WavesN;
             static constexpr uint32_t Threads = Waves * 64u;
-            static constexpr uint32_t Block   = 32u; // MFMA edge
+            static constexpr uint32_t Block   = BlockEdge_; // MFMA edge
             static constexpr uint32_t WaveM   = BlocksM * Block;
             static constexpr uint32_t WaveN   = BlocksN * Block;
             static constexpr uint32_t MacroM  = WavesM * WaveM;
@@ -67,7 +68,7 @@ namespace rocwmma_amd
 
             // Fragments of one MFMA step.  BlockK = K of the widest single instruction.
             static constexpr uint32_t KPack      = detail::maxKPack(detail::packClassOf<InT>());
-            static constexpr uint32_t BlockK     = KPack * 2u; // 32-wide blocks: 2 lane groups along K
+            static constexpr uint32_t BlockK     = KPack * (64u / Block); // 2 (32-wide) or 4 (16-wide) lane groups along K
             static constexpr uint32_t KPackBytes = KPack * sizeof(InT);
             static constexpr uint32_t KSteps     = MacroK / BlockK; // MFMA steps per stage (1 or 2)
 
@@ -93,14 +94,16 @@ namespace rocwmma_amd
             static constexpr uint32_t ReadsB       = BlocksN * (BKMajor ? KPackBytes / 16u : 2u);
             static constexpr uint32_t ReadsPerStep = ReadsA + ReadsB;
             static constexpr uint32_t MfmasPerStep = BlocksM * BlocksN;
-            // beta * C operand staged through LDS in the epilogue, in groups of 32 rows by
+            // beta * C operand staged through LDS in the epilogue, in groups of Block rows by
             // GroupBlocks blocks (256- or 512-byte rows), two group buffers per wave
             static constexpr uint32_t GroupBlocks
-                = (BlocksN == 4u && 2u * 32u * 128u * sizeof(OutT) * Waves <= LdsBytes) ? 4u : 2u;
-            static constexpr bool StagedC = sizeof(OutT) == 4u && BlocksN % 2u == 0u
+                = (WaveN == 128u && 2u * Block * 128u * sizeof(OutT) * Waves <= LdsBytes) ? 128u / Block : 64u / Block;
+            static constexpr bool StagedC = sizeof(OutT) == 4u && WaveN % 64u == 0u
                                             && BlocksM * (BlocksN / GroupBlocks) >= 2u
-                                            && 2u * 32u * GroupBlocks * Block * sizeof(OutT) * Waves <= LdsBytes;
+                                            && 2u * Block * GroupBlocks * Block * sizeof(OutT) * Waves <= LdsBytes;
 
+            static_assert(Block == 32u || Block == 16u, "MFMA blocks are 32 or 16 wide");
+            static_assert(Block == 32u || KPackBytes == 16u, "16-wide blocks: 16 bytes of K per lane (16-bit types, int8)");
             static_assert(AKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
             static_assert(BKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
             static_assert(TileA::bytes == BytesA && TileB::bytes == BytesB, "stage geometry mismatch");
@@ -108,6 +111,11 @@ namespace rocwmma_amd
                           "a stage must split into whole-wave copies evenly");
             static_assert((Stages - 1u) * Copies < 64u, "too many copies in flight for vmcnt");
             static_assert(LdsBytes <= Constants::AMDGCN_LDS_MAX_SIZE_BYTES, "macro tile does not fit the LDS");
+            // the dim-major tile's swizzle looks at K row bits 0..3: a wave's copies must all start
+            // on the same K row modulo 16
+            static_assert((AKMajor || (Waves * TileA::rowsPerCopy) % 16u == 0u)
+                              && (BKMajor || (Waves * TileB::rowsPerCopy) % 16u == 0u),
+                          "wave pool too small for the dim-major tile");
         };
 
         // Deals the 1-D grid to tiles so that the workgroups resident on one XCD (ids congruent
@@ -258,10 +266,20 @@ namespace rocwmma_amd
                 const char* ldsB = ldsA + Cfg::BytesA;
 #pragma unroll
                 for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
-                    TileA::template readBlock32<Cfg::KPackBytes>(f.a[i].x, ldsA, waveM * Cfg::WaveM + i * Cfg::Block, ks, lane);
+                {
+                    if constexpr(Cfg::Block == 32u)
+                        TileA::template readBlock32<Cfg::KPackBytes>(f.a[i].x, ldsA, waveM * Cfg::WaveM + i * Cfg::Block, ks, lane);
+                    else
+                        TileA::template readBlock16<Cfg::KPackBytes>(f.a[i].x, ldsA, waveM * Cfg::WaveM + i * Cfg::Block, ks, lane);
+                }
 #pragma unroll
                 for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
-                    TileB::template readBlock32<Cfg::KPackBytes>(f.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, ks, lane);
+                {
+                    if constexpr(Cfg::Block == 32u)
+                        TileB::template readBlock32<Cfg::KPackBytes>(f.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, ks, lane);
+                    else
+                        TileB::template readBlock16<Cfg::KPackBytes>(f.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, ks, lane);
+                }
             };
 
             typename Cfg::FragAcc acc[Cfg::BlocksM][Cfg::BlocksN];
@@ -349,7 +367,7 @@ namespace rocwmma_amd
                 // visible.  Two phases per loop trip so the fragment sets swap without copies.
                 // Every phase issues a stage, so the loop body and its wait counts are uniform:
                 // past the end of K the last stage is copied again into a ring slot nobody reads.
-                static_assert(Cfg::KSteps == 1u && Cfg::AKMajor && Cfg::BKMajor, "one-step stages are K-major only");
+                static_assert(Cfg::KSteps == 1u, "one MFMA step per stage");
                 Frags f0, f1;
 #define ROCWMMA_AMD_PHASE(STAGE, CUR, NXT, READ)                                                         \
     do                                                                                                  \
@@ -372,11 +390,18 @@ namespace rocwmma_amd
                 lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies>(); // stages 0 and 1 have landed
                 lds::barrier();
                 readFrags(f0, 0u, 0u);
+                if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
+                {
+                    lds::waitReads(); // the transposing reads are outside the compiler's tracking
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 uint32_t s = 0;
                 for(; s + 1u < stages; s += 2u)
                 {
                     ROCWMMA_AMD_PHASE(s, f0, f1, true);
-                    ROCWMMA_AMD_PHASE(s + 1u, f1, f0, s + 2u < stages);
+                    // (past the last stage this reads a ring slot whose content nobody multiplies:
+                    // an unconditional phase body keeps the instruction interleave intact)
+                    ROCWMMA_AMD_PHASE(s + 1u, f1, f0, true);
                 }
                 if(s < stages)
                     multiply(f0);
@@ -395,14 +420,19 @@ namespace rocwmma_amd
             // Plain stores: the 32-byte pieces a store instruction writes per row are merged into
             // full lines in the L2.  Non-temporal stores bypass that merge and were 3-5x slower
             // (4096 x 14336 x 256 int8: 157-277 us against 58 us).
+            // (accumulator layout: lane l owns runs of 4 consecutive columns of row l % Block;
+            // 32-wide blocks: 4 runs at columns 8 r + 4 (l / 32); 16-wide blocks: 1 run at 4 (l / 16))
+            constexpr uint32_t Runs     = Cfg::Block == 32u ? 4u : 1u; // runs per block per lane
+            const uint32_t     accRow   = lane & (Cfg::Block - 1u);
+            const uint32_t     accGroup = lane / Cfg::Block; // 0..1 or 0..3
             auto storeBlock = [&](OutT* dst, auto const& f, uint32_t ld) {
                 typedef uint32_t Words __attribute__((ext_vector_type(sizeof(OutT))));
 #pragma unroll
-                for(uint32_t r = 0; r < 4u; ++r)
+                for(uint32_t r = 0; r < Runs; ++r)
                 {
                     Words v;
                     __builtin_memcpy(&v, f.x + 4u * r, sizeof(v));
-                    *reinterpret_cast<Words*>(dst + static_cast<size_t>(lane & 31u) * ld + 8u * r + 4u * (lane >> 5)) = v;
+                    *reinterpret_cast<Words*>(dst + static_cast<size_t>(accRow) * ld + 8u * r + 4u * accGroup) = v;
                 }
             };
             auto           blockOffset = [&](uint32_t bi, uint32_t bj, uint32_t ld) {
@@ -421,11 +451,11 @@ namespace rocwmma_amd
                     // ring is free by now and every wave owns two group buffers in it.
                     constexpr uint32_t GB          = Cfg::GroupBlocks;
                     constexpr uint32_t RowBytes    = GB * Cfg::Block * sizeof(OutT); // 256 or 512
-                    constexpr uint32_t GroupBytes  = 32u * RowBytes;
+                    constexpr uint32_t GroupBytes  = Cfg::Block * RowBytes;
                     constexpr uint32_t RowChunks   = RowBytes / 16u;
                     constexpr uint32_t RowsPerCopy = 1024u / RowBytes;
                     constexpr uint32_t CopiesC     = GroupBytes / 1024u;
-                    constexpr uint32_t StoresD     = GB * 4u; // 16-byte stores per group
+                    constexpr uint32_t StoresD     = GB * Runs; // 16-byte stores per group
                     constexpr uint32_t GroupsPerRow = Cfg::BlocksN / GB;
                     constexpr uint32_t NG          = Cfg::BlocksM * GroupsPerRow;
                     static_assert((RowBytes == 256u || RowBytes == 512u) && 2u * GroupBytes * Cfg::Waves <= Cfg::LdsBytes
@@ -434,7 +464,6 @@ namespace rocwmma_amd
                     char*          myLds  = ldsRaw + wave * (2u * GroupBytes);
                     const char*    cWave  = reinterpret_cast<const char*>(c + static_cast<size_t>(wRow) * ldc + wCol);
                     const size_t   ldcB   = static_cast<size_t>(ldc) * sizeof(OutT);
-                    const uint32_t half   = lane >> 5;
                     const uint32_t cpRow  = lane / RowChunks; // row inside a copy
                     const uint32_t chunk  = lane % RowChunks; // chunk position inside the LDS row
                     auto           copyGroup = [&](uint32_t gi) {
@@ -444,11 +473,11 @@ namespace rocwmma_amd
                         {
                             const uint32_t r = RowsPerCopy * i + cpRow;
                             lds::asyncCopy16Streaming(myLds + (gi % 2u) * GroupBytes + i * 1024u,
-                                                      cWave + (bi * 32u + r) * ldcB + bj0 * Cfg::Block * sizeof(OutT)
+                                                      cWave + (bi * Cfg::Block + r) * ldcB + bj0 * Cfg::Block * sizeof(OutT)
                                                           + ((chunk ^ (r & 15u)) << 4));
                         }
                     };
-                    const uint32_t rdRow  = lane & 31u;
+                    const uint32_t rdRow  = accRow;
                     const uint32_t rdBase = rdRow * RowBytes;
                     copyGroup(0u);
                     copyGroup(1u);
@@ -471,9 +500,10 @@ namespace rocwmma_amd
 #pragma unroll
                         for(uint32_t bj = 0; bj < GB; ++bj)
 #pragma unroll
-                            for(uint32_t r = 0; r < 4u; ++r)
+                            for(uint32_t r = 0; r < Runs; ++r)
                             {
-                                const uint32_t g = bj * 8u + 2u * r + half; // logical chunk of this run
+                                // logical chunk of this run: block bj holds Block / 4 chunks per row
+                                const uint32_t g = bj * (Cfg::Block / 4u) + 2u * r + accGroup;
                                 detail::copyBytes<16u>(io[bj].x + 4u * r,
                                                        myLds + (gi % 2u) * GroupBytes + rdBase + ((g ^ (rdRow & 15u)) << 4));
                             }
@@ -616,7 +646,13 @@ namespace rocwmma_amd
         template <typename InT, typename OutT, typename CompT, bool AK, bool BK>
         int pickTile(GemmArgs const& g, hipStream_t stream)
         {
-            using Big    = BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 2, 4, 4, 2>;
+            // 256 x 256 macro tile, 8 waves of 64 x 128.  16-bit and int8 operands use 16-wide blocks
+            // (16x16x32 / 16x16x64 instructions: half the accumulator traffic per flop of the
+            // 32-wide forms, which is worth 5-7 % under the power cap); fp8 uses 32x32x64.
+            static constexpr bool Edge16 = sizeof(InT) == 2u || std::is_same<InT, int8_t>::value;
+            using Big    = std::conditional_t<Edge16,
+                                              BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 4, 8, 4, 2, 16>,
+                                              BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 2, 4, 4, 2, 32>>;
             using Small  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2>;
             if(g.m % Big::MacroM == 0u && g.n % Big::MacroN == 0u)
             {
