@@ -60,7 +60,10 @@ typedef enum rocwmma_amd_gemm_algo
 {
     ROCWMMA_AMD_GEMM_AUTO      = 0, /* blocked kernel when the shape allows, else wave-tile */
     ROCWMMA_AMD_GEMM_WAVE_TILE = 1, /* one block per wave, operands straight from global    */
-    ROCWMMA_AMD_GEMM_BLOCKED   = 2  /* LDS multi-buffered macro-tile kernel                 */
+    ROCWMMA_AMD_GEMM_BLOCKED   = 2, /* LDS multi-buffered macro-tile kernel                 */
+    ROCWMMA_AMD_GEMM_BLOCKED_256 = 3 /* the same with its 256 x 256 tile forced, however few
+                                        compute units that tiling occupies (AUTO and BLOCKED
+                                        fall back to 128 x 128 tiles below half occupancy)  */
 } rocwmma_amd_gemm_algo;
 
 /* Library identification: returns 10000*major + 100*minor + patch. */
@@ -116,8 +119,8 @@ int rocwmma_amd_gemm(int         dtype_in,
                      void*       stream);
 
 /* Same as rocwmma_amd_gemm with the kernel family forced (`algo` is a rocwmma_amd_gemm_algo).
- * ROCWMMA_AMD_GEMM_BLOCKED returns ROCWMMA_AMD_UNSUPPORTED_SHAPE when the shape does not fill
- * whole macro tiles, like the reference's perf_hgemm host (samples/perf_hgemm.cpp:735-765). */
+ * ROCWMMA_AMD_GEMM_BLOCKED / _BLOCKED_256 return ROCWMMA_AMD_UNSUPPORTED_SHAPE when the shape does not
+ * fill whole macro tiles, like the reference's perf_hgemm host (samples/perf_hgemm.cpp:735-765). */
 int rocwmma_amd_gemm_ex(int         algo,
                         int         dtype_in,
                         int         dtype_out,

@@ -13,7 +13,7 @@ _LIB_NAME = "librocwmma_amd.so"
 
 F16, BF16, E4M3, E5M2, I8, F32, I32 = range(7)
 ROW_MAJOR, COL_MAJOR = 0, 1
-GEMM_AUTO, GEMM_WAVE_TILE, GEMM_BLOCKED = 0, 1, 2
+GEMM_AUTO, GEMM_WAVE_TILE, GEMM_BLOCKED, GEMM_BLOCKED_256 = 0, 1, 2, 3
 
 EXPORTS = [
     "rocwmma_amd_version", "rocwmma_amd_status_string", "rocwmma_amd_device_info", "rocwmma_amd_gemm",

@@ -171,7 +171,8 @@ int rocwmma_amd_gemm_ex(int         algo,
     int rc = checkGemm(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, lda, b, ldb, c, ldc, d, ldd, alpha, beta);
     if(rc != ROCWMMA_AMD_OK)
         return rc;
-    if(algo != ROCWMMA_AMD_GEMM_AUTO && algo != ROCWMMA_AMD_GEMM_WAVE_TILE && algo != ROCWMMA_AMD_GEMM_BLOCKED)
+    if(algo != ROCWMMA_AMD_GEMM_AUTO && algo != ROCWMMA_AMD_GEMM_WAVE_TILE && algo != ROCWMMA_AMD_GEMM_BLOCKED
+       && algo != ROCWMMA_AMD_GEMM_BLOCKED_256)
         return ROCWMMA_AMD_INVALID_ARGUMENT;
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
@@ -202,8 +203,8 @@ int rocwmma_amd_gemm_ex(int         algo,
             lb              = flip(layout_a);
             blocked.layoutC = ROCWMMA_AMD_ROW_MAJOR;
         }
-        rc = launchGemmBlocked(dtype_in, dtype_out, la, lb, blocked, asStream(stream));
-        if(rc == ROCWMMA_AMD_OK || algo == ROCWMMA_AMD_GEMM_BLOCKED)
+        rc = launchGemmBlocked(dtype_in, dtype_out, la, lb, blocked, asStream(stream), algo == ROCWMMA_AMD_GEMM_BLOCKED_256);
+        if(rc == ROCWMMA_AMD_OK || algo == ROCWMMA_AMD_GEMM_BLOCKED || algo == ROCWMMA_AMD_GEMM_BLOCKED_256)
             return rc;
         if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE && rc != ROCWMMA_AMD_UNSUPPORTED_TYPE)
             return rc;

@@ -83,7 +83,9 @@ namespace rocwmma_amd
     // Family launchers (one translation unit each).  Return a rocwmma_amd_status;
     // ROCWMMA_AMD_UNSUPPORTED_SHAPE / _TYPE mean "this family has no kernel for it".
     int launchGemmWaveTile(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
-    int launchGemmBlocked(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
+    // forceLargeTile: the 256 x 256 tile or nothing (ROCWMMA_AMD_GEMM_BLOCKED_256)
+    int launchGemmBlocked(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream,
+                          bool forceLargeTile = false);
     int launchGemmSkinny(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
 
 } // namespace rocwmma_amd

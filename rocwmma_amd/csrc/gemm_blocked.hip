@@ -671,11 +671,12 @@ namespace rocwmma_amd
             return launchStatus();
         }
 
-        // Tile ladder: the 256 x 256 macro tile when the problem fills it, else 128 x 128; when even
-        // that leaves compute units without a tile (few token rows against a wide weight matrix),
-        // 128 x 64 tiles double the number of workgroups.
+        // Tile ladder: the 256 x 256 macro tile when the problem divides into enough of them to occupy
+        // at least half of the compute units, else 128 x 128; when even that leaves compute units
+        // without a tile (few token rows against a wide weight matrix), 128 x 64 tiles double the
+        // number of workgroups.
         template <typename InT, typename OutT, typename CompT, bool AK, bool BK>
-        int pickTile(GemmArgs const& g, hipStream_t stream)
+        int pickTile(GemmArgs const& g, hipStream_t stream, bool forceLargeTile)
         {
             // 256 x 256 macro tile, 8 waves of 64 x 128.  16-bit and int8 operands use 16-wide blocks
             // (16x16x32 / 16x16x64 instructions: half the accumulator traffic per flop of the
@@ -685,12 +686,18 @@ namespace rocwmma_amd
                                               BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 4, 8, 4, 2, 16>,
                                               BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 2, 4, 4, 2, 32>>;
             using Small  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2>;
-            if(g.m % Big::MacroM == 0u && g.n % Big::MacroN == 0u)
+            // (a 256 x 256 tiling that covers less than half of the compute units loses to 128 x 128
+            // tiles: 2048^3 f16 47 -> 24 us, 1024^3 30 -> 9 us, 512 x 14336 x 4096 int8 51 -> 42 us;
+            // from 144 tiles on 256 units the large tile wins again)
+            if(g.m % Big::MacroM == 0u && g.n % Big::MacroN == 0u
+               && (forceLargeTile || 2u * (g.m / Big::MacroM) * (g.n / Big::MacroN) >= computeUnits()))
             {
                 int rc = launchCfg<Big>(g, stream);
                 if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
                     return rc;
             }
+            if(forceLargeTile)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             if constexpr(AK && BK)
             {
                 using Narrow = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1>;
@@ -706,47 +713,48 @@ namespace rocwmma_amd
         }
 
         template <typename InT, typename OutT, typename CompT>
-        int pickLayout16(int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream)
+        int pickLayout16(int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream, bool big)
         {
             const bool ak = layoutA == ROCWMMA_AMD_ROW_MAJOR;
             const bool bk = layoutB == ROCWMMA_AMD_COL_MAJOR;
             if(ak && bk)
-                return pickTile<InT, OutT, CompT, true, true>(g, stream);
+                return pickTile<InT, OutT, CompT, true, true>(g, stream, big);
             if(ak && !bk)
-                return pickTile<InT, OutT, CompT, true, false>(g, stream);
+                return pickTile<InT, OutT, CompT, true, false>(g, stream, big);
             if(!ak && bk)
-                return pickTile<InT, OutT, CompT, false, true>(g, stream);
-            return pickTile<InT, OutT, CompT, false, false>(g, stream);
+                return pickTile<InT, OutT, CompT, false, true>(g, stream, big);
+            return pickTile<InT, OutT, CompT, false, false>(g, stream, big);
         }
 
         template <typename InT, typename OutT, typename CompT>
-        int pickLayout8(int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream)
+        int pickLayout8(int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream, bool big)
         {
             // 8-bit operands: only the K-contiguous pairing (row-major A, col-major B)
             if(layoutA == ROCWMMA_AMD_ROW_MAJOR && layoutB == ROCWMMA_AMD_COL_MAJOR)
-                return pickTile<InT, OutT, CompT, true, true>(g, stream);
+                return pickTile<InT, OutT, CompT, true, true>(g, stream, big);
             return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
         }
     } // namespace
 
-    int launchGemmBlocked(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream)
+    int launchGemmBlocked(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream,
+                          bool forceLargeTile)
     {
         if(g.layoutC != ROCWMMA_AMD_ROW_MAJOR)
             return ROCWMMA_AMD_UNSUPPORTED_SHAPE; // caller transposes the problem first
         if(dtypeIn == ROCWMMA_AMD_F16 && dtypeOut == ROCWMMA_AMD_F32)
-            return pickLayout16<float16_t, float32_t, float32_t>(layoutA, layoutB, g, stream);
+            return pickLayout16<float16_t, float32_t, float32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         if(dtypeIn == ROCWMMA_AMD_BF16 && dtypeOut == ROCWMMA_AMD_F32)
-            return pickLayout16<bfloat16_t, float32_t, float32_t>(layoutA, layoutB, g, stream);
+            return pickLayout16<bfloat16_t, float32_t, float32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         if(dtypeIn == ROCWMMA_AMD_F16 && dtypeOut == ROCWMMA_AMD_F16)
-            return pickLayout16<float16_t, float16_t, float32_t>(layoutA, layoutB, g, stream);
+            return pickLayout16<float16_t, float16_t, float32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         if(dtypeIn == ROCWMMA_AMD_BF16 && dtypeOut == ROCWMMA_AMD_BF16)
-            return pickLayout16<bfloat16_t, bfloat16_t, float32_t>(layoutA, layoutB, g, stream);
+            return pickLayout16<bfloat16_t, bfloat16_t, float32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         if(dtypeIn == ROCWMMA_AMD_I8 && dtypeOut == ROCWMMA_AMD_I32)
-            return pickLayout8<int8_t, int32_t, int32_t>(layoutA, layoutB, g, stream);
+            return pickLayout8<int8_t, int32_t, int32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         if(dtypeIn == ROCWMMA_AMD_E4M3 && dtypeOut == ROCWMMA_AMD_F32)
-            return pickLayout8<float8_t, float32_t, float32_t>(layoutA, layoutB, g, stream);
+            return pickLayout8<float8_t, float32_t, float32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         if(dtypeIn == ROCWMMA_AMD_E5M2 && dtypeOut == ROCWMMA_AMD_F32)
-            return pickLayout8<bfloat8_t, float32_t, float32_t>(layoutA, layoutB, g, stream);
+            return pickLayout8<bfloat8_t, float32_t, float32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         return ROCWMMA_AMD_UNSUPPORTED_TYPE;
     }
 

@@ -14,6 +14,18 @@ pytestmark = pytest.mark.gpu
 OUT_OF = {orc.F16: orc.F32, orc.BF16: orc.F32, orc.E4M3: orc.F32, orc.E5M2: orc.F32, orc.I8: orc.I32}
 
 
+# kernel families a test runs through; GEMM_BLOCKED_256 forces the 256 x 256 configuration, which
+# GEMM_BLOCKED only picks for problems that occupy at least half of the compute units
+ALGOS = [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED, rw.GEMM_BLOCKED_256]
+
+
+def tile_dims(algo, m, n):
+    """Problem size for `algo`: the forced 256 x 256 tile needs multiples of 256."""
+    if algo == rw.GEMM_BLOCKED_256:
+        return -(-m // 256) * 256, -(-n // 256) * 256
+    return m, n
+
+
 def run_gemm(dtype_in, dtype_out, la, lb, lc, m, n, k, a, b, c, alpha, beta, algo):
     import torch
 
@@ -43,7 +55,7 @@ def check(dtype_in, dtype_out, got, want, tol):
 
 
 # ------------------------------------------------ type combinations of the reference's GEMM tests
-@pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED])
+@pytest.mark.parametrize("algo", ALGOS)
 @pytest.mark.parametrize("la,lb", [(RM, CM), (CM, RM), (RM, RM), (CM, CM)])
 @pytest.mark.parametrize("dtype_in,dtype_out,tol", [
     (orc.F16, orc.F16, 1e-3),    # <f16, f16, f32>
@@ -53,9 +65,10 @@ def check(dtype_in, dtype_out, got, want, tol):
 def test_narrow_output_and_f32_type_combinations(dtype_in, dtype_out, tol, la, lb, algo):
     """Input/Output/Compute triples of test/gemm/gemm_common_test_params.hpp:51-111 beyond the
     f32-output ones: C and D in the input type, f32 compute."""
-    if dtype_in == orc.F32 and algo == rw.GEMM_BLOCKED:
+    if dtype_in == orc.F32 and algo != rw.GEMM_WAVE_TILE:
         pytest.skip("f32 inputs run on the wave-tile kernel only")
     m, n, k = 256, 384, 192
+    m, n = tile_dims(algo, m, n)
     a = uniform_bits(51, dtype_in, m * k)
     b = uniform_bits(52, dtype_in, k * n)
     c = uniform_bits(53, dtype_out, m * n)
@@ -77,13 +90,14 @@ def test_config1_256_cubed_f16_alpha_beta_2(algo):
 
 
 # ---------------------------------------------------------------- all types x layouts, both families
-@pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED])
+@pytest.mark.parametrize("algo", ALGOS)
 @pytest.mark.parametrize("lc", [RM, CM])
 @pytest.mark.parametrize("lb", [RM, CM])
 @pytest.mark.parametrize("la", [RM, CM])
 @pytest.mark.parametrize("dtype_in", [orc.F16, orc.BF16])
 def test_16bit_types_all_layouts(dtype_in, la, lb, lc, algo):
     m, n, k = 256, 384, 192
+    m, n = tile_dims(algo, m, n)
     a = uniform_bits(21, dtype_in, m * k)
     b = uniform_bits(22, dtype_in, k * n)
     c = np.random.default_rng(23).uniform(-1, 1, m * n).astype(np.float32)
@@ -92,7 +106,7 @@ def test_16bit_types_all_layouts(dtype_in, la, lb, lc, algo):
     check(dtype_in, orc.F32, got, want, 1e-3)
 
 
-@pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED])
+@pytest.mark.parametrize("algo", ALGOS)
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3, orc.E5M2])
 def test_8bit_types_k_contiguous(dtype_in, algo):
     m, n, k = 256, 256, 512
@@ -126,7 +140,7 @@ def test_8bit_types_other_layouts_wave_tile(dtype_in, la, lb):
     check(dtype_in, out, got, want, tol_for(dtype_in))
 
 
-@pytest.mark.parametrize("algo", [rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED])
+@pytest.mark.parametrize("algo", ALGOS)
 @pytest.mark.parametrize("dtype_in", [orc.F16, orc.BF16, orc.E4M3, orc.E5M2, orc.I8])
 def test_exact_integer_pattern_is_bit_exact(dtype_in, algo):
     """The reference's fill makes every partial sum an exact integer, so any summation order
@@ -170,7 +184,7 @@ def test_leading_dimensions_larger_than_extent():
     A = orc.encode(orc.F16, rng.uniform(-1, 1, (m, lda)).astype(np.float32))
     B = orc.encode(orc.F16, rng.uniform(-1, 1, (n, ldb)).astype(np.float32))  # col-major B: n columns of ldb
     C = rng.uniform(-1, 1, (m, ldc)).astype(np.float32)
-    for algo in (rw.GEMM_WAVE_TILE, rw.GEMM_BLOCKED):
+    for algo in ALGOS:
         d = torch.full((m, ldc), 777.0, device="cuda")
         rw.gemm(orc.F16, orc.F32, RM, CM, RM, m, n, k, to_device(A), to_device(B), to_device(C), d, 1.0, 1.0,
                 lda=lda, ldb=ldb, ldc=ldc, ldd=ldc, algo=algo)
@@ -194,7 +208,7 @@ def test_c_may_alias_d(dtype_in, dtype_out):
     c = uniform_bits(83, dtype_out, m * n)
     alpha, beta = (1.0, 1.0) if dtype_in == orc.I8 else (0.5, 1.5)
     want = orc.gemm(dtype_in, dtype_out, RM, CM, RM, RM, m, n, k, a, b, c, alpha, beta)
-    for algo in (rw.GEMM_BLOCKED, rw.GEMM_WAVE_TILE):
+    for algo in ALGOS:
         cd = to_device(c.copy())
         rw.gemm(dtype_in, dtype_out, RM, CM, RM, m, n, k, to_device(a), to_device(b), cd, cd, alpha, beta, algo=algo)
         torch.cuda.synchronize()
@@ -217,7 +231,7 @@ def test_padded_leading_dimensions_every_layout_many_tiles(la, lb):
     C = rng.uniform(-1, 1, (m, n + pad_c)).astype(np.float32)
     want = orc.gemm(orc.F16, orc.F32, la, lb, RM, RM, m, n, k, np.ascontiguousarray(A[:, :a_cols]),
                     np.ascontiguousarray(B[:, :b_cols]), np.ascontiguousarray(C[:, :n]), 1.0, -2.0)
-    for algo in (rw.GEMM_BLOCKED, rw.GEMM_WAVE_TILE):
+    for algo in ALGOS:
         d = torch.full((m, n + pad_c), 777.0, device="cuda")
         rw.gemm(orc.F16, orc.F32, la, lb, RM, m, n, k, to_device(A), to_device(B), to_device(C), d, 1.0, -2.0,
                 lda=a_cols + pad_a, ldb=b_cols + pad_b, ldc=n + pad_c, ldd=n + pad_c, algo=algo)
