@@ -466,6 +466,44 @@ namespace rocwmma_amd
                     *reinterpret_cast<Words*>(dst + static_cast<size_t>(accRow) * ld + 8u * r + 4u * accGroup) = v;
                 }
             };
+            // 16-bit outputs with 16-wide blocks: a lane's run is only 8 bytes, a store instruction would
+            // write 32-byte pieces.  Two neighbouring blocks are handled together: v_permlane16_swap
+            // exchanges the second block's run of a lane in an even 16-lane row with the first block's
+            // run of its partner in the next row, after which every lane owns 8 consecutive columns
+            // (even rows: of the first block, odd rows: of the second) and moves 16 bytes; an
+            // instruction then covers 64 contiguous bytes per matrix row.  The exchange is its own
+            // inverse, so C is read the same way.
+            constexpr bool PairIO = Cfg::Block == 16u && sizeof(OutT) == 2u && Cfg::BlocksN % 2u == 0u;
+            const uint32_t pairCol = (accGroup & 1u) * 16u + 4u * (accGroup & 2u);
+            auto           swapPair = [](auto& fx, auto& fy) {
+                uint32_t x[2], y[2];
+                __builtin_memcpy(x, fx.x, 8);
+                __builtin_memcpy(y, fy.x, 8);
+#pragma unroll
+                for(uint32_t w = 0; w < 2u; ++w)
+                {
+                    auto r = __builtin_amdgcn_permlane16_swap(x[w], y[w], false, false);
+                    x[w]   = r[0];
+                    y[w]   = r[1];
+                }
+                __builtin_memcpy(fx.x, x, 8);
+                __builtin_memcpy(fy.x, y, 8);
+            };
+            auto storePair = [&](OutT* dst, auto& fx, auto& fy, uint32_t ld) {
+                swapPair(fx, fy);
+                typedef uint32_t Words __attribute__((ext_vector_type(4)));
+                Words            v;
+                __builtin_memcpy(&v, fx.x, 8);
+                __builtin_memcpy(reinterpret_cast<char*>(&v) + 8, fy.x, 8);
+                *reinterpret_cast<Words*>(dst + static_cast<size_t>(accRow) * ld + pairCol) = v;
+            };
+            auto loadPair = [&](auto& fx, auto& fy, const OutT* src, uint32_t ld) {
+                typedef uint32_t Words __attribute__((ext_vector_type(4)));
+                const Words      v = *reinterpret_cast<const Words*>(src + static_cast<size_t>(accRow) * ld + pairCol);
+                __builtin_memcpy(fx.x, &v, 8);
+                __builtin_memcpy(fy.x, reinterpret_cast<const char*>(&v) + 8, 8);
+                swapPair(fx, fy);
+            };
             auto           blockOffset = [&](uint32_t bi, uint32_t bj, uint32_t ld) {
                 return static_cast<size_t>(wRow + bi * Cfg::Block) * ld + wCol + bj * Cfg::Block;
             };
@@ -562,9 +600,18 @@ namespace rocwmma_amd
                 {
                 typename Cfg::FragC fc[2][Cfg::BlocksN];
                 auto                loadGroup = [&](uint32_t bi) {
+                    if constexpr(PairIO)
+                    {
 #pragma unroll
-                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                        load_matrix_sync(fc[bi % 2u][bj], c + blockOffset(bi, bj, ldc), ldc);
+                        for(uint32_t bj = 0; bj < Cfg::BlocksN; bj += 2u)
+                            loadPair(fc[bi % 2u][bj], fc[bi % 2u][bj + 1u], c + blockOffset(bi, bj, ldc), ldc);
+                    }
+                    else
+                    {
+#pragma unroll
+                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                            load_matrix_sync(fc[bi % 2u][bj], c + blockOffset(bi, bj, ldc), ldc);
+                    }
                 };
                 loadGroup(0u);
                 if constexpr(Cfg::BlocksM > 1u)
@@ -580,9 +627,18 @@ namespace rocwmma_amd
                         for(uint32_t e = 0; e < io.num_elements; ++e)
                             io.x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e] + beta * static_cast<CompT>(io.x[e]));
                     }
+                    if constexpr(PairIO)
+                    {
 #pragma unroll
-                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                        storeBlock(d + blockOffset(bi, bj, ldd), fc[bi % 2u][bj], ldd);
+                        for(uint32_t bj = 0; bj < Cfg::BlocksN; bj += 2u)
+                            storePair(d + blockOffset(bi, bj, ldd), fc[bi % 2u][bj], fc[bi % 2u][bj + 1u], ldd);
+                    }
+                    else
+                    {
+#pragma unroll
+                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                            storeBlock(d + blockOffset(bi, bj, ldd), fc[bi % 2u][bj], ldd);
+                    }
                     if(bi + 2u < Cfg::BlocksM)
                         loadGroup(bi + 2u);
                     __builtin_amdgcn_sched_barrier(0);
@@ -618,9 +674,18 @@ namespace rocwmma_amd
                             for(uint32_t e = 0; e < fd[bj].num_elements; ++e)
                                 fd[bj].x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e]);
                         }
+                        if constexpr(PairIO)
+                        {
 #pragma unroll
-                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                            storeBlock(d + blockOffset(bi, bj, ldd), fd[bj], ldd);
+                            for(uint32_t bj = 0; bj < Cfg::BlocksN; bj += 2u)
+                                storePair(d + blockOffset(bi, bj, ldd), fd[bj], fd[bj + 1u], ldd);
+                        }
+                        else
+                        {
+#pragma unroll
+                            for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                                storeBlock(d + blockOffset(bi, bj, ldd), fd[bj], ldd);
+                        }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }

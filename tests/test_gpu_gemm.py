@@ -62,7 +62,8 @@ def check(dtype_in, dtype_out, got, want, tol):
     (orc.BF16, orc.BF16, 4e-3),  # <bf16, bf16, f32>: one bf16 ulp (2^-8) of a value v costs v/(2v+1) * 2^-8 <= 2e-3
     (orc.F32, orc.F32, 1e-5),    # <f32, f32, f32> (wave-tile kernel only)
 ])
-def test_narrow_output_and_f32_type_combinations(dtype_in, dtype_out, tol, la, lb, algo):
+@pytest.mark.parametrize("beta", [-0.5, 0.0])
+def test_narrow_output_and_f32_type_combinations(dtype_in, dtype_out, tol, la, lb, algo, beta):
     """Input/Output/Compute triples of test/gemm/gemm_common_test_params.hpp:51-111 beyond the
     f32-output ones: C and D in the input type, f32 compute."""
     if dtype_in == orc.F32 and algo != rw.GEMM_WAVE_TILE:
@@ -72,8 +73,8 @@ def test_narrow_output_and_f32_type_combinations(dtype_in, dtype_out, tol, la, l
     a = uniform_bits(51, dtype_in, m * k)
     b = uniform_bits(52, dtype_in, k * n)
     c = uniform_bits(53, dtype_out, m * n)
-    got = run_gemm(dtype_in, dtype_out, la, lb, RM, m, n, k, a, b, c, 1.5, -0.5, algo)
-    want = orc.gemm(dtype_in, dtype_out, la, lb, RM, RM, m, n, k, a, b, c, 1.5, -0.5)
+    got = run_gemm(dtype_in, dtype_out, la, lb, RM, m, n, k, a, b, c if beta else None, 1.5, beta, algo)
+    want = orc.gemm(dtype_in, dtype_out, la, lb, RM, RM, m, n, k, a, b, c if beta else None, 1.5, beta)
     check(dtype_in, dtype_out, got, want, tol)
 
 
