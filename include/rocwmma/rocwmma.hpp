@@ -427,6 +427,21 @@ namespace rocwmma
         using type = typename fragment<MatrixT, BlockM, BlockN, BlockK, DataT, DataLayoutT>::IOTraits;
     };
 
+    // I/O description of a fragment (reference: accessors.hpp:43-49): here only its traits
+    template <typename FragT>
+    struct GetIOConfig;
+    template <typename MatrixT, uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT, typename DataLayoutT>
+    struct GetIOConfig<fragment<MatrixT, BlockM, BlockN, BlockK, DataT, DataLayoutT>>
+    {
+        struct type
+        {
+            using IOTraits = typename fragment<MatrixT, BlockM, BlockN, BlockK, DataT, DataLayoutT>::IOTraits;
+            using IOShape  = rocwmma::IOShape<MatrixT, BlockM, BlockN, BlockK>;
+        };
+    };
+    template <typename FragT>
+    using GetIOConfig_t = typename GetIOConfig<std::decay_t<FragT>>::type;
+
     template <typename FragT>
     using GetDataType_t = typename GetDataType<std::decay_t<FragT>>::type;
     template <typename FragT>

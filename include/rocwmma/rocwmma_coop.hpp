@@ -2,11 +2,13 @@
 // each wave a share of it.
 //
 // Same overload set and argument meaning as rocWMMA's cooperative API (reference:
-// library/include/rocwmma/rocwmma_coop.hpp:78-412).  The work is split into the fragment's
-// items (see internal/fragment_io.hpp); wave `waveIndex` of `waveCount` moves items
-// waveIndex, waveIndex + waveCount, ...  A fragment filled by a cooperative load holds only
-// that wave's share and must be written back by the cooperative store with the same
-// (waveIndex, waveCount).  Waves beyond the number of items do nothing.  The deprecated
+// library/include/rocwmma/rocwmma_coop.hpp:78-412).  Wave `waveIndex` of `waveCount` moves
+// the register elements [waveIndex * size / waveCount, (waveIndex + 1) * size / waveCount) of
+// the fragment (whole items, or equal pieces of an item when there are more waves than items;
+// see internal/fragment_io.hpp) and leaves the others alone.  A fragment filled by a
+// cooperative load holds only that wave's share, at its ordinary register positions, and must
+// be written back by a cooperative store with the same (waveIndex, waveCount), as the same
+// fragment type or reinterpreted as another one with the same element count.  The deprecated
 // splitCount arguments are accepted and ignored, as in the reference
 // (rocwmma_coop_impl.hpp:44-53,116-132).
 //

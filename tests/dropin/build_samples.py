@@ -23,6 +23,9 @@ coop_gemm_cases() enumerates: the axes of the reference's own test matrix
 (test/gemm/gemm_common_test_params.hpp:44-330, test/gemm/gemm_PGR1_LB2_MP0_MB_CP/test/*):
 element types, block sizes, A/B/C layouts, LDS layout, cooperation level and LDS mapping, blocks
 per wave, thread-block shape.  tests/test_gpu_reference_kernel_matrix.py runs the executables.
+
+Unit-test kernels and DLRM kernels: tests/dropin/unit_kernels.cpp and tests/dropin/dlrm_kernels.cpp are
+the host sides for the device kernels under test/unit/*/device and test/dlrm/device.
 """
 import os
 import shutil
@@ -273,6 +276,25 @@ def build_unit_kernels(verbose=False):
                              [REFERENCE_TESTS, os.path.join(REFERENCE_TESTS, "unit")], verbose)
 
 
+def build_dlrm_kernels(verbose=False):
+    """Compiles the reference's four DLRM test kernels (test/dlrm/device/*.hpp) with the host side in
+    tests/dropin/dlrm_kernels.cpp; returns the executable's path in a list."""
+    if not (os.path.isdir(os.path.join(REFERENCE_TESTS, "dlrm")) and _hipcc() is not None):
+        return []
+    os.makedirs(BIN, exist_ok=True)
+    exe = os.path.join(BIN, "dlrm_kernels")
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-std=c++17", "-O2", "-DROCWMMA_AMD_REPORT_ARCH_ID=0x942",
+           "-I" + os.path.join(ROOT, "include"), "-I" + REFERENCE_TESTS, "-I" + os.path.join(REFERENCE_TESTS, "dlrm"),
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+           os.path.join(HERE, "dlrm_kernels.cpp"), "-o", exe]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"dlrm_kernels: hipcc failed\n{res.stdout[-3000:]}")
+    if verbose:
+        print(exe)
+    return [exe]
+
+
 if __name__ == "__main__":
     if not available():
         print("reference checkout or hipcc not present: nothing built")
@@ -280,3 +302,4 @@ if __name__ == "__main__":
     build(verbose=True)
     build_coop_gemm_matrix(verbose=True)
     build_unit_kernels(verbose=True)
+    build_dlrm_kernels(verbose=True)

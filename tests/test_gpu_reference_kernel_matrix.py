@@ -14,6 +14,12 @@ MappingUtil coordinate maps and their overrides), over the reference's block siz
 (16..256 x 8..256, test/unit/unit_test_params.hpp:89-141), both layouts, eight element types and six
 thread-block shapes; each must move exactly the elements its contract says (tests/dropin/unit_kernels.cpp).
 
+Part 3: the reference's DLRM dot-interaction test kernels (test/dlrm/device/dlrm_dot_{fwd,bwd}.hpp and the
+LDS variants dlrm_dot_{fwd,bwd}_lds.hpp, which keep fragments in LDS as a register file and, in the backward
+pass, reinterpret cooperatively loaded fragments as register-file fragments), for f16 and f32, tiles of 16
+and 32 and the reference's problem sizes; inputs are -1, 0, 1 so results must equal a CPU loop exactly
+(tests/dropin/dlrm_kernels.cpp).
+
 tests/dropin/build_samples.py enumerates the cases and builds the executables
 on the development machine (where the reference checkout is); they travel with the tree.  Where
 they are absent the tests are skipped."""
@@ -70,3 +76,18 @@ def test_reference_unit_test_kernels(unit):
     assert nfailed == 0 and passed + skipped == expected, tail
     # the kernels' own guard rejects blocks that exceed a wave's register budget (e.g. 256 x 256 f64)
     assert passed >= 0.8 * expected, tail
+
+
+def test_reference_dlrm_test_kernels():
+    exe = os.path.join(BIN, "dlrm_kernels")
+    if not os.path.exists(exe):
+        pytest.skip("DLRM kernel executable not built on this machine (tests/dropin/build_samples.py)")
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+    tail = res.stdout[-2000:]
+    failed = [line for line in res.stdout.splitlines() if line.startswith("FAILED")]
+    assert not failed, "\n".join(failed[:10])
+    assert res.returncode == 0, tail
+    summary = re.search(r"SUMMARY: (\d+) passed, (\d+) failed, (\d+) skipped", res.stdout)
+    assert summary, tail
+    # 2 element types x 2 tile sizes x 4 problem sizes x {forward, backward} x {plain, LDS}
+    assert tuple(map(int, summary.groups())) == (64, 0, 0), tail
