@@ -42,7 +42,7 @@ namespace rocwmma_amd
                   uint32_t BlocksM_,
                   uint32_t BlocksN_,
                   uint32_t Stages_       = 4u, // LDS ring depth
-                  uint32_t WavesPerSimd_ = 1u, // resident waves per SIMD the register budget must allow
+                  uint32_t WavesPerSimd_ = 1u, // waves per SIMD: sizes the register budget, and no more become resident
                   uint32_t BlockEdge_    = 32u> // MFMA block edge: 32 (32x32xK) or 16 (16x16x2K)
         struct BlockedConfig
         {
@@ -750,7 +750,12 @@ namespace rocwmma_amd
             using Big    = std::conditional_t<Edge16,
                                               BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 4, 8, 4, 2, 16>,
                                               BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 2, 4, 4, 2, 32>>;
-            using Small  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2>;
+            // (the 4-wave configurations declare the occupancy their LDS use allows, two and three
+            // workgroups per compute unit: the compiler pads the register count of a kernel that
+            // declares one wave per SIMD so that no second workgroup fits, and problems with more
+            // tiles than compute units then ran in whole rounds: 512 x 14336 x 4096 f16 90 -> 77 us,
+            // 256 x 14336 x 4096 fp8 36 -> 30 us)
+            using Small  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2, 4, 2>;
             // (a 256 x 256 tiling that covers less than half of the compute units loses to 128 x 128
             // tiles: 2048^3 f16 47 -> 24 us, 1024^3 30 -> 9 us, 512 x 14336 x 4096 int8 51 -> 42 us;
             // from 144 tiles on 256 units the large tile wins again)
@@ -765,7 +770,13 @@ namespace rocwmma_amd
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             if constexpr(AK && BK)
             {
-                using Narrow = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1>;
+                #ifndef NARROW_STAGES
+#define NARROW_STAGES 4
+#endif
+                #ifndef NARROW_WAVES
+#define NARROW_WAVES 1
+#endif
+                using Narrow = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, NARROW_STAGES, NARROW_WAVES>;
                 if(g.m % Small::MacroM == 0u && g.n % Small::MacroN == 0u
                    && (g.m / Small::MacroM) * (g.n / Small::MacroN) < computeUnits())
                 {
