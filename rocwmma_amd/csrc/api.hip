@@ -178,9 +178,10 @@ int rocwmma_amd_gemm_ex(int         algo,
         return ROCWMMA_AMD_NO_DEVICE;
 
     GemmArgs args{m, n, k, a, b, c, d, lda, ldb, c ? ldc : ldd, ldd, alpha, beta, layout_c};
-    if(algo == ROCWMMA_AMD_GEMM_AUTO && m <= 32u)
+    if(algo == ROCWMMA_AMD_GEMM_AUTO && m <= 128u)
     {
-        // few token rows against a wide 8-bit weight matrix: the weight-streaming kernel
+        // few token rows against a wide 8-bit weight matrix: the weight-streaming kernels (<= 32 rows;
+        // 48..112 rows with the K slices spread over workgroups)
         rc = launchGemmSkinny(dtype_in, dtype_out, layout_a, layout_b, args, asStream(stream));
         if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE && rc != ROCWMMA_AMD_UNSUPPORTED_TYPE)
             return rc;

@@ -1,5 +1,6 @@
 // Skinny quantised GEMM: D = alpha * A * B + beta * C for M <= 32 token rows against an
-// N x K weight matrix (8-bit A row-major, B col-major, C/D row-major).
+// N x K weight matrix (8-bit A row-major, B col-major, C/D row-major), and a K-sliced variant
+// for 48..112 token rows further down.
 //
 // At these shapes (the reference's GEMM kernels, samples/perf_hgemm.cpp:518-714, need whole
 // 128-wide macro tiles in M and would leave most of the chip idle) the job is streaming the
@@ -183,9 +184,255 @@ namespace rocwmma_amd
             return launchStatus();
         }
 
+
+        // ---- 48..112 token rows: K slices over workgroups ------------------------------------
+        // With more than 32 token rows A no longer fits the LDS whole, and the blocked kernel needs
+        // whole 128-row tiles.  Here a workgroup keeps one K slice of A (at most 128 KiB)
+        // in LDS and its 8 waves stream the same K slice of 32 weight rows each, so a compute
+        // unit reads its slice of A once.  The K slices of a block of outputs belong to different
+        // workgroups: D is first set to beta * C by a small kernel, then every workgroup adds
+        // alpha * (its partial product) with atomic adds.  The partial tile goes through LDS
+        // (the A slice is no longer needed) so that an atomic instruction covers 256 contiguous
+        // bytes of one output row.  int32 sums are exact in any order; f32 sums of more than two
+        // slices depend on the order the workgroups arrive in (last-bit differences between runs).
+        // The atomic adds set the pace (about 3 ns per output element and slice over the whole
+        // chip: 64 x 14336 x 4096 takes 24 us, 128 rows would take 36 us against 25 us on the
+        // blocked kernel, which therefore keeps the multiples of 128).
+        constexpr uint32_t kSlicedWaves = 8;
+        constexpr uint32_t kSlicedNB    = 2; // blocks of 16 weight rows per wave
+        constexpr uint32_t kSlicedCols  = kSlicedWaves * kSlicedNB * 16u; // output columns per workgroup
+        constexpr uint32_t kSlicedAhead = 4;
+        constexpr uint32_t kSlicedMaxM  = 128;
+
+        template <typename OutT, typename CompT>
+        __global__ void __launch_bounds__(256)
+            initOutputKernel(uint32_t m, uint32_t n, OutT const* c, uint32_t ldc, OutT* d, uint32_t ldd, CompT beta)
+        {
+            typedef OutT Vec __attribute__((ext_vector_type(4)));
+            const uint32_t perRow = n / 4u;
+            const uint32_t idx    = blockIdx.x * 256u + threadIdx.x;
+            if(idx >= m * perRow)
+                return;
+            const uint32_t row = idx / perRow, col = (idx % perRow) * 4u;
+            Vec            v   = {0, 0, 0, 0};
+            if(beta != static_cast<CompT>(0))
+            {
+                const Vec cv = *reinterpret_cast<const Vec*>(c + static_cast<size_t>(row) * ldc + col);
+#pragma unroll
+                for(uint32_t e = 0; e < 4u; ++e)
+                    v[e] = static_cast<OutT>(beta * static_cast<CompT>(cv[e]));
+            }
+            *reinterpret_cast<Vec*>(d + static_cast<size_t>(row) * ldd + col) = v;
+        }
+
+        ROCWMMA_DEVICE inline void addTo(int32_t* p, int32_t v)
+        {
+            __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        ROCWMMA_DEVICE inline void addTo(float* p, float v)
+        {
+            unsafeAtomicAdd(p, v);
+        }
+
+        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks>
+        __global__ void __launch_bounds__(64 * kSlicedWaves) gemmSlicedKernel(uint32_t   m,
+                                                                              uint32_t   n,
+                                                                              uint32_t   k,
+                                                                              InT const* a,
+                                                                              InT const* b,
+                                                                              OutT*      d,
+                                                                              uint32_t   lda,
+                                                                              uint32_t   ldb,
+                                                                              uint32_t   ldd,
+                                                                              CompT      alpha)
+        {
+            using FragA   = fragment<matrix_a, 16, 16, kSkinnyK, InT, row_major>;
+            using FragB   = fragment<matrix_b, 16, 16, kSkinnyK, InT, col_major>;
+            using FragAcc = fragment<accumulator, 16, 16, kSkinnyK, CompT>;
+            using MapA    = detail::InputMap<16, kSkinnyK, 16, detail::packClassOf<InT>()>;
+            static_assert(sizeof(InT) == 1 && std::is_same<OutT, CompT>::value, "8-bit operands, 32-bit results");
+            constexpr uint32_t Ahead = kSlicedAhead;
+
+            extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
+            char* aTile = ldsRaw; // [m][kLen] bytes, chunk c of row r at chunk position c ^ (r % 16)
+
+            const uint32_t lane   = threadIdx.x & 63u;
+            const uint32_t wave   = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            const uint32_t kLen   = k / gridDim.y;
+            const uint32_t kBeg   = blockIdx.y * kLen;
+            constexpr uint32_t NB = kSlicedNB;
+            const InT*         bPtr[NB];
+#pragma unroll
+            for(uint32_t j = 0; j < NB; ++j)
+            {
+                const uint32_t nBlock = (blockIdx.x * kSlicedWaves + wave) * NB + j; // block of 16 weight rows
+                const uint32_t n0     = (nBlock * 16u < n ? nBlock : 0u) * 16u; // idle blocks shadow block 0
+                bPtr[j]               = b + static_cast<size_t>(n0) * ldb + kBeg;
+            }
+
+            // this lane's A operand rows in LDS and its swizzle
+            const uint32_t aRow = lane & 15u;
+            auto           loadB = [&](FragB(&fb)[Ahead][NB], uint32_t kk) {
+#pragma unroll
+                for(uint32_t u = 0; u < Ahead; ++u)
+#pragma unroll
+                    for(uint32_t j = 0; j < NB; ++j)
+                        load_matrix_sync(fb[u][j], bPtr[j] + kk + u * kSkinnyK, ldb);
+            };
+            // the first batch of weight fragments is requested before anything else
+            FragB fb[Ahead][NB];
+            loadB(fb, 0u);
+
+            // A slice -> LDS: whole-wave 1 KiB copies, kLen / 1024 per row
+            {
+                const uint32_t perRow = kLen / 1024u;
+                const uint32_t copies = m * perRow;
+                for(uint32_t j = wave; j < copies; j += kSlicedWaves)
+                {
+                    const uint32_t r   = j / perRow;
+                    const uint32_t pos = (j % perRow) * 64u + lane; // chunk position inside the LDS row
+                    lds::asyncCopy16(aTile + r * kLen + (j % perRow) * 1024u,
+                                     reinterpret_cast<const char*>(a) + static_cast<size_t>(r) * lda + kBeg
+                                         + ((pos ^ (r & 15u)) << 4));
+                }
+            }
+
+            FragAcc acc[MBlocks][NB];
+#pragma unroll
+            for(uint32_t i = 0; i < MBlocks; ++i)
+#pragma unroll
+                for(uint32_t j = 0; j < NB; ++j)
+                    fill_fragment(acc[i][j], static_cast<CompT>(0));
+
+            auto multiply = [&](FragB(&fb)[Ahead][NB], uint32_t kk) {
+#pragma unroll
+                for(uint32_t u = 0; u < Ahead; ++u)
+#pragma unroll
+                    for(uint32_t i = 0; i < MBlocks; ++i)
+                    {
+                        FragA          fa;
+                        const uint32_t row = i * 16u + aRow;
+#pragma unroll
+                        for(uint32_t ch = 0; ch < MapA::nchunks; ++ch)
+#pragma unroll
+                            for(uint32_t piece = 0; piece < MapA::kpack / 16u; ++piece)
+                            {
+                                const uint32_t kByte = kk + u * kSkinnyK + MapA::chunkK(ch, lane) + piece * 16u;
+                                detail::copyBytes<16u>(fa.x + ch * MapA::kpack + piece * 16u,
+                                                       aTile + row * kLen + (((kByte >> 4) ^ (row & 15u)) << 4));
+                            }
+#pragma unroll
+                        for(uint32_t j = 0; j < NB; ++j)
+                            mma_sync(acc[i][j], fa, fb[u][j], acc[i][j]);
+                    }
+            };
+
+            lds::waitCopiesAndReads<0>();
+            __syncthreads();
+            multiply(fb, 0u);
+            for(uint32_t kk = Ahead * kSkinnyK; kk < kLen; kk += Ahead * kSkinnyK)
+            {
+                loadB(fb, kk);
+                multiply(fb, kk);
+            }
+
+            // The partial tile (m x 256 results) replaces the A slice in LDS: rows of 64 16-byte
+            // chunks, chunk c of row r at position c ^ (r % 16) (conflict-free for the 16 rows a
+            // quarter-wave writes and for the 64 consecutive columns a wave reads back).
+            __syncthreads();
+            using Quad     = CompT __attribute__((ext_vector_type(4)));
+            Quad* outTile  = reinterpret_cast<Quad*>(ldsRaw);
+            constexpr uint32_t RowChunks = kSlicedCols / 4u;
+#pragma unroll
+            for(uint32_t i = 0; i < MBlocks; ++i)
+#pragma unroll
+                for(uint32_t j = 0; j < NB; ++j)
+                {
+                    const uint32_t row   = i * 16u + (lane & 15u);
+                    const uint32_t chunk = (wave * NB + j) * 4u + (lane >> 4);
+                    Quad           v     = *reinterpret_cast<Quad*>(acc[i][j].x);
+                    outTile[row * RowChunks + (chunk ^ (row & 15u))] = alpha * v;
+                }
+            __syncthreads();
+            const CompT* outFlat = reinterpret_cast<const CompT*>(ldsRaw);
+            for(uint32_t row = wave; row < m; row += kSlicedWaves)
+            {
+#pragma unroll
+                for(uint32_t q = 0; q < kSlicedCols / 64u; ++q)
+                {
+                    const uint32_t col  = q * 64u + lane;
+                    const uint32_t gcol = blockIdx.x * kSlicedCols + col;
+                    const CompT    v    = outFlat[(row * RowChunks + ((col >> 2) ^ (row & 15u))) * 4u + (col & 3u)];
+                    if(gcol < n)
+                        addTo(d + static_cast<size_t>(row) * ldd + gcol, v);
+                }
+            }
+        }
+
+        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks>
+        int launchSliced(GemmArgs const& g, hipStream_t stream, uint32_t slices)
+        {
+            const uint32_t kLen   = g.k / slices;
+            const uint32_t tile   = g.m * kSlicedCols * static_cast<uint32_t>(sizeof(CompT));
+            const uint32_t lds    = g.m * kLen > tile ? g.m * kLen : tile;
+            auto           kernel = gemmSlicedKernel<InT, OutT, CompT, MBlocks>;
+            if(lds > 65536u
+               && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(lds))
+                      != hipSuccess)
+                return ROCWMMA_AMD_LAUNCH_FAILED;
+            const uint32_t quads = g.m * (g.n / 4u);
+            hipLaunchKernelGGL((initOutputKernel<OutT, CompT>), dim3((quads + 255u) / 256u), dim3(256), 0, stream, g.m, g.n,
+                               static_cast<OutT const*>(g.c), g.ldc, static_cast<OutT*>(g.d), g.ldd,
+                               static_cast<CompT>(g.beta));
+            hipLaunchKernelGGL(kernel, dim3((g.n + kSlicedCols - 1u) / kSlicedCols, slices), dim3(64u * kSlicedWaves), lds,
+                               stream, g.m, g.n, g.k, static_cast<InT const*>(g.a), static_cast<InT const*>(g.b),
+                               static_cast<OutT*>(g.d), g.lda, g.ldb, g.ldd, static_cast<CompT>(g.alpha));
+            return launchStatus();
+        }
+
+        template <typename InT, typename OutT, typename CompT>
+        int pickSliced(GemmArgs const& g, hipStream_t stream)
+        {
+            if(g.m % 16u != 0u || g.m >= kSlicedMaxM || g.n % 16u != 0u || g.k % 1024u != 0u)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            // K slices: whole 1 KiB copies per row and whole batches of fragment steps per slice, the
+            // A slice within 128 KiB of LDS; as few slices as fill the compute units
+            const uint32_t groups = (g.n + kSlicedCols - 1u) / kSlicedCols;
+            const uint32_t units  = g.k / 1024u;
+            uint32_t       slices = 0;
+            for(uint32_t s = 1; s <= units; ++s)
+            {
+                if(units % s != 0u || g.m * (g.k / s) > kSkinnyMaxA)
+                    continue;
+                slices = s;
+                if(groups * s >= computeUnits() * 3u / 4u)
+                    break;
+            }
+            if(slices == 0u)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            switch(g.m / 16u)
+            {
+            case 3:
+                return launchSliced<InT, OutT, CompT, 3>(g, stream, slices);
+            case 4:
+                return launchSliced<InT, OutT, CompT, 4>(g, stream, slices);
+            case 5:
+                return launchSliced<InT, OutT, CompT, 5>(g, stream, slices);
+            case 6:
+                return launchSliced<InT, OutT, CompT, 6>(g, stream, slices);
+            case 7:
+                return launchSliced<InT, OutT, CompT, 7>(g, stream, slices);
+            default:
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            }
+        }
+
         template <typename InT, typename OutT, typename CompT>
         int pickShape(GemmArgs const& g, hipStream_t stream)
         {
+            if(g.m > 32u)
+                return pickSliced<InT, OutT, CompT>(g, stream);
             // whole 1 KiB copies per row of A, whole fragment steps per K slice, A resident in LDS
             if(g.m % 16u != 0u || g.m > 32u || g.n % 16u != 0u || g.k % 1024u != 0u || g.m * g.k > kSkinnyMaxA)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;

@@ -264,6 +264,46 @@ def test_skinny_weight_streaming_kernel(dtype_in, m, k):
         check(dtype_in, out, ref, want, tol_for(dtype_in))
 
 
+@pytest.mark.parametrize("m,n,k", [(48, 352, 1024), (64, 352, 2048), (96, 352, 4096), (112, 1040, 2048),
+                                   (64, 14336, 4096)])
+@pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3, orc.E5M2])
+def test_sliced_weight_streaming_kernel(dtype_in, m, n, k):
+    """48..112 token rows, 8-bit, A row / B col, K a multiple of 1024: a K slice of A stays in LDS, the K
+    slices of an output belong to different workgroups and meet in D through atomic adds (AUTO).
+    int8 must be bit-exact; beta != 0 goes through the kernel that initialises D; C may be D."""
+    import torch
+
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(81, orc.I8, m * k), uniform_bits(82, orc.I8, k * n)
+        c = uniform_bits(83, orc.I32, m * n)
+    else:
+        a, b = normal_fp8_bits(81, dtype_in, m * k), normal_fp8_bits(82, dtype_in, k * n)
+        c = np.random.default_rng(83).uniform(-1, 1, m * n).astype(np.float32)
+    out = OUT_OF[dtype_in]
+    for alpha, beta in [(1.0, 0.0), (2.0, -3.0)]:
+        got = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, c, alpha, beta, rw.GEMM_AUTO)
+        want = orc.gemm(dtype_in, out, RM, CM, RM, RM, m, n, k, a, b, c, alpha, beta)
+        check(dtype_in, out, got, want, tol_for(dtype_in))
+    # in place: D holds C
+    d = to_device(c)
+    rw.gemm(dtype_in, out, RM, CM, RM, m, n, k, to_device(a), to_device(b), d, d, 2.0, -3.0)
+    torch.cuda.synchronize()
+    check(dtype_in, out, to_host(d, orc.storage_dtype(out)), want, tol_for(dtype_in))
+
+
+@pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3, orc.E5M2])
+def test_sliced_kernel_exact_integer_pattern(dtype_in):
+    """Integer-valued operands: every partial sum is exact, so the result must match bit for bit
+    whatever order the K slices arrive in."""
+    m, n, k = 64, 512, 4096
+    a, b = exact_int_bits(dtype_in, m, k, RM), exact_int_bits(dtype_in, k, n, CM)
+    out = OUT_OF[dtype_in]
+    c = exact_int_bits(out, m, n, RM)
+    got = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, c, 2.0, 2.0, rw.GEMM_AUTO)
+    want = orc.gemm(dtype_in, out, RM, CM, RM, RM, m, n, k, a, b, c, 2.0, 2.0)
+    assert np.array_equal(got, want)
+
+
 # ---------------------------------------------------------------- config 3: quantised shapes
 @pytest.mark.parametrize("m", [16, 128, 4096])
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3])
