@@ -770,13 +770,7 @@ namespace rocwmma_amd
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             if constexpr(AK && BK)
             {
-                #ifndef NARROW_STAGES
-#define NARROW_STAGES 4
-#endif
-                #ifndef NARROW_WAVES
-#define NARROW_WAVES 1
-#endif
-                using Narrow = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, NARROW_STAGES, NARROW_WAVES>;
+                using Narrow = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 3>;
                 if(g.m % Small::MacroM == 0u && g.n % Small::MacroN == 0u
                    && (g.m / Small::MacroM) * (g.n / Small::MacroN) < computeUnits())
                 {
