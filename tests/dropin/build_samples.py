@@ -7,7 +7,9 @@ the rest of the tree.  tests/test_gpu_reference_samples.py runs them there: each
 validates its own GPU result against its own CPU code and prints PASSED or FAILED.
 
   simple_hgemm, simple_dlrm : compiled as they are, with their own main().
-  simple_sgemv, perf_hgemm  : their host code asks the helper header which device it runs on,
+  simple_sgemv, perf_hgemm, simple_sgemm, perf_sgemm (the two f32 GEMM samples are outside the
+                              workloads this library is built for and come along for free)
+                            : their host code asks the helper header which device it runs on,
                               and that helper (samples/common.hpp:65-80, 113-130) only knows
                               gfx908..gfx942.  The sample is included from a two-line driver that
                               answers "yes" for it and calls the sample's test function (for
@@ -50,6 +52,33 @@ DRIVERS = {
 int main()
 {
     sgemv_test(256, T_BLOCK_Y * ROCWMMA_N, 256, 2.1f, 2.1f);
+    return 0;
+}
+""",
+    "simple_sgemm": """
+#include <rocwmma/rocwmma.hpp>
+#include "common.hpp"
+#define isF32Supported() true
+#define main reference_sample_main
+#include "simple_sgemm.cpp"
+#undef main
+int main()
+{
+    gemm_test(256, 256, 256, 2.1f, 2.1f);
+    return 0;
+}
+""",
+    "perf_sgemm": """
+#include <rocwmma/rocwmma.hpp>
+#include "common.hpp"
+#define isF32Supported() true
+#define isGfx9() true
+#define main reference_sample_main
+#include "perf_sgemm.cpp"
+#undef main
+int main()
+{
+    gemm_test(1024, 1024, 1024, 2, 2);
     return 0;
 }
 """,
