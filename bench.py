@@ -200,10 +200,26 @@ def main():
 
 
 def run_extras(rw, torch, dev, gen, args):
-    """Quantised GEMMs (config 3), GEMV (config 4), DLRM (config 5): kernel time by events."""
+    """The small GEMM (config 1), quantised GEMMs (config 3), GEMV (config 4), DLRM (config 5): kernel
+    time by events."""
     RM, CM = rw.ROW_MAJOR, rw.COL_MAJOR
     out = {}
     iters = 20
+
+    # config 1: 256^3 f16 -> f32, A row / B col, alpha = beta = 2: launch latency, reported only
+    m1 = 256
+    A1 = (torch.rand(m1 * m1, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+    B1 = (torch.rand(m1 * m1, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+    C1 = torch.rand(m1 * m1, device=dev, generator=gen) * 2 - 1
+    D1 = torch.empty(m1 * m1, device=dev)
+    for tag, algo in (("wave_tile", rw.GEMM_WAVE_TILE), ("blocked", rw.GEMM_BLOCKED)):
+        def fn1():
+            rw.gemm(rw.F16, rw.F32, RM, CM, RM, m1, m1, m1, A1, B1, C1, D1, 2.0, 2.0, algo=algo)
+
+        fn1()
+        ms = event_ms(fn1, 100, torch)
+        out[f"gemm_f16_256cubed_{tag}"] = {"us": round(ms * 1e3, 2), "tflops": round(2.0 * m1 ** 3 / ms / 1e9, 2),
+                                           "note": "back-to-back launches, launch-latency bound"}
 
     # config 3: N = 14336, K = 4096, M in {16, 128, 4096}; int8 and e4m3, A row / B col.  The weight
     # matrix (56 MiB) would stay in the 256 MiB Infinity Cache between launches, so the timed loop
