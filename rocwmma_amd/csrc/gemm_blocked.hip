@@ -779,7 +779,20 @@ namespace rocwmma_amd
                         return rc;
                 }
             }
-            return launchCfg<Small>(g, stream);
+            {
+                int rc = launchCfg<Small>(g, stream);
+                if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                    return rc;
+            }
+            // multiples of 64 that are not multiples of 128: 64 x 64 tiles, one 32 x 32 block per wave
+            // (K-contiguous operands only: the dim-major LDS tile is at least 128 wide)
+            if constexpr(AK && BK)
+            {
+                using Tiny = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 1, 4, 4>;
+                return launchCfg<Tiny>(g, stream);
+            }
+            else
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
         }
 
         template <typename InT, typename OutT, typename CompT>

@@ -265,7 +265,7 @@ def test_skinny_weight_streaming_kernel(dtype_in, m, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(48, 352, 1024), (64, 352, 2048), (96, 352, 4096), (112, 1040, 2048),
-                                   (64, 14336, 4096)])
+                                   (80, 14336, 4096)])
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3, orc.E5M2])
 def test_sliced_weight_streaming_kernel(dtype_in, m, n, k):
     """48..112 token rows, 8-bit, A row / B col, K a multiple of 1024: a K slice of A stays in LDS, the K
@@ -302,6 +302,31 @@ def test_sliced_kernel_exact_integer_pattern(dtype_in):
     got = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, c, 2.0, 2.0, rw.GEMM_AUTO)
     want = orc.gemm(dtype_in, out, RM, CM, RM, RM, m, n, k, a, b, c, 2.0, 2.0)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 192, 512), (192, 64, 256), (320, 448, 256), (64, 14336, 4096)])
+@pytest.mark.parametrize("dtype_in,dtype_out", [(orc.F16, orc.F32), (orc.BF16, orc.BF16), (orc.I8, orc.I32),
+                                                (orc.E4M3, orc.F32)])
+def test_blocked_kernel_64x64_tiles(dtype_in, dtype_out, m, n, k):
+    """Multiples of 64 that are not multiples of 128 (K-contiguous operands) run on the blocked
+    kernel's 64 x 64 tile configuration instead of the wave-tile kernel."""
+    if m * n * k > 1 << 30 and dtype_in not in (orc.I8, orc.F16):
+        pytest.skip("full-size shape: one 16-bit and one 8-bit type")
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(91, orc.I8, m * k), uniform_bits(92, orc.I8, k * n)
+        c = uniform_bits(93, orc.I32, m * n)
+    elif dtype_in == orc.E4M3:
+        a, b = normal_fp8_bits(91, dtype_in, m * k), normal_fp8_bits(92, dtype_in, k * n)
+        c = np.random.default_rng(93).uniform(-1, 1, m * n).astype(np.float32)
+    else:
+        a, b = uniform_bits(91, dtype_in, m * k), uniform_bits(92, dtype_in, k * n)
+        c = (uniform_bits(93, dtype_out, m * n) if dtype_out != orc.F32
+             else np.random.default_rng(93).uniform(-1, 1, m * n).astype(np.float32))
+    tol = 4e-3 if dtype_out == orc.BF16 else tol_for(dtype_in)
+    for alpha, beta in [(1.0, 0.0), (2.0, -1.0)]:
+        got = run_gemm(dtype_in, dtype_out, RM, CM, RM, m, n, k, a, b, c, alpha, beta, rw.GEMM_BLOCKED)
+        want = orc.gemm(dtype_in, dtype_out, RM, CM, RM, RM, m, n, k, a, b, c, alpha, beta)
+        check(dtype_in, dtype_out, got, want, tol)
 
 
 # ---------------------------------------------------------------- config 3: quantised shapes
