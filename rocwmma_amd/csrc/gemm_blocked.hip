@@ -737,8 +737,8 @@ namespace rocwmma_amd
         }
 
         // Tile ladder: the 256 x 256 macro tile when the problem divides into enough of them to occupy
-        // at least half of the compute units, else 128 x 128; when even that leaves compute units
-        // without a tile (few token rows against a wide weight matrix), 128 x 64 tiles double the
+        // at least half of the compute units, else 128 x 128; when that gives at most one tile per two
+        // compute units (few token rows against a wide weight matrix), 128 x 64 tiles double the
         // number of workgroups.
         template <typename InT, typename OutT, typename CompT, bool AK, bool BK>
         int pickTile(GemmArgs const& g, hipStream_t stream, bool forceLargeTile)
@@ -771,8 +771,11 @@ namespace rocwmma_amd
             if constexpr(AK && BK)
             {
                 using Narrow = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 3>;
+                // (up to one 128 x 128 tile per two compute units; with two resident workgroups per
+                // compute unit the 128 x 128 tiling wins from 144 tiles on, fewer bytes per compute
+                // unit: 256 x 14336 x 4096 int8 30 -> 24 us, f16 73 -> 52 us)
                 if(g.m % Small::MacroM == 0u && g.n % Small::MacroN == 0u
-                   && (g.m / Small::MacroM) * (g.n / Small::MacroN) < computeUnits())
+                   && 2u * (g.m / Small::MacroM) * (g.n / Small::MacroN) <= computeUnits())
                 {
                     int rc = launchCfg<Narrow>(g, stream);
                     if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
