@@ -770,6 +770,17 @@ namespace rocwmma_amd
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             if constexpr(AK && BK)
             {
+                // small problems, at most one 128 x 128 tile per four compute units: 64 x 64 tiles put
+                // four times as many workgroups to work (512 x 512 x 4096 int8 13 -> 11 us,
+                // 256 x 256 x 8192 f16 45 -> 40 us)
+                using Tiny0 = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 1, 4, 4>;
+                if(g.m % Small::MacroM == 0u && g.n % Small::MacroN == 0u
+                   && 4u * (g.m / Small::MacroM) * (g.n / Small::MacroN) <= computeUnits())
+                {
+                    int rc = launchCfg<Tiny0>(g, stream);
+                    if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                        return rc;
+                }
                 using Narrow = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 3>;
                 // (up to one 128 x 128 tile per two compute units; with two resident workgroups per
                 // compute unit the 128 x 128 tiling wins from 144 tiles on, fewer bytes per compute

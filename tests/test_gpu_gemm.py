@@ -329,6 +329,24 @@ def test_blocked_kernel_64x64_tiles(dtype_in, dtype_out, m, n, k):
         check(dtype_in, dtype_out, got, want, tol)
 
 
+@pytest.mark.parametrize("m,n", [(256, 256), (1024, 1152), (1536, 1536)])
+@pytest.mark.parametrize("dtype_in", [orc.F16, orc.I8, orc.E4M3])
+def test_blocked_kernel_tile_ladder(dtype_in, m, n):
+    """K-contiguous operands through every rung below the 256 x 256 tile on a 256-unit device:
+    4 tiles of 128 x 128 -> 64 x 64 tiles, 72 -> 128 x 64, 144 -> 128 x 128."""
+    k = 256
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(61, orc.I8, m * k), uniform_bits(62, orc.I8, k * n)
+    elif dtype_in == orc.E4M3:
+        a, b = normal_fp8_bits(61, dtype_in, m * k), normal_fp8_bits(62, dtype_in, k * n)
+    else:
+        a, b = uniform_bits(61, dtype_in, m * k), uniform_bits(62, dtype_in, k * n)
+    out = OUT_OF[dtype_in]
+    got = run_gemm(dtype_in, out, RM, CM, RM, m, n, k, a, b, None, 1.0, 0.0, rw.GEMM_BLOCKED)
+    want = orc.gemm(dtype_in, out, RM, CM, RM, RM, m, n, k, a, b, None, 1.0, 0.0)
+    check(dtype_in, out, got, want, tol_for(dtype_in))
+
+
 # ---------------------------------------------------------------- config 3: quantised shapes
 @pytest.mark.parametrize("m", [16, 128, 4096])
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3])
