@@ -1,12 +1,12 @@
-// Skinny quantised GEMM: D = alpha * A * B + beta * C for M <= 32 token rows against an
-// N x K weight matrix (8-bit A row-major, B col-major, C/D row-major), and a K-sliced variant
-// for 48..112 token rows further down.
+// Skinny GEMM: D = alpha * A * B + beta * C for M <= 32 token rows against an N x K weight
+// matrix (8-bit or 16-bit A row-major, B col-major, 32-bit C/D row-major), and a K-sliced variant
+// further down for more token rows (up to 112) or when A does not fit the LDS whole.
 //
 // At these shapes (the reference's GEMM kernels, samples/perf_hgemm.cpp:518-714, need whole
 // 128-wide macro tiles in M and would leave most of the chip idle) the job is streaming the
 // weights from HBM exactly once, so the kernel is built for memory-level parallelism:
 //   * a workgroup of 16 waves = 4 blocks of 16 weight rows x 4 slices of K; every wave walks
-//     its K slice of its weight rows in 128-byte steps with 16 x 16 x 128 fragments loaded
+//     its K slice of its weight rows in 128-byte steps with 16 x 16 x 128 (16-bit: x 64) fragments loaded
 //     straight from global memory (one v_mfma_f32_16x16x128_f8f6f4, or two
 //     v_mfma_i32_16x16x64_i8, per step), several steps in flight;
 //   * the token matrix A is copied into LDS once per workgroup (direct-to-LDS copies, 16-byte
@@ -27,7 +27,7 @@ namespace rocwmma_amd
         constexpr uint32_t kSkinnySlices = 4;   // K slices per block of weight rows
         constexpr uint32_t kSkinnyBlocks = 4;   // blocks of 16 weight rows per workgroup
         constexpr uint32_t kSkinnyWaves  = kSkinnySlices * kSkinnyBlocks;
-        constexpr uint32_t kSkinnyK      = 128; // K elements (= bytes) per fragment step
+        constexpr uint32_t kSkinnyKBytes = 128; // bytes of K per fragment step (128 8-bit or 64 16-bit elements)
         constexpr uint32_t kSkinnyMaxA   = 131072; // bytes of LDS the token matrix may take
 
         template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t Ahead>
@@ -45,18 +45,20 @@ namespace rocwmma_amd
                                                                               CompT       alpha,
                                                                               CompT       beta)
         {
+            constexpr uint32_t E       = sizeof(InT); // bytes per element
+            constexpr uint32_t kSkinnyK = kSkinnyKBytes / E; // K elements per fragment step
             using FragA   = fragment<matrix_a, 16, 16, kSkinnyK, InT, row_major>;
             using FragB   = fragment<matrix_b, 16, 16, kSkinnyK, InT, col_major>;
             using FragAcc = fragment<accumulator, 16, 16, kSkinnyK, CompT>;
             using FragC   = fragment<accumulator, 16, 16, kSkinnyK, OutT, row_major>;
             using MapA    = detail::InputMap<16, kSkinnyK, 16, detail::packClassOf<InT>()>;
-            static_assert(sizeof(InT) == 1, "8-bit operands");
+            static_assert(sizeof(InT) <= 2, "8- and 16-bit operands");
 
             extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
-            char* aTile = ldsRaw; // [m][k] bytes, chunk c of row r at chunk position c ^ (r % 16)
+            char* aTile = ldsRaw; // [m][k * E] bytes, chunk c of row r at chunk position c ^ (r % 16)
             // partial[wave][mblock][lane] : the 4 accumulator registers of a lane as one 16-byte unit
             using Quad    = CompT __attribute__((ext_vector_type(4)));
-            Quad* partial = reinterpret_cast<Quad*>(ldsRaw + m * k);
+            Quad* partial = reinterpret_cast<Quad*>(ldsRaw + m * k * E);
 
             const uint32_t lane   = threadIdx.x & 63u;
             const uint32_t wave   = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -70,14 +72,15 @@ namespace rocwmma_amd
 
             // A -> LDS: whole-wave 1 KiB copies, k / 1024 per row
             {
-                const uint32_t perRow = k / 1024u;
+                const uint32_t perRow = k * E / 1024u;
                 const uint32_t copies = m * perRow;
                 for(uint32_t j = wave; j < copies; j += kSkinnyWaves)
                 {
                     const uint32_t r   = j / perRow;
                     const uint32_t pos = (j % perRow) * 64u + lane; // chunk position inside the LDS row
-                    lds::asyncCopy16(aTile + r * k + (j % perRow) * 1024u,
-                                     reinterpret_cast<const char*>(a) + static_cast<size_t>(r) * lda + ((pos ^ (r & 15u)) << 4));
+                    lds::asyncCopy16(aTile + r * k * E + (j % perRow) * 1024u,
+                                     reinterpret_cast<const char*>(a) + static_cast<size_t>(r) * lda * E
+                                         + ((pos ^ (r & 15u)) << 4));
                 }
             }
 
@@ -106,11 +109,12 @@ namespace rocwmma_amd
 #pragma unroll
                         for(uint32_t ch = 0; ch < MapA::nchunks; ++ch)
 #pragma unroll
-                            for(uint32_t piece = 0; piece < MapA::kpack / 16u; ++piece)
+                            for(uint32_t piece = 0; piece < MapA::kpack * E / 16u; ++piece)
                             {
-                                const uint32_t kByte = kBeg + kk + u * kSkinnyK + MapA::chunkK(ch, lane) + piece * 16u;
-                                detail::copyBytes<16u>(fa.x + ch * MapA::kpack + piece * 16u,
-                                                       aTile + row * k + (((kByte >> 4) ^ (row & 15u)) << 4));
+                                const uint32_t kByte
+                                    = (kBeg + kk + u * kSkinnyK + MapA::chunkK(ch, lane)) * E + piece * 16u;
+                                detail::copyBytes<16u>(fa.x + ch * MapA::kpack + piece * (16u / E),
+                                                       aTile + row * k * E + (((kByte >> 4) ^ (row & 15u)) << 4));
                             }
                         mma_sync(acc[i], fa, fb[u], acc[i]);
                     }
@@ -169,7 +173,7 @@ namespace rocwmma_amd
         template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t Ahead>
         int launchOne(GemmArgs const& g, hipStream_t stream)
         {
-            const uint32_t lds    = g.m * g.k + kSkinnyWaves * MBlocks * 1024u;
+            const uint32_t lds    = g.m * g.k * static_cast<uint32_t>(sizeof(InT)) + kSkinnyWaves * MBlocks * 1024u;
             auto           kernel = gemmSkinnyKernel<InT, OutT, CompT, MBlocks, Ahead>;
             if(lds > 65536u
                && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -246,15 +250,17 @@ namespace rocwmma_amd
                                                                               uint32_t   ldd,
                                                                               CompT      alpha)
         {
+            constexpr uint32_t E       = sizeof(InT); // bytes per element
+            constexpr uint32_t kSkinnyK = kSkinnyKBytes / E; // K elements per fragment step
             using FragA   = fragment<matrix_a, 16, 16, kSkinnyK, InT, row_major>;
             using FragB   = fragment<matrix_b, 16, 16, kSkinnyK, InT, col_major>;
             using FragAcc = fragment<accumulator, 16, 16, kSkinnyK, CompT>;
             using MapA    = detail::InputMap<16, kSkinnyK, 16, detail::packClassOf<InT>()>;
-            static_assert(sizeof(InT) == 1 && std::is_same<OutT, CompT>::value, "8-bit operands, 32-bit results");
+            static_assert(sizeof(InT) <= 2 && std::is_same<OutT, CompT>::value, "8- or 16-bit operands, 32-bit results");
             constexpr uint32_t Ahead = kSlicedAhead;
 
             extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
-            char* aTile = ldsRaw; // [m][kLen] bytes, chunk c of row r at chunk position c ^ (r % 16)
+            char* aTile = ldsRaw; // [m][kLen * E] bytes, chunk c of row r at chunk position c ^ (r % 16)
 
             const uint32_t lane   = threadIdx.x & 63u;
             const uint32_t wave   = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -285,14 +291,14 @@ namespace rocwmma_amd
 
             // A slice -> LDS: whole-wave 1 KiB copies, kLen / 1024 per row
             {
-                const uint32_t perRow = kLen / 1024u;
+                const uint32_t perRow = kLen * E / 1024u;
                 const uint32_t copies = m * perRow;
                 for(uint32_t j = wave; j < copies; j += kSlicedWaves)
                 {
                     const uint32_t r   = j / perRow;
                     const uint32_t pos = (j % perRow) * 64u + lane; // chunk position inside the LDS row
-                    lds::asyncCopy16(aTile + r * kLen + (j % perRow) * 1024u,
-                                     reinterpret_cast<const char*>(a) + static_cast<size_t>(r) * lda + kBeg
+                    lds::asyncCopy16(aTile + r * kLen * E + (j % perRow) * 1024u,
+                                     reinterpret_cast<const char*>(a) + (static_cast<size_t>(r) * lda + kBeg) * E
                                          + ((pos ^ (r & 15u)) << 4));
                 }
             }
@@ -315,11 +321,11 @@ namespace rocwmma_amd
 #pragma unroll
                         for(uint32_t ch = 0; ch < MapA::nchunks; ++ch)
 #pragma unroll
-                            for(uint32_t piece = 0; piece < MapA::kpack / 16u; ++piece)
+                            for(uint32_t piece = 0; piece < MapA::kpack * E / 16u; ++piece)
                             {
-                                const uint32_t kByte = kk + u * kSkinnyK + MapA::chunkK(ch, lane) + piece * 16u;
-                                detail::copyBytes<16u>(fa.x + ch * MapA::kpack + piece * 16u,
-                                                       aTile + row * kLen + (((kByte >> 4) ^ (row & 15u)) << 4));
+                                const uint32_t kByte = (kk + u * kSkinnyK + MapA::chunkK(ch, lane)) * E + piece * 16u;
+                                detail::copyBytes<16u>(fa.x + ch * MapA::kpack + piece * (16u / E),
+                                                       aTile + row * kLen * E + (((kByte >> 4) ^ (row & 15u)) << 4));
                             }
 #pragma unroll
                         for(uint32_t j = 0; j < NB; ++j)
@@ -372,9 +378,9 @@ namespace rocwmma_amd
         template <typename InT, typename OutT, typename CompT, uint32_t MBlocks>
         int launchSliced(GemmArgs const& g, hipStream_t stream, uint32_t slices)
         {
-            const uint32_t kLen   = g.k / slices;
+            const uint32_t slice  = g.m * (g.k / slices) * static_cast<uint32_t>(sizeof(InT)); // bytes of A per slice
             const uint32_t tile   = g.m * kSlicedCols * static_cast<uint32_t>(sizeof(CompT));
-            const uint32_t lds    = g.m * kLen > tile ? g.m * kLen : tile;
+            const uint32_t lds    = slice > tile ? slice : tile;
             auto           kernel = gemmSlicedKernel<InT, OutT, CompT, MBlocks>;
             if(lds > 65536u
                && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -394,7 +400,8 @@ namespace rocwmma_amd
         template <typename InT, typename OutT, typename CompT>
         int pickSliced(GemmArgs const& g, hipStream_t stream)
         {
-            if(g.m % 16u != 0u || g.m >= kSlicedMaxM || g.n % 16u != 0u || g.k % 1024u != 0u)
+            constexpr uint32_t E = sizeof(InT);
+            if(g.m % 16u != 0u || g.m >= kSlicedMaxM || g.n % 16u != 0u || (g.k * E) % 1024u != 0u)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             // 64 rows against a multiple of 64 columns: the blocked kernel's 64 x 64 tiles are as fast
             // (24 against 25 us at 64 x 14336 x 4096), in one launch and without atomic adds
@@ -403,11 +410,11 @@ namespace rocwmma_amd
             // K slices: whole 1 KiB copies per row and whole batches of fragment steps per slice, the
             // A slice within 128 KiB of LDS; as few slices as fill the compute units
             const uint32_t groups = (g.n + kSlicedCols - 1u) / kSlicedCols;
-            const uint32_t units  = g.k / 1024u;
+            const uint32_t units  = g.k * E / 1024u;
             uint32_t       slices = 0;
             for(uint32_t s = 1; s <= units; ++s)
             {
-                if(units % s != 0u || g.m * (g.k / s) > kSkinnyMaxA)
+                if(units % s != 0u || g.m * (g.k / s) * E > kSkinnyMaxA)
                     continue;
                 slices = s;
                 if(groups * s >= computeUnits() * 3u / 4u)
@@ -417,6 +424,10 @@ namespace rocwmma_amd
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             switch(g.m / 16u)
             {
+            case 1: // (16 and 32 rows come here only when all of A does not fit the LDS)
+                return launchSliced<InT, OutT, CompT, 1>(g, stream, slices);
+            case 2:
+                return launchSliced<InT, OutT, CompT, 2>(g, stream, slices);
             case 3:
                 return launchSliced<InT, OutT, CompT, 3>(g, stream, slices);
             case 4:
@@ -435,13 +446,14 @@ namespace rocwmma_amd
         template <typename InT, typename OutT, typename CompT>
         int pickShape(GemmArgs const& g, hipStream_t stream)
         {
-            if(g.m > 32u)
+            constexpr uint32_t E = sizeof(InT);
+            if(g.m > 32u || g.m * g.k * E > kSkinnyMaxA)
                 return pickSliced<InT, OutT, CompT>(g, stream);
             // whole 1 KiB copies per row of A, whole fragment steps per K slice, A resident in LDS
-            if(g.m % 16u != 0u || g.m > 32u || g.n % 16u != 0u || g.k % 1024u != 0u || g.m * g.k > kSkinnyMaxA)
+            if(g.m % 16u != 0u || g.n % 16u != 0u || (g.k * E) % 1024u != 0u)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             // K steps of a wave's slice fetched together: as many as divide the slice, up to 8
-            const uint32_t steps = g.k / (kSkinnySlices * kSkinnyK);
+            const uint32_t steps = g.k * E / (kSkinnySlices * kSkinnyKBytes);
             if(g.m == 16u)
             {
                 if(steps % 8u == 0u)
@@ -468,6 +480,10 @@ namespace rocwmma_amd
             return pickShape<float8_t, float32_t, float32_t>(g, stream);
         if(dtypeIn == ROCWMMA_AMD_E5M2 && dtypeOut == ROCWMMA_AMD_F32)
             return pickShape<bfloat8_t, float32_t, float32_t>(g, stream);
+        if(dtypeIn == ROCWMMA_AMD_F16 && dtypeOut == ROCWMMA_AMD_F32)
+            return pickShape<float16_t, float32_t, float32_t>(g, stream);
+        if(dtypeIn == ROCWMMA_AMD_BF16 && dtypeOut == ROCWMMA_AMD_F32)
+            return pickShape<bfloat16_t, float32_t, float32_t>(g, stream);
         return ROCWMMA_AMD_UNSUPPORTED_TYPE;
     }
 

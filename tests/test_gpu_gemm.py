@@ -347,6 +347,30 @@ def test_blocked_kernel_tile_ladder(dtype_in, m, n):
     check(dtype_in, out, got, want, tol_for(dtype_in))
 
 
+@pytest.mark.parametrize("m,n,k", [(16, 352, 2048), (16, 14336, 4096), (32, 352, 2048), (32, 352, 4096),
+                                   (48, 1040, 1536), (80, 352, 4096), (112, 352, 1024)])
+@pytest.mark.parametrize("dtype_in", [orc.F16, orc.BF16])
+def test_skinny_and_sliced_kernels_16bit(dtype_in, m, n, k):
+    """The weight-streaming kernels also take f16 / bf16 operands (f32 results): all of A in LDS
+    while m * k * 2 <= 128 KiB, K slices over workgroups beyond that (AUTO); beta != 0 and C = D."""
+    import torch
+
+    a, b = uniform_bits(51, dtype_in, m * k), uniform_bits(52, dtype_in, k * n)
+    c = np.random.default_rng(53).uniform(-1, 1, m * n).astype(np.float32)
+    for alpha, beta in [(1.0, 0.0), (2.0, -3.0)]:
+        got = run_gemm(dtype_in, orc.F32, RM, CM, RM, m, n, k, a, b, c, alpha, beta, rw.GEMM_AUTO)
+        want = orc.gemm(dtype_in, orc.F32, RM, CM, RM, RM, m, n, k, a, b, c, alpha, beta)
+        check(dtype_in, orc.F32, got, want, 1e-3)
+    d = to_device(c)
+    rw.gemm(dtype_in, orc.F32, RM, CM, RM, m, n, k, to_device(a), to_device(b), d, d, 2.0, -3.0)
+    torch.cuda.synchronize()
+    check(dtype_in, orc.F32, to_host(d, np.float32), want, 1e-3)
+    # integer-valued operands: exact whatever the summation order
+    ai, bi = exact_int_bits(dtype_in, m, k, RM), exact_int_bits(dtype_in, k, n, CM)
+    got = run_gemm(dtype_in, orc.F32, RM, CM, RM, m, n, k, ai, bi, None, 1.0, 0.0, rw.GEMM_AUTO)
+    assert np.array_equal(got, orc.gemm(dtype_in, orc.F32, RM, CM, RM, RM, m, n, k, ai, bi, None, 1.0, 0.0))
+
+
 # ---------------------------------------------------------------- config 3: quantised shapes
 @pytest.mark.parametrize("m", [16, 128, 4096])
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3])
