@@ -793,6 +793,20 @@ namespace rocwmma_amd
                         return rc;
                 }
             }
+            else if constexpr(AK != BK)
+            {
+                // one operand dim-major: its LDS tile is at least 128 wide, the other side may be 64
+                // (128 x 64 tiles with a K-contiguous B, 64 x 128 with a K-contiguous A)
+                using Half = std::conditional_t<BK, BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 3>,
+                                                BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 2, 4, 3>>;
+                if(g.m % Small::MacroM == 0u && g.n % Small::MacroN == 0u
+                   && 2u * (g.m / Small::MacroM) * (g.n / Small::MacroN) <= computeUnits())
+                {
+                    int rc = launchCfg<Half>(g, stream);
+                    if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                        return rc;
+                }
+            }
             {
                 int rc = launchCfg<Small>(g, stream);
                 if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
