@@ -401,7 +401,8 @@ namespace rocwmma_amd
         int pickSliced(GemmArgs const& g, hipStream_t stream)
         {
             constexpr uint32_t E = sizeof(InT);
-            if(g.m % 16u != 0u || g.m >= kSlicedMaxM || g.n % 16u != 0u || (g.k * E) % 1024u != 0u)
+            // (n: the kernel that initialises D counts 4-element groups in 32 bits)
+            if(g.m % 16u != 0u || g.m >= kSlicedMaxM || g.n % 16u != 0u || g.n > (1u << 24) || (g.k * E) % 1024u != 0u)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             // 64 rows against a multiple of 64 columns: the blocked kernel's 64 x 64 tiles are as fast
             // (24 against 25 us at 64 x 14336 x 4096), in one launch and without atomic adds
