@@ -96,3 +96,14 @@ def test_product_code_never_touches_the_oracle():
                 if fn.endswith((".py", ".hip", ".hpp", ".h", ".cpp")):
                     text = open(os.path.join(dirpath, fn), errors="ignore").read()
                     assert "liboracle" not in text and "import oracle" not in text, os.path.join(dirpath, fn)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more exits with a message instead of running."""
+    import subprocess
+    import sys
+
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                         stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert res.returncode != 0
+    assert "one GPU" in res.stdout
