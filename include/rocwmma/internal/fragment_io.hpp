@@ -2,7 +2,7 @@
 //
 // A fragment is a sequence of "items": for input fragments an item is one MFMA operand
 // (kpack elements contiguous in K, see fragment_map.hpp); for accumulators an item is a run
-// of four consecutive columns of one row.  Items whose elements are contiguous in memory
+// of four consecutive columns of one row (a single element for 64-bit accumulators).  Items whose elements are contiguous in memory
 // (K-contiguous operands; row-major accumulators) move as one 2..32-byte vector access,
 // the others element by element.
 //
@@ -103,7 +103,7 @@ namespace rocwmma
         struct AccIO
         {
             static constexpr uint32_t Items     = Map::nruns;
-            static constexpr uint32_t ItemElems = 4u;
+            static constexpr uint32_t ItemElems = Map::runLen; // 4 (1 for 64-bit accumulators)
 
             template <uint32_t Count>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void

@@ -31,7 +31,8 @@
 //                                                  col = bj*16 + (lane/16)*4 + i
 //        tile 32: e = (bi * nbj + bj) * 16 + i     row = bi*32 + lane%32
 //                                                  col = bj*32 + 8*(i/4) + (lane/32)*4 + i%4
-//    Row-major C/D tiles therefore move with 16-byte vector accesses.
+//    Row-major C/D tiles therefore move with 16-byte vector accesses.  (64-bit accumulators differ:
+//    see AccMapStrided.)
 #ifndef ROCWMMA_FRAGMENT_MAP_HPP
 #define ROCWMMA_FRAGMENT_MAP_HPP
 
@@ -170,6 +171,7 @@ namespace rocwmma
             static constexpr uint32_t nbi      = BlockM / Tile;
             static constexpr uint32_t nbj      = BlockN / tileN;
             static constexpr uint32_t perBlock = Tile * tileN / kWaveSize; // 4 or 16
+            static constexpr uint32_t runLen   = 4u; // consecutive columns a lane holds per run
             static constexpr uint32_t runs     = perBlock / 4u; // 4-column runs per block per lane
             static constexpr uint32_t nruns    = nbi * nbj * runs;
             static constexpr uint32_t size     = nbi * nbj * perBlock;
@@ -195,6 +197,48 @@ namespace rocwmma
             static constexpr uint32_t colOf(uint32_t e, uint32_t lane)
             {
                 return runCol(e / 4u, lane) + e % 4u;
+            }
+        };
+
+        // Accumulators of 64-bit elements.  v_mfma_f64_16x16x4_f64 spreads a lane's four results over
+        // rows (lane / 16) + 4 i of the instruction's result, not over four consecutive ones, so with
+        // the multiplicands swapped as for the other types a lane owns row lane % 16 and the columns
+        // (lane / 16) + 4 i of each 16 x 16 tile: runs of one element.  Blocks of any multiple of 16 are
+        // tiled with 16 x 16 tiles (there is no 32-wide f64 instruction).
+        template <uint32_t BlockM, uint32_t BlockN>
+        struct AccMapStrided
+        {
+            static constexpr uint32_t tile  = 16u;
+            static constexpr uint32_t tileN = 16u;
+            static_assert(BlockM % 16u == 0u && BlockN % 16u == 0u, "accumulator block must be a multiple of 16 x 16");
+
+            static constexpr uint32_t nbi      = BlockM / 16u;
+            static constexpr uint32_t nbj      = BlockN / 16u;
+            static constexpr uint32_t perBlock = 4u;
+            static constexpr uint32_t runLen   = 1u;
+            static constexpr uint32_t runs     = 4u;
+            static constexpr uint32_t nruns    = nbi * nbj * runs;
+            static constexpr uint32_t size     = nbi * nbj * perBlock;
+
+            static constexpr uint32_t blockIndex(uint32_t bi, uint32_t bj)
+            {
+                return bi * nbj + bj;
+            }
+            static constexpr uint32_t runRow(uint32_t r, uint32_t lane)
+            {
+                return ((r / runs) / nbj) * 16u + lane % 16u;
+            }
+            static constexpr uint32_t runCol(uint32_t r, uint32_t lane)
+            {
+                return ((r / runs) % nbj) * 16u + lane / 16u + 4u * (r % runs);
+            }
+            static constexpr uint32_t rowOf(uint32_t e, uint32_t lane)
+            {
+                return runRow(e, lane);
+            }
+            static constexpr uint32_t colOf(uint32_t e, uint32_t lane)
+            {
+                return runCol(e, lane);
             }
         };
 

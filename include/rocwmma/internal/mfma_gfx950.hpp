@@ -22,6 +22,7 @@
 //   i8     32    8      v_mfma_i32_32x32x16_i8               16
 //   f32    16    1      v_mfma_f32_16x16x4_f32               4
 //   f32    32    1      v_mfma_f32_32x32x2_f32               2
+//   f64    16    1      v_mfma_f64_16x16x4_f64               4   (results strided over rows: AccMapStrided)
 #ifndef ROCWMMA_MFMA_GFX950_HPP
 #define ROCWMMA_MFMA_GFX950_HPP
 
@@ -42,6 +43,8 @@ namespace rocwmma
         typedef float    f32x16_t __attribute__((ext_vector_type(16), may_alias));
         typedef long     i64x1_t __attribute__((may_alias));
         typedef float    f32x1_t __attribute__((may_alias));
+        typedef double   f64x1_t __attribute__((may_alias));
+        typedef double   f64x4_t __attribute__((ext_vector_type(4), may_alias));
 
         // Accumulator register block of one MFMA: 4 (16x16) or 16 (32x32) values.
         template <typename AccT, uint32_t Tile>
@@ -60,6 +63,11 @@ namespace rocwmma
         struct AccRegs<int32_t, 16>
         {
             using type = i32x4_t;
+        };
+        template <>
+        struct AccRegs<double, 16>
+        {
+            using type = f64x4_t;
         };
         template <>
         struct AccRegs<int32_t, 32>
@@ -130,6 +138,7 @@ namespace rocwmma
 
         ROCWMMA_MFMA_ENTRY(F32, F32, float, 16, 1, f32x1_t, __builtin_amdgcn_mfma_f32_16x16x4f32(X, Y, acc, 0, 0, 0))
         ROCWMMA_MFMA_ENTRY(F32, F32, float, 32, 1, f32x1_t, __builtin_amdgcn_mfma_f32_32x32x2f32(X, Y, acc, 0, 0, 0))
+        ROCWMMA_MFMA_ENTRY(F64, F64, double, 16, 1, f64x1_t, __builtin_amdgcn_mfma_f64_16x16x4f64(X, Y, acc, 0, 0, 0))
 
         // Wide-K fp8 family: one opcode, operand formats chosen by cbsz / blgp, scales unused
         // (scale operands of 0 select the unscaled form of the instruction).

@@ -59,7 +59,8 @@ namespace rocwmma
             F8, // E4M3
             BF8, // E5M2
             I8,
-            F32
+            F32,
+            F64
         };
 
         template <typename T>
@@ -103,6 +104,11 @@ namespace rocwmma
         struct TypeInfo<float32_t>
         {
             static constexpr MmaClass cls = MmaClass::F32;
+        };
+        template <>
+        struct TypeInfo<float64_t>
+        {
+            static constexpr MmaClass cls = MmaClass::F64;
         };
 
         // Plain register words used to move fragments without caring about element type.

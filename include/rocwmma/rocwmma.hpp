@@ -120,6 +120,14 @@ namespace rocwmma
             }
         }
 
+        // MFMA tile edge of an input fragment: 64-bit elements only have the 16 x 16 x 4 instruction
+        template <typename DataT>
+        constexpr uint32_t fragTileDim(uint32_t blockM, uint32_t blockN, uint32_t blockDim)
+        {
+            const uint32_t t = inputTileDim(blockM, blockN, blockDim);
+            return sizeof(DataT) == 8u && t == 32u ? 16u : t;
+        }
+
         // Binds fragment template parameters to a register map and its movers.
         template <typename MatrixT, uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT>
         struct FragConfig;
@@ -127,7 +135,7 @@ namespace rocwmma
         template <uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT>
         struct FragConfig<matrix_a, BlockM, BlockN, BlockK, DataT>
         {
-            using Map = InputMap<BlockM, BlockK, inputTileDim(BlockM, BlockN, BlockM), packClassOf<DataT>()>;
+            using Map = InputMap<BlockM, BlockK, fragTileDim<DataT>(BlockM, BlockN, BlockM), packClassOf<DataT>()>;
             // K runs along a row of A
             template <typename Layout>
             using IO = InputIO<Map, DataT, std::is_same<Layout, row_major>::value>;
@@ -135,7 +143,7 @@ namespace rocwmma
         template <uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT>
         struct FragConfig<matrix_b, BlockM, BlockN, BlockK, DataT>
         {
-            using Map = InputMap<BlockN, BlockK, inputTileDim(BlockM, BlockN, BlockN), packClassOf<DataT>()>;
+            using Map = InputMap<BlockN, BlockK, fragTileDim<DataT>(BlockM, BlockN, BlockN), packClassOf<DataT>()>;
             // K runs along a column of B
             template <typename Layout>
             using IO = InputIO<Map, DataT, std::is_same<Layout, col_major>::value>;
@@ -143,7 +151,10 @@ namespace rocwmma
         template <uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT>
         struct FragConfig<accumulator, BlockM, BlockN, BlockK, DataT>
         {
-            using Map = AccMap<BlockM, BlockN, accTileRows(BlockM, BlockN)>;
+            // 64-bit accumulators in blocks of whole 16 x 16 tiles use the layout of the f64 instruction
+            using Map = std::conditional_t<sizeof(DataT) == 8u && BlockM % 16u == 0u && BlockN % 16u == 0u,
+                                           AccMapStrided<BlockM % 16u == 0u ? BlockM : 16u, BlockN % 16u == 0u ? BlockN : 16u>,
+                                           AccMap<BlockM, BlockN, accTileRows(BlockM, BlockN)>>;
             template <typename Layout>
             using IO = AccIO<Map, DataT, std::is_same<Layout, row_major>::value>;
         };

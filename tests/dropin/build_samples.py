@@ -7,8 +7,9 @@ the rest of the tree.  tests/test_gpu_reference_samples.py runs them there: each
 validates its own GPU result against its own CPU code and prints PASSED or FAILED.
 
   simple_hgemm, simple_dlrm : compiled as they are, with their own main().
-  simple_sgemv, perf_hgemm, simple_sgemm, perf_sgemm (the two f32 GEMM samples are outside the
-                              workloads this library is built for and come along for free)
+  simple_sgemv, perf_hgemm, simple_sgemm, perf_sgemm, simple_dgemm, perf_dgemm, simple_dgemv (the f32
+                              and f64 samples are outside the workloads this library is built for
+                              and come along with the header API)
                             : their host code asks the helper header which device it runs on,
                               and that helper (samples/common.hpp:65-80, 113-130) only knows
                               gfx908..gfx942.  The sample is included from a two-line driver that
@@ -82,6 +83,46 @@ int main()
     return 0;
 }
 """,
+    "simple_dgemm": """
+#include <rocwmma/rocwmma.hpp>
+#include "common.hpp"
+#define isF64Supported() true
+#define main reference_sample_main
+#include "simple_dgemm.cpp"
+#undef main
+int main()
+{
+    gemm_test(256, 256, 256, 2.1, 2.1);
+    return 0;
+}
+""",
+    "perf_dgemm": """
+#include <rocwmma/rocwmma.hpp>
+#include "common.hpp"
+#define isF64Supported() true
+#define isGfx9() true
+#define main reference_sample_main
+#include "perf_dgemm.cpp"
+#undef main
+int main()
+{
+    gemm_test(1024, 1024, 1024, 2, 2);
+    return 0;
+}
+""",
+    "simple_dgemv": """
+#include <rocwmma/rocwmma.hpp>
+#include "common.hpp"
+#define isF64Supported() true
+#define main reference_sample_main
+#include "simple_dgemv.cpp"
+#undef main
+int main()
+{
+    dgemv_test(256, T_BLOCK_Y * ROCWMMA_N, 256, 2.1, 2.1);
+    return 0;
+}
+""",
     "perf_hgemm": """
 #include <rocwmma/rocwmma.hpp>
 #include "common.hpp"
@@ -118,6 +159,7 @@ _MATRIX_TYPES = [
     (("i8", "i32", "i32"), [(16, 32), (16, 64), (32, 16), (32, 32)]),
     (("f8", "f32", "f32"), [(16, 32), (16, 64), (16, 128), (32, 16), (32, 64)]),
     (("bf8", "f32", "f32"), [(16, 32), (16, 128), (32, 16), (32, 64)]),
+    (("f64", "f64", "f64"), [(16, 4), (16, 8), (16, 16)]),
 ]
 _CONFIGS = ["Block::LdsNT", "Block::LdsTN", "Block::LdsRF", "Wave::LdsNT", "Wave::LdsTN", "Wg::LdsNT", "Wg::LdsTN"]
 _BLOCKS = [(1, 1), (2, 2), (1, 2), (2, 1), (4, 2), (2, 4), (4, 4), (1, 4)]

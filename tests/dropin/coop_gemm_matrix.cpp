@@ -215,6 +215,7 @@ namespace
     using f16       = float16_t;
     using bf16      = bfloat16_t;
     using f32       = float32_t;
+    using f64       = float64_t;
     using f8        = float8_t;
     using bf8       = bfloat8_t;
     using i8        = int8_t;

@@ -73,6 +73,29 @@ void checkAcc(const char* name)
         CHECK(seen[i] == 1, "%s: element %u covered %d times", name, i, seen[i]);
 }
 
+// 64-bit accumulators: v_mfma_f64_16x16x4_f64 puts register i of lane l on row (l / 16) + 4 i and column
+// l % 16 of its result; with the multiplicands swapped that is row l % 16, column (l / 16) + 4 i of D.
+template <uint32_t BM, uint32_t BN>
+void checkAccStrided(const char* name)
+{
+    using M = AccMapStrided<BM, BN>;
+    std::vector<int> seen(BM * BN, 0);
+    CHECK(M::size * 64 == BM * BN && M::nruns == M::size && M::runLen == 1, "%s: sizes", name);
+    for(uint32_t lane = 0; lane < 64; ++lane)
+        for(uint32_t e = 0; e < M::size; ++e)
+        {
+            uint32_t r = M::rowOf(e, lane), c = M::colOf(e, lane);
+            CHECK(r < BM && c < BN, "%s: out of range", name);
+            if(r < BM && c < BN)
+                seen[r * BN + c]++;
+            CHECK(r % 16 == lane % 16, "%s: row rule", name);
+            CHECK(c % 16 == lane / 16 + 4 * (e % 4), "%s: column rule", name);
+            CHECK(r / 16 == (e / 4) / M::nbj && c / 16 == (e / 4) % M::nbj, "%s: tile order", name);
+        }
+    for(uint32_t i = 0; i < BM * BN; ++i)
+        CHECK(seen[i] == 1, "%s: element %u covered %d times", name, i, seen[i]);
+}
+
 int main()
 {
     // K packing picks the widest gfx950 instruction that divides BlockK
@@ -104,6 +127,11 @@ int main()
     checkAcc<48, 16, 16>("acc 48x16");
     checkAcc<32, 64, 32>("acc 32x64");
     checkAcc<128, 128, 32>("acc 128x128");
+    checkAccStrided<16, 16>("f64 acc 16x16");
+    checkAccStrided<32, 32>("f64 acc 32x32");
+    checkAccStrided<64, 16>("f64 acc 64x16");
+    checkInput<16, 4, 16, PackClass::Other>("f64 16x4 t16", 1); // 16x16x4
+    checkInput<32, 16, 16, PackClass::Other>("f64 32x16 t16", 1);
     // blocks with an edge of 8: load / store only
     checkInput<8, 32, 8, PackClass::Bits16>("f16 8x32 t8", 4);
     checkInput<8, 256, 8, PackClass::Bits16>("f16 8x256 t8", 8);

@@ -13,9 +13,10 @@ pytestmark = pytest.mark.gpu
 
 BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "dropin", "_bin")
 # sample -> number of self-checks it prints
-# (the two f32 GEMM samples are not among the workloads the library is built for; they compile and
+# (the f32 and f64 samples are not among the workloads the library is built for; they compile and
 # pass as they are and are kept as further evidence for the header API)
-SAMPLES = {"simple_hgemm": 1, "perf_hgemm": 1, "simple_sgemv": 1, "simple_dlrm": 3, "simple_sgemm": 1, "perf_sgemm": 1}
+SAMPLES = {"simple_hgemm": 1, "perf_hgemm": 1, "simple_sgemv": 1, "simple_dlrm": 3, "simple_sgemm": 1, "perf_sgemm": 1,
+           "simple_dgemm": 1, "perf_dgemm": 1, "simple_dgemv": 1}
 
 
 @pytest.mark.parametrize("sample", sorted(SAMPLES))

@@ -1,8 +1,8 @@
 """Drop-in proof for the header API: the reference's own sample kernels compile unchanged.
 
 The four samples the hot path is made of (samples/simple_hgemm.cpp, perf_hgemm.cpp,
-simple_dlrm.cpp, simple_sgemv.cpp in the reference tree) and its two f32 GEMM samples
-(simple_sgemm.cpp, perf_sgemm.cpp) are compiled for gfx950, device and
+simple_dlrm.cpp, simple_sgemv.cpp in the reference tree) and its f32 / f64 samples
+(simple_sgemm.cpp, perf_sgemm.cpp, simple_dgemm.cpp, perf_dgemm.cpp, simple_dgemv.cpp) are compiled for gfx950, device and
 host pass, with this repository's include/ in front of the include path.  The dependency list of
 each compilation must contain this repository's rocwmma headers and none from the reference's
 library/ directory or from the rocWMMA that ships with the toolchain.
@@ -18,7 +18,8 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REFERENCE = "/root/reference"
-SAMPLES = ["simple_hgemm", "perf_hgemm", "simple_dlrm", "simple_sgemv", "simple_sgemm", "perf_sgemm"]
+SAMPLES = ["simple_hgemm", "perf_hgemm", "simple_dlrm", "simple_sgemv", "simple_sgemm", "perf_sgemm",
+           "simple_dgemm", "perf_dgemm", "simple_dgemv"]
 
 
 def _hipcc():
