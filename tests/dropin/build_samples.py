@@ -160,6 +160,8 @@ _MATRIX_TYPES = [
     (("f8", "f32", "f32"), [(16, 32), (16, 64), (16, 128), (32, 16), (32, 64)]),
     (("bf8", "f32", "f32"), [(16, 32), (16, 128), (32, 16), (32, 64)]),
     (("f64", "f64", "f64"), [(16, 4), (16, 8), (16, 16)]),
+    (("h16", "f32", "f32"), [(16, 32), (32, 16)]),
+    (("h16", "h16", "f32"), [(16, 16), (32, 8)]),
 ]
 _CONFIGS = ["Block::LdsNT", "Block::LdsTN", "Block::LdsRF", "Wave::LdsNT", "Wave::LdsTN", "Wg::LdsNT", "Wg::LdsTN"]
 _BLOCKS = [(1, 1), (2, 2), (1, 2), (2, 1), (4, 2), (2, 4), (4, 4), (1, 4)]
