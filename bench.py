@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0
 # file (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB; the factors come from a plain 1 GiB device copy,
 # --calibrate-copy).  Counters cannot be read from inside this process, so the figure is the one
 # recorded with the committed counter summary; None for cases that were not profiled.
-MEASURED_TRAFFIC_BYTES = {("f16_rc", 8192): (2 * 923670 + 262172) * 1024}
+MEASURED_TRAFFIC_BYTES = {("f16_rc", 8192): (2 * 926924 + 262185) * 1024}
 
 
 def parse_args():
