@@ -95,7 +95,11 @@ int rocwmma_amd_device_info(int* compute_units, int* clock_mhz, int* is_gfx950);
  * c may be NULL when beta == 0.  c may equal d.
  * Shapes: m and n multiples of 16, k a multiple of 32 bytes' worth of elements per row is the
  * minimum every kernel accepts (k % 16 == 0 for 16-bit types, k % 32 == 0 for 8-bit types);
- * the blocked kernel additionally needs whole macro tiles and is chosen automatically.
+ * the blocked kernel additionally needs whole macro tiles (multiples of 64) and is chosen
+ * automatically, as are the weight-streaming kernels for up to 112 rows of A against a col-major B.
+ * One of those (48, 80, 96, 112 rows, or a 16-bit A too large for the LDS) runs as two launches on the
+ * stream and adds its K slices into D with atomic adds: I32 results are exact, F32 results can differ
+ * in the last bit from run to run.
  * Alignment: base pointers and leading dimensions must be multiples of 16 bytes.
  */
 int rocwmma_amd_gemm(int         dtype_in,
