@@ -390,6 +390,8 @@ namespace rocwmma
 #pragma unroll
             for(uint32_t bj = 0; bj < MapAcc::nbj; ++bj)
                 *reinterpret_cast<Acc*>(&d.x[MapAcc::blockIndex(bi, bj) * MapAcc::perBlock]) = acc[bi][bj];
+#else
+        (void)d, (void)a, (void)b, (void)c;
 #endif // ROCWMMA_ARCH_GFX950
     }
 

@@ -144,12 +144,13 @@ namespace rocwmma_amd
         template <uint32_t Mfmas, uint32_t Reads, uint32_t Copies>
         ROCWMMA_DEVICE ROCWMMA_INLINE void scheduleInterleaved()
         {
+            constexpr uint32_t Div = Mfmas > 0u ? Mfmas : 1u; // (an empty group: the loop does not run)
 #pragma unroll
             for(uint32_t j = 0; j < Mfmas; ++j)
             {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
-                const uint32_t r = ((j + 1u) * Reads) / Mfmas - (j * Reads) / Mfmas;
-                const uint32_t c = ((j + 1u) * Copies) / Mfmas - (j * Copies) / Mfmas;
+                const uint32_t r = ((j + 1u) * Reads) / Div - (j * Reads) / Div;
+                const uint32_t c = ((j + 1u) * Copies) / Div - (j * Copies) / Div;
                 if(r == 1u)
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
                 else if(r == 2u)

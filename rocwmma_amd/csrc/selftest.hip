@@ -204,6 +204,8 @@ namespace rocwmma_amd
                 using GRBuffB     = fragment<matrix_b, BM, MacroY, BK, float16_t, LB>;
                 using LWBuffA     = ApplyDataLayout_t<GRBuffA, LdsLayout>;
                 using LWBuffB     = ApplyDataLayout_t<ApplyTranspose_t<GRBuffB>, LdsLayout>;
+                static_assert(std::is_same<GetDataLayout_t<LWBuffA>, GetDataLayout_t<LWBuffB>>::value,
+                              "A and transposed-B slabs share the LDS layout");
                 using LRFragA     = ApplyDataLayout_t<MfmaFragA, LdsLayout>;
                 using LRFragB     = ApplyDataLayout_t<ApplyTranspose_t<MfmaFragB>, LdsLayout>;
 
