@@ -217,7 +217,7 @@ def coop_gemm_cases():
 # (BlockM, BlockN) of the reference's unit tests (test/unit/unit_test_params.hpp:89-141)
 _UNIT_SIZES = ([(16, k) for k in (16, 32, 64, 128, 256)]
                + [(b, k) for b in (32, 64, 128, 256) for k in (8, 16, 32, 64, 128, 256)])
-_UNIT_TYPES = ["f16", "f32", "i8", "bf16", "f64", "f8", "i32", "bf8"]
+_UNIT_TYPES = ["f16", "h16", "f32", "i8", "bf16", "f64", "f8", "i32", "bf8"]
 _UNIT_TBLOCKS = [(64, 1), (64, 2), (128, 1), (64, 4), (128, 2), (256, 1)]
 
 

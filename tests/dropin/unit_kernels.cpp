@@ -213,6 +213,7 @@ namespace
     using C    = col_major;
     using f16  = float16_t;
     using bf16 = bfloat16_t;
+    using h16  = hfloat16_t;
     using f32  = float32_t;
     using f64  = float64_t;
     using f8   = float8_t;

@@ -11,7 +11,7 @@ accumulation order.
 Part 2: the device kernels of the reference's unit tests that use only the public API
 (test/unit/*/device/*.hpp: load / store, cooperative load / store, fill, load and store contamination,
 MappingUtil coordinate maps and their overrides), over the reference's block sizes
-(16..256 x 8..256, test/unit/unit_test_params.hpp:89-141), both layouts, eight element types and six
+(16..256 x 8..256, test/unit/unit_test_params.hpp:89-141), both layouts, nine element types and six
 thread-block shapes; each must move exactly the elements its contract says (tests/dropin/unit_kernels.cpp).
 
 Part 3: the reference's DLRM dot-interaction test kernels (test/dlrm/device/dlrm_dot_{fwd,bwd}.hpp and the
