@@ -371,6 +371,42 @@ def test_skinny_and_sliced_kernels_16bit(dtype_in, m, n, k):
     assert np.array_equal(got, orc.gemm(dtype_in, orc.F32, RM, CM, RM, RM, m, n, k, ai, bi, None, 1.0, 0.0))
 
 
+def _random_cases(count):
+    rng = np.random.default_rng(20240607)
+    out = []
+    for i in range(count):
+        dtype_in = [orc.F16, orc.BF16, orc.I8, orc.E4M3][i % 4]
+        m = int(rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 192, 256, 320]))
+        n = int(rng.choice([16, 64, 128, 192, 256, 352, 448, 512, 1040]))
+        k = int(rng.choice([64, 128, 256, 512, 1024, 2048]))
+        if dtype_in in (orc.I8, orc.E4M3) or rng.random() < 0.5:
+            la, lb = RM, CM
+        else:
+            la, lb = [(RM, RM), (CM, CM), (CM, RM)][int(rng.integers(3))]
+        out.append((dtype_in, m, n, k, la, lb, float(rng.choice([1.0, 2.0])), float(rng.choice([0.0, 1.0, -2.0]))))
+    return out
+
+
+@pytest.mark.parametrize("case", _random_cases(48), ids=lambda c: "-".join(str(x) for x in c))
+def test_auto_dispatch_on_seeded_random_shapes(case):
+    """Whatever kernel AUTO picks (weight-streaming, K-sliced, any rung of the blocked kernel's ladder,
+    wave-tile) the result must match the oracle: shapes drawn so that every path is hit."""
+    dtype_in, m, n, k, la, lb, alpha, beta = case
+    out = OUT_OF[dtype_in]
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(7, orc.I8, m * k), uniform_bits(8, orc.I8, k * n)
+        c = uniform_bits(9, orc.I32, m * n)
+    elif dtype_in == orc.E4M3:
+        a, b = normal_fp8_bits(7, dtype_in, m * k), normal_fp8_bits(8, dtype_in, k * n)
+        c = np.random.default_rng(9).uniform(-1, 1, m * n).astype(np.float32)
+    else:
+        a, b = uniform_bits(7, dtype_in, m * k), uniform_bits(8, dtype_in, k * n)
+        c = np.random.default_rng(9).uniform(-1, 1, m * n).astype(np.float32)
+    got = run_gemm(dtype_in, out, la, lb, RM, m, n, k, a, b, c, alpha, beta, rw.GEMM_AUTO)
+    want = orc.gemm(dtype_in, out, la, lb, RM, RM, m, n, k, a, b, c, alpha, beta)
+    check(dtype_in, out, got, want, tol_for(dtype_in))
+
+
 # ---------------------------------------------------------------- config 3: quantised shapes
 @pytest.mark.parametrize("m", [16, 128, 4096])
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3])
