@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device copy (known traffic) for counter calibration")
+    ap.add_argument("--shapes", action="store_true",
+                    help="also time GEMM shapes below the headline size, one per kernel / tile configuration "
+                         "(extra.shapes in the JSON line)")
     ap.add_argument("--only", default=None,
                     help="run one headline case only, e.g. f16_rc (dtype_{r|c}{r|c} = A,B layout): for profiling")
     return ap.parse_args()
@@ -217,6 +220,8 @@ def main():
     extra = {"device": info, "cases": per_case}
     if not args.no_extras and not args.only:
         extra.update(run_extras(rw, torch, dev, gen, args))
+    if args.shapes:
+        extra["shapes"] = run_shapes(rw, torch, dev, gen)
 
     print(json.dumps({
         "metric": "gemm_tflops_8192cubed_f16_bf16_4layouts", "value": round(value, 2), "unit": "TFLOP/s",
@@ -227,6 +232,65 @@ def main():
                                f"({len(cases)} GEMMs per step), alpha=beta=1"},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "extra": extra,
     }))
+
+
+def run_shapes(rw, torch, dev, gen):
+    """GEMM shapes off the headline size, through AUTO, one or two per kernel / rung of the tile
+    ladder: microseconds per launch with the weights rotated over buffers of more than 256 MiB in
+    total (so they come from HBM), A row-major / B col-major unless noted."""
+    RM, CM = rw.ROW_MAJOR, rw.COL_MAJOR
+    shapes = [
+        # dtype, m, n, k, (layout a, layout b), what serves it on a 256-unit device
+        ("f16", 16, 14336, 4096, (RM, CM), "weight-streaming, all of A in LDS"),
+        ("f16", 32, 14336, 4096, (RM, CM), "K-sliced weight-streaming"),
+        ("f16", 48, 14336, 4096, (RM, CM), "K-sliced weight-streaming"),
+        ("f16", 64, 14336, 4096, (RM, CM), "blocked, 64 x 64 tiles"),
+        ("f16", 192, 14336, 4096, (RM, CM), "blocked, 64 x 64 tiles"),
+        ("f16", 128, 14336, 4096, (RM, CM), "blocked, 128 x 64 tiles"),
+        ("f16", 256, 14336, 4096, (RM, CM), "blocked, 128 x 128 tiles"),
+        ("f16", 512, 512, 4096, (RM, CM), "blocked, 64 x 64 tiles (small problem)"),
+        ("f16", 512, 512, 4096, (RM, RM), "blocked, 64 x 128 tiles (B row-major)"),
+        ("f16", 512, 512, 4096, (CM, RM), "blocked, 128 x 128 tiles (A col-major, B row-major)"),
+        ("f16", 2048, 2048, 2048, (RM, CM), "blocked, 128 x 128 tiles"),
+        ("f16", 3072, 3072, 3072, (RM, CM), "blocked, 256 x 256 tiles, 144 of them"),
+        ("f16", 4096, 4096, 4096, (RM, CM), "blocked, 256 x 256 tiles"),
+        ("i8", 48, 14336, 4096, (RM, CM), "K-sliced weight-streaming"),
+        ("i8", 64, 14336, 4096, (RM, CM), "blocked, 64 x 64 tiles"),
+        ("i8", 112, 14336, 4096, (RM, CM), "K-sliced weight-streaming"),
+        ("i8", 256, 14336, 4096, (RM, CM), "blocked, 128 x 128 tiles"),
+        ("i8", 8192, 8192, 8192, (RM, CM), "blocked, 256 x 256 tiles"),
+        ("fp8", 256, 14336, 4096, (RM, CM), "blocked, 128 x 128 tiles"),
+        ("fp8", 8192, 8192, 8192, (RM, CM), "blocked, 256 x 256 tiles"),
+    ]
+    out = []
+    for tag, m, n, k, (la, lb), what in shapes:
+        esize = 2 if tag == "f16" else 1
+        copies = max(2, min(6, -(-(300 << 20) // (n * k * esize))))  # weights rotate over >= 300 MiB, at most 6 buffers
+        if tag == "f16":
+            A = (torch.rand(m * k, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+            Bs = [(torch.rand(k * n, device=dev, generator=gen) * 2 - 1).to(torch.float16) for _ in range(copies)]
+            code, ocode, D = rw.F16, rw.F32, torch.empty(m * n, device=dev)
+        elif tag == "i8":
+            A = torch.randint(-128, 128, (m * k,), device=dev, dtype=torch.int8, generator=gen)
+            Bs = [torch.randint(-128, 128, (k * n,), device=dev, dtype=torch.int8, generator=gen) for _ in range(copies)]
+            code, ocode, D = rw.I8, rw.I32, torch.empty(m * n, device=dev, dtype=torch.int32)
+        else:
+            A = (torch.randn(m * k, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+            Bs = [(torch.randn(k * n, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn) for _ in range(copies)]
+            code, ocode, D = rw.E4M3, rw.F32, torch.empty(m * n, device=dev)
+        state = {"i": 0}
+
+        def fn():
+            rw.gemm(code, ocode, la, lb, RM, m, n, k, A, Bs[state["i"] % copies], None, D, 1.0, 0.0)
+            state["i"] += 1
+
+        fn(), fn()
+        ms = min(event_ms(fn, 20, torch) for _ in range(3))
+        out.append({"dtype": tag, "m": m, "n": n, "k": k, "a": "row" if la == RM else "col",
+                    "b": "col" if lb == CM else "row", "us": round(ms * 1e3, 1),
+                    "tflops": round(2.0 * m * n * k / ms / 1e9, 1), "kernel": what})
+        del A, Bs, D
+    return out
 
 
 def run_extras(rw, torch, dev, gen, args):
