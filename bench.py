@@ -9,12 +9,21 @@ resident in HBM when the timed region starts.
 
 Prints ONE JSON line.  Besides the contract fields it carries
   roofline     : the dominant kernel (f16, A row-major, B col-major) against the 2.5 PFLOP/s dense
-                 f16 MFMA peak, timed with events on the launch stream;
+                 f16 MFMA peak, timed with events on the launch stream; next to the nominal peak,
+                 what a loop of nothing but matrix instructions sustains on this box on the same
+                 operand distribution and on all-zero operands (the part is power managed and the
+                 sustained rate depends on the operand bits), and the same kernel on all-zero operands;
   cpu_baseline : the CPU oracle (a port of the reference's OpenMP gemm_CPU) timed on this box's
-                 host cores on a bounded sample of the same workload;
+                 host cores on a bounded sample of the same workload; the rows it computes also
+                 check the GPU result of the timed case (outside the timed region);
   extra        : the other configurations (quantised GEMMs, GEMV, DLRM) with their own rooflines.
+
+--only NAME runs one case alone (for profiling): a headline case (f16_rc, bf16_cr, ...: dtype_{A}{B}
+layouts) or one of the extra cases by its key in the JSON line (gemm_fp8_m4096, gemm_i8_m128,
+gemv_8192x8192_n8, dlrm_bwd_b262144, ...).
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -26,11 +35,35 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0, "i8": 5000.0}  # dense MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
-# Bytes moved through the L2s per launch of the dominant kernel, from rocprofv3 counter runs of this
-# file (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB; the factors come from a plain 1 GiB device copy,
-# --calibrate-copy).  Counters cannot be read from inside this process, so the figure is the one
-# recorded with the committed counter summary; None for cases that were not profiled.
-MEASURED_TRAFFIC_BYTES = {("f16_rc", 8192): (2 * 926924 + 262185) * 1024}
+FP8_BLOCKED_SHAPE = "fp8_32x32x64"  # the matrix instruction of the blocked kernel's 256 x 256 fp8 configuration
+# Bytes moved through the L2s per launch come from rocprofv3 counter runs of this file (counters cannot
+# be read from inside this process): profiles/traffic.json holds the figures of the committed counter
+# summaries together with a digest of the kernel sources they were taken on, and a figure whose digest
+# no longer matches is reported as null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+KERNEL_SOURCES = {
+    "gemm_blocked": ["rocwmma_amd/csrc/gemm_blocked.hip", "include/rocwmma/rocwmma_lds.hpp"],
+}
+
+
+def sources_digest(family):
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES[family]:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(key, family):
+    """Bytes per launch recorded for `key`, or None when nothing current is recorded."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f).get(key)
+    except (OSError, ValueError):
+        return None
+    if not rec or rec.get("sources_digest") != sources_digest(family):
+        return None
+    return rec.get("bytes")
 
 
 def parse_args():
@@ -47,7 +80,8 @@ def parse_args():
                     help="also time GEMM shapes below the headline size, one per kernel / tile configuration "
                          "(extra.shapes in the JSON line)")
     ap.add_argument("--only", default=None,
-                    help="run one headline case only, e.g. f16_rc (dtype_{r|c}{r|c} = A,B layout): for profiling")
+                    help="run one case only: a headline case such as f16_rc (dtype_{r|c}{r|c} = A,B layout) or an "
+                         "extra case by its JSON key (gemm_fp8_m4096, gemv_8192x8192_n8, ...): for profiling")
     return ap.parse_args()
 
 
@@ -104,6 +138,9 @@ def launch_stats(fn, iters, torch):
     return t[len(t) // 2], t[0]
 
 
+HEADLINE_TAGS = [f"{d}_{a}{b}" for d in ("f16", "bf16") for a in "rc" for b in "rc"]
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -116,7 +153,7 @@ def main():
 
     import rocwmma_amd as rw
 
-    if not os.path.exists(rw.library_path()):
+    if not os.path.exists(rw.library_path()) or not os.path.exists(rw.aux_library_path()):
         import __graft_entry__ as g
 
         g.build()
@@ -135,6 +172,13 @@ def main():
         ms = event_ms(lambda: dst.copy_(src), 5, torch)
         print(json.dumps({"calibrate_copy_bytes_each_way": src.numel() * 4, "ms": round(ms, 4),
                           "gbs": round(2 * src.numel() * 4 / ms / 1e6, 1)}))
+        return
+
+    if args.only and args.only not in HEADLINE_TAGS:
+        # one extra case alone (profiling): a few launches, nothing else on the device
+        out = run_extras(rw, torch, dev, gen, only=args.only)
+        assert out, f"no case matches --only {args.only}"
+        print(json.dumps({"only": args.only, "device": info, "result": out}))
         return
 
     def rand(count, dtype):
@@ -185,18 +229,40 @@ def main():
         per_case[case[0]] = {"ms": round(ms, 4), "tflops": round(flops_per_gemm / ms / 1e9, 1),
                              "ms_median": round(med, 4), "ms_min": round(best, 4)}
     dom = "f16_rc" if "f16_rc" in per_case else cases[0][0]
-    dom_peak = PEAK_TFLOPS["bf16" if dom.startswith("bf16") else "f16"]
+    dom_dtype = "bf16" if dom.startswith("bf16") else "f16"
+    dom_peak = PEAK_TFLOPS[dom_dtype]
     roofline = {
         "bound": "mfma", "kernel": f"gemmBlockedKernel {dom} {S}^3",
         "achieved": per_case[dom]["tflops"], "peak": dom_peak, "unit": "TFLOP/s",
         "frac": round(per_case[dom]["tflops"] / dom_peak, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get((dom, S)),
+        "traffic": measured_traffic(f"{dom}_{S}", "gemm_blocked"),
         "ms": per_case[dom]["ms"],
     }
 
+    # The matrix pipes' own ceiling on this box (no memory traffic at all) for the dominant kernel's
+    # instruction, on this operand distribution and on all-zero operands, and the dominant kernel on
+    # all-zero operands: the gap between the two operand patterns is the device's power management,
+    # not the kernel's schedule.
+    if not args.only or args.only == dom:
+        ceiling = run_ceiling(rw, torch, dev, gen, [dom_dtype] if args.only else None)
+        key = f"{dom_dtype}_16x16x32"
+        dom_case = next(c for c in cases if c[0] == dom)
+        zeros = torch.zeros(S * S, device=dev, dtype=dom_case[4].dtype)
+        rw.gemm(dom_case[1], rw.F32, dom_case[2], dom_case[3], RM, S, S, S, zeros, zeros, C, D, 1.0, 1.0)
+        ms_zero = event_ms(lambda: rw.gemm(dom_case[1], rw.F32, dom_case[2], dom_case[3], RM, S, S, S, zeros, zeros,
+                                           C, D, 1.0, 1.0), max(args.steps, 5), torch)
+        del zeros
+        roofline["mfma_only_ceiling"] = ceiling
+        roofline["frac_of_mfma_only_ceiling"] = round(per_case[dom]["tflops"] / ceiling[key]["data"], 4)
+        roofline["zero_operands"] = {
+            "ms": round(ms_zero, 4), "tflops": round(flops_per_gemm / ms_zero / 1e9, 1),
+            "frac": round(flops_per_gemm / ms_zero / 1e9 / dom_peak, 4),
+            "frac_of_mfma_only_ceiling": round(flops_per_gemm / ms_zero / 1e9 / ceiling[key]["zero"], 4),
+        }
+
     # ------------------------------------------------------------------ CPU baseline (oracle port)
     cpu_baseline = None
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and "f16_rc" in per_case:
         import oracle as orc
 
         rows_n = 1024 if S >= 4096 else S
@@ -206,20 +272,35 @@ def main():
         b_bits = B.view(torch.int16).cpu().numpy().view(np.uint16)
         c_host = C.cpu().numpy()
         t0 = time.perf_counter()
-        orc.gemm(orc.F16, orc.F32, 0, 1, 0, 0, S, S, S, a_bits, b_bits, c_host, 1.0, 1.0, rows=rows)
+        want = orc.gemm(orc.F16, orc.F32, 0, 1, 0, 0, S, S, S, a_bits, b_bits, c_host, 1.0, 1.0, rows=rows)
         dt = time.perf_counter() - t0
+        # the same rows of the GPU result of the timed f16 A-row / B-col case, outside the timed region
+        D.fill_(float("nan"))
+        run_case(next(c for c in cases if c[0] == "f16_rc"))
+        torch.cuda.synchronize()
+        got = D.view(S, S)[torch.from_numpy(rows.astype(np.int64)).to(dev)].cpu().numpy().ravel()
+        ref = want.reshape(S, S)[rows].ravel()
+        err, inf, nan = orc.compare_equal(orc.F32, got, orc.F32, ref)
+        assert not inf and not nan and err <= 1e-3, f"timed GEMM differs from the CPU oracle: {err} {inf} {nan}"
+        assert not bool(torch.isnan(D).any()), "NaN left in D after the timed case"
         cpu_baseline = {
             "value": round(2.0 * rows.size * S * S / dt / 1e12, 5), "unit": "TFLOP/s",
             "cores": orc.num_threads(), "kind": "port",
             "sample": f"{rows.size} of {S} output rows (every column) of the f16 A-row/B-col {S}^3 case, "
                       f"{dt:.1f} s incl. operand decode",
+            "gpu_result_checked": {"rows": int(rows.size), "max_rel_err": float(f"{err:.3e}"), "tolerance": 1e-3},
         }
-        del a_bits, b_bits, c_host
+        del a_bits, b_bits, c_host, want
 
     # ------------------------------------------------------------------ other configurations
     extra = {"device": info, "cases": per_case}
     if not args.no_extras and not args.only:
-        extra.update(run_extras(rw, torch, dev, gen, args))
+        extra.update(run_extras(rw, torch, dev, gen))
+        # the MFMA-bound quantised case against the matrix pipes' own ceiling for its instruction
+        for key, shape in (("gemm_i8_m4096", "i8_16x16x64"), ("gemm_fp8_m4096", FP8_BLOCKED_SHAPE)):
+            if key in extra and shape in roofline.get("mfma_only_ceiling", {}):
+                extra[key]["frac_of_mfma_only_ceiling"] = round(
+                    extra[key]["tops"] / roofline["mfma_only_ceiling"][shape]["data"], 4)
     if args.shapes:
         extra["shapes"] = run_shapes(rw, torch, dev, gen)
 
@@ -232,6 +313,45 @@ def main():
                                f"({len(cases)} GEMMs per step), alpha=beta=1"},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "extra": extra,
     }))
+
+
+def run_ceiling(rw, torch, dev, gen, dtypes=None):
+    """TFLOP/s (TOP/s) of a loop of nothing but matrix instructions, two waves per SIMD on every compute
+    unit, operands in registers: per instruction shape, on the benchmark's operand distribution for
+    that type ("data") and on all-zero operands ("zero").  Each figure is a launch of about 10 ms
+    after a warm-up launch of the same length (shorter launches still see the clock ramp)."""
+    n = 65536
+    tables = {
+        "f16": (torch.rand(n // 2, device=dev, generator=gen) * 2 - 1).to(torch.float16).view(torch.uint8),
+        "bf16": (torch.rand(n // 2, device=dev, generator=gen) * 2 - 1).to(torch.bfloat16).view(torch.uint8),
+        "i8": torch.randint(-128, 128, (n,), device=dev, dtype=torch.int8, generator=gen).view(torch.uint8),
+        "fp8": (torch.randn(n, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn).view(torch.uint8),
+        "zero": torch.zeros(n, device=dev, dtype=torch.uint8),
+    }
+    shapes = [("f16_16x16x32", rw.MFMA_F16_16X16X32, "f16", 20000), ("f16_32x32x16", rw.MFMA_F16_32X32X16, "f16", 7000),
+              ("bf16_16x16x32", rw.MFMA_BF16_16X16X32, "bf16", 20000), ("i8_16x16x64", rw.MFMA_I8_16X16X64, "i8", 20000),
+              ("fp8_32x32x64", rw.MFMA_F8_32X32X64, "fp8", 5000), ("fp8_16x16x128", rw.MFMA_F8_16X16X128, "fp8", 10000)]
+    sink = torch.empty(info_lanes(rw), device=dev)
+    out = {}
+    for name, shape, kind, trips in shapes:
+        if dtypes is not None and kind not in dtypes:
+            continue
+        res = {}
+        for label, table in (("data", tables[kind]), ("zero", tables["zero"])):
+            rw.bench_mfma_ceiling(shape, trips, 2, table, sink)
+            torch.cuda.synchronize()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            ops = rw.bench_mfma_ceiling(shape, trips, 2, table, sink)
+            stop.record()
+            stop.synchronize()
+            res[label] = round(ops / start.elapsed_time(stop) / 1e9, 1)
+        out[name] = res
+    return out
+
+
+def info_lanes(rw):
+    return rw.device_info()["compute_units"] * 2 * 256
 
 
 def run_shapes(rw, torch, dev, gen):
@@ -293,44 +413,59 @@ def run_shapes(rw, torch, dev, gen):
     return out
 
 
-def run_extras(rw, torch, dev, gen, args):
+def run_extras(rw, torch, dev, gen, only=None):
     """The small GEMM (config 1), quantised GEMMs (config 3), GEMV (config 4), DLRM (config 5): kernel
-    time by events."""
+    time by events.  `only`: one case by its key (a few launches of that case and nothing else)."""
     RM, CM = rw.ROW_MAJOR, rw.COL_MAJOR
     out = {}
-    iters = 20
+    iters = 20 if only is None else 5
+
+    def wanted(key):
+        return only is None or only == key
 
     # config 1: 256^3 f16 -> f32, A row / B col, alpha = beta = 2: launch latency, reported only
     m1 = 256
-    A1 = (torch.rand(m1 * m1, device=dev, generator=gen) * 2 - 1).to(torch.float16)
-    B1 = (torch.rand(m1 * m1, device=dev, generator=gen) * 2 - 1).to(torch.float16)
-    C1 = torch.rand(m1 * m1, device=dev, generator=gen) * 2 - 1
-    D1 = torch.empty(m1 * m1, device=dev)
-    for tag, algo in (("wave_tile", rw.GEMM_WAVE_TILE), ("blocked", rw.GEMM_BLOCKED)):
-        def fn1():
-            rw.gemm(rw.F16, rw.F32, RM, CM, RM, m1, m1, m1, A1, B1, C1, D1, 2.0, 2.0, algo=algo)
+    if any(wanted(f"gemm_f16_256cubed_{t}") for t in ("wave_tile", "blocked")):
+        A1 = (torch.rand(m1 * m1, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        B1 = (torch.rand(m1 * m1, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        C1 = torch.rand(m1 * m1, device=dev, generator=gen) * 2 - 1
+        D1 = torch.empty(m1 * m1, device=dev)
+        for tag, algo in (("wave_tile", rw.GEMM_WAVE_TILE), ("blocked", rw.GEMM_BLOCKED)):
+            if not wanted(f"gemm_f16_256cubed_{tag}"):
+                continue
 
-        fn1()
-        ms = event_ms(fn1, 100, torch)
-        msg = graph_ms(fn1, 50, torch)
-        out[f"gemm_f16_256cubed_{tag}"] = {"us": round(ms * 1e3, 2), "tflops": round(2.0 * m1 ** 3 / ms / 1e9, 2),
-                                           "us_graph_replay": None if msg is None else round(msg * 1e3, 2),
-                                           "note": "back-to-back launches, launch-latency bound"}
+            def fn1():
+                rw.gemm(rw.F16, rw.F32, RM, CM, RM, m1, m1, m1, A1, B1, C1, D1, 2.0, 2.0, algo=algo)
+
+            fn1()
+            ms = event_ms(fn1, 100, torch)
+            msg = graph_ms(fn1, 50, torch) if only is None else None
+            out[f"gemm_f16_256cubed_{tag}"] = {"us": round(ms * 1e3, 2), "tflops": round(2.0 * m1 ** 3 / ms / 1e9, 2),
+                                               "us_graph_replay": None if msg is None else round(msg * 1e3, 2),
+                                               "note": "back-to-back launches, launch-latency bound"}
 
     # config 3: N = 14336, K = 4096, M in {16, 128, 4096}; int8 and e4m3, A row / B col.  The weight
     # matrix (56 MiB) would stay in the 256 MiB Infinity Cache between launches, so the timed loop
     # rotates over 5 weight buffers (280 MiB); the cache-resident time is reported beside it.
     n, k = 14336, 4096
     wcopies = 5
-    Bq = [torch.randint(-128, 128, (k * n,), device=dev, dtype=torch.int8, generator=gen) for _ in range(wcopies)]
-    Bf = [(torch.randn(k * n, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn) for _ in range(wcopies)]
-    for m in (16, 128, 4096):
-        Aq = torch.randint(-128, 128, (m * k,), device=dev, dtype=torch.int8, generator=gen)
-        Af = (torch.randn(m * k, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
-        Di = torch.empty(m * n, device=dev, dtype=torch.int32)
-        Df = torch.empty(m * n, device=dev, dtype=torch.float32)
-        flops = 2.0 * m * n * k
-        for tag, code, ocode, A, Bs, Dx in (("i8", rw.I8, rw.I32, Aq, Bq, Di), ("fp8", rw.E4M3, rw.F32, Af, Bf, Df)):
+    q_keys = [(tag, m) for m in (16, 128, 4096) for tag in ("i8", "fp8") if wanted(f"gemm_{tag}_m{m}")]
+    if q_keys:
+        Bq = Bf = None
+        if any(t == "i8" for t, _ in q_keys):
+            Bq = [torch.randint(-128, 128, (k * n,), device=dev, dtype=torch.int8, generator=gen) for _ in range(wcopies)]
+        if any(t == "fp8" for t, _ in q_keys):
+            Bf = [(torch.randn(k * n, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn) for _ in range(wcopies)]
+        for tag, m in q_keys:
+            if tag == "i8":
+                A = torch.randint(-128, 128, (m * k,), device=dev, dtype=torch.int8, generator=gen)
+                Dx = torch.empty(m * n, device=dev, dtype=torch.int32)
+                code, ocode, Bs = rw.I8, rw.I32, Bq
+            else:
+                A = (torch.randn(m * k, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+                Dx = torch.empty(m * n, device=dev, dtype=torch.float32)
+                code, ocode, Bs = rw.E4M3, rw.F32, Bf
+            flops = 2.0 * m * n * k
             state = {"i": 0}
 
             def fn():
@@ -351,13 +486,16 @@ def run_extras(rw, torch, dev, gen, args):
                 "gbs": round(byts / ms / 1e6, 1), "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4),
                 "ms_weights_cache_resident": round(ms_res, 4),
             }
-    del Bq, Bf
+        del Bq, Bf
 
     # config 4: GEMV, buffers rotated over > 512 MB so the 256 MB Infinity Cache cannot serve A
     for (m, kk) in ((8192, 8192), (14336, 4096)):
+        cols = [nc for nc in (1, 4, 8) if wanted(f"gemv_{m}x{kk}_n{nc}")]
+        if not cols:
+            continue
         copies = 5
         As = [(torch.rand(m * kk, device=dev, generator=gen) * 2 - 1).to(torch.float16) for _ in range(copies)]
-        for ncols in (1, 4, 8):
+        for ncols in cols:
             x = (torch.rand(kk * ncols, device=dev, generator=gen) * 2 - 1).to(torch.float16)
             y = torch.zeros(m * ncols, device=dev)
             state = {"i": 0}
@@ -377,6 +515,8 @@ def run_extras(rw, torch, dev, gen, args):
     mm, kd = 27, 128
     width = kd + mm * (mm - 1) // 2
     for batch, copies in ((2048, 1), (262144, 3)):
+        if not (wanted(f"dlrm_fwd_b{batch}") or wanted(f"dlrm_bwd_b{batch}")):
+            continue
         Fs = [(torch.rand(batch * mm * kd, device=dev, generator=gen) * 2 - 1).to(torch.float16) for _ in range(copies)]
         up = (torch.rand(batch * width, device=dev, generator=gen) * 2 - 1).to(torch.float16)
         o = torch.empty(batch * width, device=dev, dtype=torch.float16)
@@ -392,18 +532,17 @@ def run_extras(rw, torch, dev, gen, args):
             rw.dlrm_bwd(Fs[state["i"] % copies], up, gr, mg, mm, kd, batch)
             state["i"] += 1
 
-        fwd(), bwd()
-        ms_f = event_ms(fwd, iters, torch)
-        ms_b = event_ms(bwd, iters, torch)
         bf = batch * (mm * kd * 2.0 + width * 2.0)
         bb = batch * (mm * kd * 2.0 + width * 2.0 + mm * kd * 2.0 + kd * 2.0)
-        out[f"dlrm_fwd_b{batch}"] = {"ms": round(ms_f, 5), "gbs": round(bf / ms_f / 1e6, 1),
-                                     "frac_hbm": round(bf / ms_f / 1e6 / PEAK_HBM_GBS, 4)}
-        out[f"dlrm_bwd_b{batch}"] = {"ms": round(ms_b, 5), "gbs": round(bb / ms_b / 1e6, 1),
-                                     "frac_hbm": round(bb / ms_b / 1e6 / PEAK_HBM_GBS, 4)}
-        if batch == 2048:
-            # the kernels take 4-10 us, less than a Python loop needs per launch: graph replay as well
-            for tag, fnx, byts in (("fwd", fwd, bf), ("bwd", bwd, bb)):
+        for tag, fnx, byts in (("fwd", fwd, bf), ("bwd", bwd, bb)):
+            if not wanted(f"dlrm_{tag}_b{batch}"):
+                continue
+            fnx()
+            ms = event_ms(fnx, iters, torch)
+            out[f"dlrm_{tag}_b{batch}"] = {"ms": round(ms, 5), "gbs": round(byts / ms / 1e6, 1),
+                                           "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4)}
+            if batch == 2048 and only is None:
+                # the kernels take 4-10 us, less than a Python loop needs per launch: graph replay as well
                 msg = graph_ms(fnx, iters, torch)
                 if msg is not None:
                     out[f"dlrm_{tag}_b{batch}"].update({"ms_graph_replay": round(msg, 5),

@@ -113,31 +113,43 @@ namespace rocwmma
         //                   swapped (argument = row bits 2..3)
         // swz = 0, 2, 3, 1 for rows 0-3, 4-7, 8-11, 12-15 satisfies both.
         // ---------------------------------------------------------------------------------
-        template <uint32_t Dim>
+        //
+        // With RowBytes = 128 a row is one whole 128-byte line of the operand (eight chunks), so a
+        // copy instruction requests eight full lines instead of sixteen half lines.  Two rows then
+        // span the 256 bytes the banks cover, and the 16 lanes served together must differ in
+        // (row parity, chunk position): swz = row bits 1..3 does that for both readers (the eight
+        // even rows of a 16-row group get eight different XOR masks; of the two K chunks a group
+        // touches, one goes with masks {0,1,6,7} and the other, differing in bit 0, with {2,3,4,5}).
+        template <uint32_t Dim, uint32_t RowBytes = 64u>
         struct KMajorTile
         {
-            static constexpr uint32_t rowBytes    = 64u;
-            static constexpr uint32_t chunks      = 4u;
-            static constexpr uint32_t rowsPerCopy = 1024u / rowBytes; // 16
+            static_assert(RowBytes == 64u || RowBytes == 128u, "stage rows of 64 or 128 bytes");
+            static constexpr uint32_t rowBytes    = RowBytes;
+            static constexpr uint32_t chunks      = RowBytes / 16u;
+            static constexpr uint32_t rowsPerCopy = 1024u / rowBytes; // 16 or 8
             static constexpr uint32_t bytes       = Dim * rowBytes;
             static constexpr uint32_t copies      = bytes / 1024u; // whole-wave copies per stage
 
             ROCWMMA_HOST_DEVICE static constexpr uint32_t swz(uint32_t row)
             {
-                // 0, 2, 3, 1 for rows 0-3, 4-7, 8-11, 12-15
-                return (0x78u >> ((row >> 1) & 6u)) & 3u;
+                if constexpr(RowBytes == 64u)
+                    return (0x78u >> ((row >> 1) & 6u)) & 3u; // 0, 2, 3, 1 for rows 0-3, 4-7, 8-11, 12-15
+                else
+                    return (row >> 1) & 7u;
             }
             ROCWMMA_HOST_DEVICE static constexpr uint32_t offset(uint32_t row, uint32_t chunk)
             {
                 return row * rowBytes + ((chunk ^ swz(row)) << 4);
             }
-            // Source byte offset of `lane` inside any copy, relative to the copy's first row at
-            // the stage's first K byte: lane i owns LDS position (row i/4, chunk position i%4).
-            // (swz only looks at row bits 2..3, so the copy index does not matter.)
-            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t laneSourceOffset(uint32_t lane, uint32_t /*wave*/, uint32_t ldBytes)
+            // Source byte offset of `lane` inside a copy issued by wave `wave`, relative to the copy's
+            // first row at the stage's first K byte: lane i owns LDS position (row i / chunks, chunk
+            // position i % chunks).  swz looks at row bits below 4 only; copy c of a wave starts at row
+            // (c * waves + wave) * rowsPerCopy, and waves * rowsPerCopy is a multiple of 16 for every
+            // wave pool used, so the copy index does not matter, only the wave.
+            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t laneSourceOffset(uint32_t lane, uint32_t wave, uint32_t ldBytes)
             {
-                const uint32_t row = lane >> 2;
-                return row * ldBytes + (((lane & 3u) ^ swz(row)) << 4);
+                const uint32_t row = lane / chunks;
+                return row * ldBytes + (((lane % chunks) ^ swz(wave * rowsPerCopy + row)) << 4);
             }
             // Source byte offset of copy `copy` (wave uniform)
             ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t copySourceOffset(uint32_t copy, uint32_t ldBytes)
@@ -166,17 +178,17 @@ namespace rocwmma
             }
 
             // Operand of one 16-wide MFMA block with 16 bytes of K per lane (16x16x32 f16 / bf16,
-            // 16x16x64 i8): rows [row0, row0+16), the whole 64 bytes of K of the stage; lane l
-            // holds row l % 16, chunk l / 16.  A quarter-wave reads 16 rows at one chunk index:
+            // 16x16x64 i8): rows [row0, row0+16), 64 bytes of K (K step `ks` of the stage); lane l
+            // holds row l % 16, chunk 4 ks + l / 16.  A quarter-wave reads 16 rows at one chunk index:
             // 16 distinct bank groups by the choice of swz.
             template <uint32_t KPackBytes>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
-                readBlock16(void* regs, const char* ldsTile, uint32_t row0, uint32_t /*ks*/, uint32_t lane)
+                readBlock16(void* regs, const char* ldsTile, uint32_t row0, uint32_t ks, uint32_t lane)
             {
-                static_assert(KPackBytes == 16u, "a 64-byte stage row feeds 16-wide blocks with 16 bytes per lane");
+                static_assert(KPackBytes == 16u, "16-wide blocks take 16 bytes of K per lane");
                 const uint32_t row = row0 + (lane & 15u);
                 *reinterpret_cast<detail::u32x4*>(regs)
-                    = *reinterpret_cast<const detail::u32x4*>(ldsTile + offset(row, lane >> 4));
+                    = *reinterpret_cast<const detail::u32x4*>(ldsTile + offset(row, ks * 4u + (lane >> 4)));
             }
         };
 
@@ -187,11 +199,12 @@ namespace rocwmma
         // K rows of two neighbouring segments (32-wide blocks) or K rows k..k+3 and k+8..k+11 of
         // one segment (16-wide blocks): swz puts both patterns on eight distinct 32-byte positions.
         // ---------------------------------------------------------------------------------
-        template <uint32_t Dim>
+        template <uint32_t Dim, uint32_t KRows = 32u>
         struct DimMajorTile
         {
             static_assert(Dim % 128u == 0u, "tile rows must hold at least eight 32-byte segments");
-            static constexpr uint32_t kRows       = 32u;
+            static_assert(KRows == 32u || KRows == 64u, "stages of 32 or 64 K rows");
+            static constexpr uint32_t kRows       = KRows;
             static constexpr uint32_t rowBytes    = Dim * 2u;
             static constexpr uint32_t bytes       = kRows * rowBytes;
             static constexpr uint32_t copies      = bytes / 1024u;
@@ -259,11 +272,11 @@ namespace rocwmma
             }
 
             // Operand of one 16-wide MFMA block with 8 K values per lane (v_mfma_*_16x16x32):
-            // lane l ends up with dim = dim0 + l % 16 and k = (l/16)*8 + 0..7 (the stage's 32 K
-            // rows in one step).  Same remarks as for readBlock32.
+            // lane l ends up with dim = dim0 + l % 16 and k = 32 ks + (l/16)*8 + 0..7 (32 K rows
+            // per step).  Same remarks as for readBlock32.
             template <uint32_t KPackBytes = 16u>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
-                readBlock16(void* regs, const char* ldsTile, uint32_t dim0, uint32_t /*ks*/, uint32_t lane)
+                readBlock16(void* regs, const char* ldsTile, uint32_t dim0, uint32_t ks, uint32_t lane)
             {
                 static_assert(KPackBytes == 16u, "transposing reads feed the 8-halves-per-lane MFMA shapes");
                 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -271,7 +284,7 @@ namespace rocwmma
                 const uint32_t group   = lane >> 4;
                 const uint32_t s       = lane & 15u;
                 const uint32_t seg     = dim0 >> 4;
-                const uint32_t kBase   = group * 8u + (s >> 2);
+                const uint32_t kBase   = ks * 32u + group * 8u + (s >> 2);
                 const uint32_t inSeg   = (s & 3u) << 3;
 #pragma unroll
                 for(uint32_t kk = 0; kk < 2u; ++kk)

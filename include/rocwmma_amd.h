@@ -214,48 +214,6 @@ int rocwmma_amd_dlrm_bwd(const void* input,
                          uint32_t    batch,
                          void*       stream);
 
-/*
- * Fragment API self-tests (device side of the API-semantics tests; each launches a tiny kernel
- * written only with the public rocwmma:: API and returns a status).
- *
- * rocwmma_amd_selftest_roundtrip: out = store(load(in)) for one fragment kind; mirrors the
- * reference unit test test/unit/load_store_matrix_sync_test/device/load_store_matrix_sync.hpp:35-117
- * (and, with coop != 0, the cooperative twin load_store_matrix_coop_sync_test).
- *   context : 0 matrix_a, 1 matrix_b, 2 accumulator
- *   `in`/`out` are rows x cols matrices of `dtype` in `layout` with leading dimension ld; the
- *   grid covers the matrix with one fragment per wave (or per workgroup of 4 waves when coop).
- *   block   : 16 or 32 (BlockM = BlockN), blockk : K extent of the fragment.
- */
-int rocwmma_amd_selftest_roundtrip(int         context,
-                                   int         dtype,
-                                   int         layout,
-                                   int         block,
-                                   int         blockk,
-                                   int         coop,
-                                   uint32_t    rows,
-                                   uint32_t    cols,
-                                   const void* in,
-                                   void*       out,
-                                   uint32_t    ld,
-                                   void*       stream);
-
-/* Runs the reference's perf_hgemm data flow (cooperative global read -> applyDataLayout /
- * applyTranspose -> cooperative LDS write -> LDS read -> mma_sync) written only against the
- * public API, f16 in / f32 out, for the four A/B layout combinations.  Used to test the
- * cooperative and transform API end to end. */
-int rocwmma_amd_selftest_coop_gemm(int         layout_a,
-                                   int         layout_b,
-                                   uint32_t    m,
-                                   uint32_t    n,
-                                   uint32_t    k,
-                                   const void* a,
-                                   const void* b,
-                                   const float* c,
-                                   float*      d,
-                                   float       alpha,
-                                   float       beta,
-                                   void*       stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,101 @@
+/*
+ * rocwmma_amd_aux.h -- C ABI of librocwmma_amd_aux.so: test and benchmark support that is not part
+ * of the product library (librocwmma_amd.so, rocwmma_amd.h).
+ *
+ *   - the device side of the fragment-API semantics tests: tiny kernels written only against the
+ *     public rocwmma:: device API, launched from the host tests;
+ *   - measurement probes the benchmark reports beside its kernels: a loop of nothing but matrix
+ *     instructions (what the matrix pipes sustain under the board's power management), and a
+ *     blocked GEMM written with the public fragment API only.
+ *
+ * Same conventions as rocwmma_amd.h: device pointers owned by the caller, work enqueued on
+ * `stream`, a rocwmma_amd_status is returned.
+ */
+#ifndef ROCWMMA_AMD_AUX_H
+#define ROCWMMA_AMD_AUX_H
+
+#include "rocwmma_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Fragment API self-tests (device side of the API-semantics tests; each launches a tiny kernel
+ * written only with the public rocwmma:: API and returns a status).
+ *
+ * rocwmma_amd_selftest_roundtrip: out = store(load(in)) for one fragment kind; mirrors the
+ * reference unit test test/unit/load_store_matrix_sync_test/device/load_store_matrix_sync.hpp:35-117
+ * (and, with coop != 0, the cooperative twin load_store_matrix_coop_sync_test).
+ *   context : 0 matrix_a, 1 matrix_b, 2 accumulator
+ *   `in`/`out` are rows x cols matrices of `dtype` in `layout` with leading dimension ld; the
+ *   grid covers the matrix with one fragment per wave (or per workgroup of 4 waves when coop).
+ *   block   : 16 or 32 (BlockM = BlockN), blockk : K extent of the fragment.
+ */
+int rocwmma_amd_selftest_roundtrip(int         context,
+                                   int         dtype,
+                                   int         layout,
+                                   int         block,
+                                   int         blockk,
+                                   int         coop,
+                                   uint32_t    rows,
+                                   uint32_t    cols,
+                                   const void* in,
+                                   void*       out,
+                                   uint32_t    ld,
+                                   void*       stream);
+
+/* Runs the reference's perf_hgemm data flow (cooperative global read -> applyDataLayout /
+ * applyTranspose -> cooperative LDS write -> LDS read -> mma_sync) written only against the
+ * public API, f16 in / f32 out, for the four A/B layout combinations.  Used to test the
+ * cooperative and transform API end to end. */
+int rocwmma_amd_selftest_coop_gemm(int         layout_a,
+                                   int         layout_b,
+                                   uint32_t    m,
+                                   uint32_t    n,
+                                   uint32_t    k,
+                                   const void* a,
+                                   const void* b,
+                                   const float* c,
+                                   float*      d,
+                                   float       alpha,
+                                   float       beta,
+                                   void*       stream);
+
+/* Instruction shapes of rocwmma_amd_bench_mfma_ceiling. */
+typedef enum rocwmma_amd_mfma_shape
+{
+    ROCWMMA_AMD_MFMA_F16_16X16X32  = 0,
+    ROCWMMA_AMD_MFMA_F16_32X32X16  = 1,
+    ROCWMMA_AMD_MFMA_BF16_16X16X32 = 2,
+    ROCWMMA_AMD_MFMA_BF16_32X32X16 = 3,
+    ROCWMMA_AMD_MFMA_I8_16X16X64   = 4,
+    ROCWMMA_AMD_MFMA_I8_32X32X32   = 5,
+    ROCWMMA_AMD_MFMA_F8_16X16X128  = 6, /* v_mfma_f32_16x16x128_f8f6f4 on e4m3 operands */
+    ROCWMMA_AMD_MFMA_F8_32X32X64   = 7
+} rocwmma_amd_mfma_shape;
+
+/*
+ * Matrix-pipe ceiling probe: every SIMD of the device runs `waves_per_simd` (1 or 2) waves that
+ * issue nothing but matrix instructions of `shape` on operands held in registers, 32 instructions
+ * per trip, `trips` trips.  The operand registers are filled from `operands`, a 64 KiB table of
+ * operand bits the caller chooses (all zero, or the bit patterns of the data distribution of
+ * interest): the sustained rate depends on them because the part is power managed.
+ * `out` receives one float per launched lane (256 x waves_per_simd x compute units).  *ops is set
+ * to the number of floating-point (integer) operations of the launch (2 per multiply-add).
+ * Has no counterpart in the reference, whose efficiency figure divides by a nominal peak
+ * (test/performance.hpp:435-442).
+ */
+int rocwmma_amd_bench_mfma_ceiling(int         shape,
+                                   uint32_t    trips,
+                                   uint32_t    waves_per_simd,
+                                   const void* operands,
+                                   float*      out,
+                                   double*     ops,
+                                   void*       stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ROCWMMA_AMD_AUX_H */

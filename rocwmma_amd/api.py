@@ -18,8 +18,12 @@ GEMM_AUTO, GEMM_WAVE_TILE, GEMM_BLOCKED, GEMM_BLOCKED_256 = 0, 1, 2, 3
 EXPORTS = [
     "rocwmma_amd_version", "rocwmma_amd_status_string", "rocwmma_amd_device_info", "rocwmma_amd_gemm",
     "rocwmma_amd_gemm_ex", "rocwmma_amd_gemv", "rocwmma_amd_dlrm_fwd", "rocwmma_amd_dlrm_bwd",
-    "rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm",
 ]
+# librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
+_AUX_LIB_NAME = "librocwmma_amd_aux.so"
+AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_bench_mfma_ceiling"]
+(MFMA_F16_16X16X32, MFMA_F16_32X32X16, MFMA_BF16_16X16X32, MFMA_BF16_32X32X16, MFMA_I8_16X16X64, MFMA_I8_32X32X32,
+ MFMA_F8_16X16X128, MFMA_F8_32X32X64) = range(8)
 
 
 class RocwmmaError(RuntimeError):
@@ -61,12 +65,34 @@ def library():
         L.rocwmma_amd_dlrm_fwd.restype = i
         L.rocwmma_amd_dlrm_bwd.argtypes = [vp, vp, vp, vp, u, u, u, vp]
         L.rocwmma_amd_dlrm_bwd.restype = i
+        _lib = L
+    return _lib
+
+
+def aux_library_path():
+    return os.path.join(HERE, _AUX_LIB_NAME)
+
+
+_aux = None
+
+
+def aux_library():
+    """Loads the test / benchmark support library (self-test kernels, measurement probes)."""
+    global _aux
+    if _aux is None:
+        path = aux_library_path()
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `python rocwmma_amd/build.py`")
+        L = ctypes.CDLL(path)
+        i, u, vp, f = ctypes.c_int, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_float
         L.rocwmma_amd_selftest_roundtrip.argtypes = [i, i, i, i, i, i, u, u, vp, vp, u, vp]
         L.rocwmma_amd_selftest_roundtrip.restype = i
         L.rocwmma_amd_selftest_coop_gemm.argtypes = [i, i, u, u, u, vp, vp, vp, vp, f, f, vp]
         L.rocwmma_amd_selftest_coop_gemm.restype = i
-        _lib = L
-    return _lib
+        L.rocwmma_amd_bench_mfma_ceiling.argtypes = [i, u, u, vp, vp, ctypes.POINTER(ctypes.c_double), vp]
+        L.rocwmma_amd_bench_mfma_ceiling.restype = i
+        _aux = L
+    return _aux
 
 
 def version():
@@ -145,12 +171,20 @@ def dlrm_bwd(inp, upstream, grad, mlp_grad, m, k, batch):
 
 
 def selftest_roundtrip(context, dtype, layout, block, blockk, coop, rows, cols, inp, out, ld):
-    _check(library().rocwmma_amd_selftest_roundtrip(context, dtype, layout, block, blockk, int(coop), rows, cols,
+    _check(aux_library().rocwmma_amd_selftest_roundtrip(context, dtype, layout, block, blockk, int(coop), rows, cols,
                                                     _ptr(inp), _ptr(out), ld, _stream()), "selftest_roundtrip")
     return out
 
 
 def selftest_coop_gemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta):
-    _check(library().rocwmma_amd_selftest_coop_gemm(layout_a, layout_b, m, n, k, _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+    _check(aux_library().rocwmma_amd_selftest_coop_gemm(layout_a, layout_b, m, n, k, _ptr(a), _ptr(b), _ptr(c), _ptr(d),
                                                     alpha, beta, _stream()), "selftest_coop_gemm")
     return d
+
+
+def bench_mfma_ceiling(shape, trips, waves_per_simd, operands, out):
+    """Launches the matrix-pipe ceiling probe; returns the operation count of the launch."""
+    ops = ctypes.c_double(0.0)
+    _check(aux_library().rocwmma_amd_bench_mfma_ceiling(shape, trips, waves_per_simd, _ptr(operands), _ptr(out),
+                                                        ctypes.byref(ops), _stream()), "bench_mfma_ceiling")
+    return ops.value

@@ -13,10 +13,6 @@ namespace rocwmma_amd
     int launchDlrmFwd(const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, hipStream_t stream);
     int launchDlrmBwd(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t k,
                       uint32_t batch, hipStream_t stream);
-    int selftestRoundtrip(int context, int dtype, int layout, int block, int blockk, int coop, uint32_t rows, uint32_t cols,
-                          const void* in, void* out, uint32_t ld, hipStream_t stream);
-    int selftestCoopGemm(int layoutA, int layoutB, uint32_t m, uint32_t n, uint32_t k, const void* a, const void* b,
-                         const float* c, float* d, float alpha, float beta, hipStream_t stream);
 
     namespace
     {
@@ -307,48 +303,6 @@ int rocwmma_amd_dlrm_bwd(const void* input,
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
     return launchDlrmBwd(input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
-}
-
-int rocwmma_amd_selftest_roundtrip(int         context,
-                                   int         dtype,
-                                   int         layout,
-                                   int         block,
-                                   int         blockk,
-                                   int         coop,
-                                   uint32_t    rows,
-                                   uint32_t    cols,
-                                   const void* in,
-                                   void*       out,
-                                   uint32_t    ld,
-                                   void*       stream)
-{
-    if(!in || !out || rows == 0u || cols == 0u || !validLayout(layout))
-        return ROCWMMA_AMD_INVALID_ARGUMENT;
-    if(!aligned16(in) || !aligned16(out) || (ld * dtypeSize(dtype)) % 16u != 0u)
-        return ROCWMMA_AMD_BAD_ALIGNMENT;
-    if(!isGfx950Current())
-        return ROCWMMA_AMD_NO_DEVICE;
-    return selftestRoundtrip(context, dtype, layout, block, blockk, coop, rows, cols, in, out, ld, asStream(stream));
-}
-
-int rocwmma_amd_selftest_coop_gemm(int          layout_a,
-                                   int          layout_b,
-                                   uint32_t     m,
-                                   uint32_t     n,
-                                   uint32_t     k,
-                                   const void*  a,
-                                   const void*  b,
-                                   const float* c,
-                                   float*       d,
-                                   float        alpha,
-                                   float        beta,
-                                   void*        stream)
-{
-    if(!a || !b || !c || !d || !validLayout(layout_a) || !validLayout(layout_b))
-        return ROCWMMA_AMD_INVALID_ARGUMENT;
-    if(!isGfx950Current())
-        return ROCWMMA_AMD_NO_DEVICE;
-    return selftestCoopGemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta, asStream(stream));
 }
 
 } // extern "C"

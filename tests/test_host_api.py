@@ -20,14 +20,29 @@ def lib():
     return rw.library()
 
 
-def test_exports_every_declared_symbol(lib):
-    header = open(os.path.join(ROOT, "include", "rocwmma_amd.h")).read()
+def _declared(header_name):
+    header = open(os.path.join(ROOT, "include", header_name)).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)  # declarations only, not prose
-    declared = set(re.findall(r"\b(rocwmma_amd_[a-z0-9_]+)\s*\(", header))
+    return set(re.findall(r"\b(rocwmma_amd_[a-z0-9_]+)\s*\(", header))
+
+
+def test_exports_every_declared_symbol(lib):
+    declared = _declared("rocwmma_amd.h")
     assert declared, "no declarations found"
     for name in sorted(declared):
         assert hasattr(lib, name), f"{name} declared in include/rocwmma_amd.h but not exported"
     assert declared == set(rw.api.EXPORTS)
+
+
+def test_aux_library_exports_every_declared_symbol_and_product_library_none_of_them(lib):
+    """Test and benchmark support lives in a library of its own, not in the product ABI."""
+    aux = rw.aux_library()
+    declared = _declared("rocwmma_amd_aux.h")
+    assert declared == set(rw.api.AUX_EXPORTS)
+    for name in sorted(declared):
+        assert hasattr(aux, name), f"{name} declared in include/rocwmma_amd_aux.h but not exported"
+        with pytest.raises(AttributeError):
+            getattr(lib, name)
 
 
 def test_version_and_status_strings(lib):
