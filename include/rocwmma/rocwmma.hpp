@@ -356,23 +356,37 @@ namespace rocwmma
                       "blocks with an edge of 8 can be loaded, stored and filled but not multiplied");
         // The accumulator is kept transposed: the instruction's row operand is B, its column
         // operand is A (see fragment_map.hpp).
+        // Compute types narrower than 32 bits (f16, bf16, __half accumulators): the matrix cores
+        // accumulate in f32 only, so the accumulator is widened, multiplied and narrowed again in
+        // every call, as the reference does (library/include/rocwmma/internal/mfma_impl.hpp:108-155).
+        constexpr bool NarrowCompute = sizeof(ComputeT) < 4u;
+        using NativeT                = std::conditional_t<NarrowCompute, float32_t, ComputeT>;
         using Op = detail::Mfma<detail::TypeInfo<InputTB>::cls,
                                 detail::TypeInfo<InputTA>::cls,
-                                ComputeT,
+                                NativeT,
                                 MapAcc::tile,
                                 MapA::kpack>;
         static_assert(Op::supported,
                       "no gfx950 MFMA instruction for this combination of input types, "
                       "accumulator type, block size and BlockK");
         using Acc = typename Op::Acc;
-        static_assert(sizeof(Acc) == MapAcc::perBlock * sizeof(ComputeT), "accumulator block size mismatch");
+        static_assert(sizeof(Acc) == MapAcc::perBlock * sizeof(NativeT), "accumulator block size mismatch");
 
         Acc acc[MapAcc::nbi][MapAcc::nbj];
 #pragma unroll
         for(uint32_t bi = 0; bi < MapAcc::nbi; ++bi)
 #pragma unroll
             for(uint32_t bj = 0; bj < MapAcc::nbj; ++bj)
-                acc[bi][bj] = *reinterpret_cast<const Acc*>(&c.x[MapAcc::blockIndex(bi, bj) * MapAcc::perBlock]);
+            {
+                if constexpr(NarrowCompute)
+                {
+#pragma unroll
+                    for(uint32_t e = 0; e < MapAcc::perBlock; ++e)
+                        acc[bi][bj][e] = static_cast<float32_t>(c.x[MapAcc::blockIndex(bi, bj) * MapAcc::perBlock + e]);
+                }
+                else
+                    acc[bi][bj] = *reinterpret_cast<const Acc*>(&c.x[MapAcc::blockIndex(bi, bj) * MapAcc::perBlock]);
+            }
 
             // K outermost so consecutive instructions write different accumulators
 #pragma unroll
@@ -389,7 +403,16 @@ namespace rocwmma
         for(uint32_t bi = 0; bi < MapAcc::nbi; ++bi)
 #pragma unroll
             for(uint32_t bj = 0; bj < MapAcc::nbj; ++bj)
-                *reinterpret_cast<Acc*>(&d.x[MapAcc::blockIndex(bi, bj) * MapAcc::perBlock]) = acc[bi][bj];
+            {
+                if constexpr(NarrowCompute)
+                {
+#pragma unroll
+                    for(uint32_t e = 0; e < MapAcc::perBlock; ++e)
+                        d.x[MapAcc::blockIndex(bi, bj) * MapAcc::perBlock + e] = static_cast<ComputeT>(acc[bi][bj][e]);
+                }
+                else
+                    *reinterpret_cast<Acc*>(&d.x[MapAcc::blockIndex(bi, bj) * MapAcc::perBlock]) = acc[bi][bj];
+            }
 #else
         (void)d, (void)a, (void)b, (void)c;
 #endif // ROCWMMA_ARCH_GFX950

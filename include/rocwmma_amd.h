@@ -88,10 +88,11 @@ int rocwmma_amd_device_info(int* compute_units, int* clock_mhz, int* is_gfx950);
  * A is m x k, B is k x n, C and D are m x n; C and D share `layout_c`.
  * dtype_in  : element type of A and B (F16, BF16, E4M3, E5M2, I8, F32).
  * dtype_out : element type of C and D: F32 for the float inputs (F16 also allowed with F16
- *             inputs, BF16 with BF16 inputs), I32 for I8.  These are the Input/Output/Compute
+ *             inputs, BF16 with BF16 inputs), I32 or I8 for I8.  These are the Input/Output/Compute
  *             triples of the reference's GEMM tests (test/gemm/gemm_common_test_params.hpp:51-111).
  *             The compute type is f32 (i32 for I8); alpha and beta are converted to it (for I8
- *             they must be integers).
+ *             they must be integers).  I8 results keep the low eight bits of the 32-bit result, as
+ *             the reference's static_cast<int8_t> does (test/reference_impl.hpp:77-78).
  * c may be NULL when beta == 0.  c may equal d.
  * Shapes: m and n multiples of 16, k a multiple of 32 bytes' worth of elements per row is the
  * minimum every kernel accepts (k % 16 == 0 for 16-bit types, k % 32 == 0 for 8-bit types);

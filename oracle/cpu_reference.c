@@ -308,7 +308,9 @@ static inline size_t idx2(int layout, size_t row, size_t col, size_t ld)
 
 /* ---- GEMM: the reference loop nest verbatim (test/reference_impl.hpp:66-80) ---- */
 /* dtype_out: ORC_F32 (ComputeT f32) or ORC_I32 (ComputeT i32, dtype_in must be ORC_I8),
- * or ORC_F16 / ORC_BF16 (ComputeT f32, narrow output).  alpha/beta are passed as double
+ * or ORC_F16 / ORC_BF16 (ComputeT f32, narrow output), or ORC_I8 (ComputeT i32, narrow output:
+ * the reference's <int8, int8, int32> triple, static_cast<int8_t> of the 32-bit result, which
+ * keeps its low eight bits).  alpha/beta are passed as double
  * and converted to ComputeT, like the reference's by-value ComputeT arguments. */
 int oracle_gemm_naive(int         dtype_in,
                       int         dtype_out,
@@ -331,15 +333,14 @@ int oracle_gemm_naive(int         dtype_in,
     size_t ldc = layC == ORC_ROW_MAJOR ? n : m;
     size_t ldd = layD == ORC_ROW_MAJOR ? n : m;
     long   i;
-    if(dtype_out == ORC_I32)
+    if(dtype_out == ORC_I32 || dtype_out == ORC_I8)
     {
         if(dtype_in != ORC_I8)
             return -1;
-        const int8_t*  A  = (const int8_t*)a;
-        const int8_t*  B  = (const int8_t*)b;
-        const int32_t* C  = (const int32_t*)c;
-        int32_t*       D  = (int32_t*)d;
-        int32_t        al = (int32_t)alpha, be = (int32_t)beta;
+        const int     out8 = dtype_out == ORC_I8;
+        const int8_t* A    = (const int8_t*)a;
+        const int8_t* B    = (const int8_t*)b;
+        int32_t       al = (int32_t)alpha, be = (int32_t)beta;
 #pragma omp parallel for
         for(i = 0; i < (long)m; ++i)
             for(size_t j = 0; j < n; ++j)
@@ -347,10 +348,16 @@ int oracle_gemm_naive(int         dtype_in,
                 int32_t accum = 0;
                 for(size_t h = 0; h < k; ++h)
                     accum += (int32_t)A[idx2(layA, i, h, lda)] * (int32_t)B[idx2(layB, h, j, ldb)];
+                int32_t cv = 0;
+                if(c)
+                    cv = out8 ? (int32_t)((const int8_t*)c)[idx2(layC, i, j, ldc)]
+                              : ((const int32_t*)c)[idx2(layC, i, j, ldc)];
                 /* unsigned arithmetic: same two's-complement result, no UB on wrap */
-                D[idx2(layD, i, j, ldd)]
-                    = (int32_t)((uint32_t)al * (uint32_t)accum
-                                + (uint32_t)be * (uint32_t)(C ? C[idx2(layC, i, j, ldc)] : 0));
+                const uint32_t res = (uint32_t)al * (uint32_t)accum + (uint32_t)be * (uint32_t)cv;
+                if(out8)
+                    ((int8_t*)d)[idx2(layD, i, j, ldd)] = (int8_t)(uint8_t)(res & 0xffu);
+                else
+                    ((int32_t*)d)[idx2(layD, i, j, ldd)] = (int32_t)res;
             }
         return 0;
     }
@@ -477,8 +484,9 @@ static int gemm_fast_i32(int             layA,
                          uint32_t        k,
                          const int8_t*   A,
                          const int8_t*   B,
-                         const int32_t*  C,
-                         int32_t*        D,
+                         const void*     C,
+                         void*           D,
+                         int             out8, /* C and D hold int8 (low eight bits of the result) */
                          int32_t         al,
                          int32_t         be,
                          const uint32_t* rows,
@@ -523,10 +531,16 @@ static int gemm_fast_i32(int             layA,
                 size_t jend = j0 + JB < n ? JB : n - j0;
                 for(size_t jj = 0; jj < jend; ++jj)
                 {
-                    size_t j = j0 + jj;
-                    D[idx2(layD, i, j, ldd)]
-                        = (int32_t)((uint32_t)al * (uint32_t)acc[jj]
-                                    + (uint32_t)be * (uint32_t)(C ? C[idx2(layC, i, j, ldc)] : 0));
+                    size_t  j  = j0 + jj;
+                    int32_t cv = 0;
+                    if(C)
+                        cv = out8 ? (int32_t)((const int8_t*)C)[idx2(layC, i, j, ldc)]
+                                  : ((const int32_t*)C)[idx2(layC, i, j, ldc)];
+                    const uint32_t res = (uint32_t)al * (uint32_t)acc[jj] + (uint32_t)be * (uint32_t)cv;
+                    if(out8)
+                        ((int8_t*)D)[idx2(layD, i, j, ldd)] = (int8_t)(uint8_t)(res & 0xffu);
+                    else
+                        ((int32_t*)D)[idx2(layD, i, j, ldd)] = (int32_t)res;
                 }
             }
         }
@@ -554,13 +568,12 @@ int oracle_gemm_rows(int             dtype_in,
                      const uint32_t* rows,
                      uint32_t        nrows)
 {
-    if(dtype_out == ORC_I32)
+    if(dtype_out == ORC_I32 || dtype_out == ORC_I8)
     {
         if(dtype_in != ORC_I8)
             return -1;
-        return gemm_fast_i32(layA, layB, layC, layD, m, n, k, (const int8_t*)a, (const int8_t*)b,
-                             (const int32_t*)c, (int32_t*)d, (int32_t)alpha, (int32_t)beta, rows,
-                             nrows);
+        return gemm_fast_i32(layA, layB, layC, layD, m, n, k, (const int8_t*)a, (const int8_t*)b, c, d,
+                             dtype_out == ORC_I8, (int32_t)alpha, (int32_t)beta, rows, nrows);
     }
     if(dtype_out != ORC_F32 && dtype_out != ORC_F16 && dtype_out != ORC_BF16)
         return -1;

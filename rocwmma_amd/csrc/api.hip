@@ -63,7 +63,7 @@ namespace rocwmma_amd
                                  || (dtypeIn == ROCWMMA_AMD_F16 && dtypeOut == ROCWMMA_AMD_F16)
                                  || (dtypeIn == ROCWMMA_AMD_BF16 && dtypeOut == ROCWMMA_AMD_BF16)
                                  || (dtypeIn == ROCWMMA_AMD_F32 && dtypeOut == ROCWMMA_AMD_F32)
-                                 || (dtypeIn == ROCWMMA_AMD_I8 && dtypeOut == ROCWMMA_AMD_I32);
+                                 || (dtypeIn == ROCWMMA_AMD_I8 && (dtypeOut == ROCWMMA_AMD_I32 || dtypeOut == ROCWMMA_AMD_I8));
             if(!okTypes)
                 return ROCWMMA_AMD_UNSUPPORTED_TYPE;
             if(dtypeIn == ROCWMMA_AMD_I8 && (alpha != std::nearbyint(alpha) || beta != std::nearbyint(beta)))

@@ -912,6 +912,8 @@ namespace rocwmma_amd
             return pickLayout16<bfloat16_t, bfloat16_t, float32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         if(dtypeIn == ROCWMMA_AMD_I8 && dtypeOut == ROCWMMA_AMD_I32)
             return pickLayout8<int8_t, int32_t, int32_t>(layoutA, layoutB, g, stream, forceLargeTile);
+        if(dtypeIn == ROCWMMA_AMD_I8 && dtypeOut == ROCWMMA_AMD_I8)
+            return pickLayout8<int8_t, int8_t, int32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         if(dtypeIn == ROCWMMA_AMD_E4M3 && dtypeOut == ROCWMMA_AMD_F32)
             return pickLayout8<float8_t, float32_t, float32_t>(layoutA, layoutB, g, stream, forceLargeTile);
         if(dtypeIn == ROCWMMA_AMD_E5M2 && dtypeOut == ROCWMMA_AMD_F32)

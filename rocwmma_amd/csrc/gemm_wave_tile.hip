@@ -51,8 +51,9 @@ namespace rocwmma_amd
             FragAcc acc;
             fill_fragment(acc, static_cast<CompT>(0));
 
-            const InT*     aPtr  = a + MapA::fromMatrixCoord(make_coord2d(cRow, 0u), lda);
-            const InT*     bPtr  = b + MapB::fromMatrixCoord(make_coord2d(0u, cCol), ldb);
+            // (64-bit offsets of the block's first element: operands of 2^32 elements and more)
+            const InT*     aPtr  = a + (std::is_same<LA, row_major>::value ? static_cast<size_t>(cRow) * lda : cRow);
+            const InT*     bPtr  = b + (std::is_same<LB, row_major>::value ? cCol : static_cast<size_t>(cCol) * ldb);
             const uint32_t aStep = MapA::fromMatrixCoord(make_coord2d(0u, BK), lda);
             const uint32_t bStep = MapB::fromMatrixCoord(make_coord2d(BK, 0u), ldb);
 
@@ -69,8 +70,10 @@ namespace rocwmma_amd
             }
 
             FragC          fc;
-            const uint32_t cOff = layoutC == mem_row_major ? cRow * ldc + cCol : cCol * ldc + cRow;
-            const uint32_t dOff = layoutC == mem_row_major ? cRow * ldd + cCol : cCol * ldd + cRow;
+            const size_t   cOff = layoutC == mem_row_major ? static_cast<size_t>(cRow) * ldc + cCol
+                                                           : static_cast<size_t>(cCol) * ldc + cRow;
+            const size_t   dOff = layoutC == mem_row_major ? static_cast<size_t>(cRow) * ldd + cCol
+                                                           : static_cast<size_t>(cCol) * ldd + cRow;
             if(beta != static_cast<CompT>(0))
             {
                 load_matrix_sync(fc, c + cOff, ldc, layoutC);
@@ -155,6 +158,9 @@ namespace rocwmma_amd
 
     int launchGemmWaveTile(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream)
     {
+        // the per-step pointer increments along K are 32-bit element counts (BlockK * ld at most)
+        if(static_cast<uint64_t>(g.lda) * 256u >= (1ull << 32) || static_cast<uint64_t>(g.ldb) * 256u >= (1ull << 32))
+            return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
         if(dtypeIn == ROCWMMA_AMD_F16 && dtypeOut == ROCWMMA_AMD_F32)
             return pickLayout<float16_t, float32_t, float32_t, 32, 16>(layoutA, layoutB, g, stream);
         if(dtypeIn == ROCWMMA_AMD_F16 && dtypeOut == ROCWMMA_AMD_F16)
@@ -171,6 +177,8 @@ namespace rocwmma_amd
             return pickLayout<bfloat8_t, float32_t, float32_t, 128, 64>(layoutA, layoutB, g, stream);
         if(dtypeIn == ROCWMMA_AMD_I8 && dtypeOut == ROCWMMA_AMD_I32)
             return pickLayout<int8_t, int32_t, int32_t, 64, 32>(layoutA, layoutB, g, stream);
+        if(dtypeIn == ROCWMMA_AMD_I8 && dtypeOut == ROCWMMA_AMD_I8)
+            return pickLayout<int8_t, int8_t, int32_t, 64, 32>(layoutA, layoutB, g, stream);
         return ROCWMMA_AMD_UNSUPPORTED_TYPE;
     }
 

@@ -162,6 +162,11 @@ _MATRIX_TYPES = [
     (("f64", "f64", "f64"), [(16, 4), (16, 8), (16, 16)]),
     (("h16", "f32", "f32"), [(16, 32), (32, 16)]),
     (("h16", "h16", "f32"), [(16, 16), (32, 8)]),
+    # narrow outputs and 16-bit compute types (test/gemm/gemm_common_test_params.hpp:51-56,88-113)
+    (("i8", "i8", "i32"), [(16, 64), (32, 32)]),
+    (("f16", "f16", "f16"), [(16, 32), (32, 16)]),
+    (("bf16", "bf16", "bf16"), [(16, 32), (32, 8)]),
+    (("h16", "h16", "h16"), [(16, 16), (32, 16)]),
 ]
 _CONFIGS = ["Block::LdsNT", "Block::LdsTN", "Block::LdsRF", "Wave::LdsNT", "Wave::LdsTN", "Wg::LdsNT", "Wg::LdsTN"]
 _BLOCKS = [(1, 1), (2, 2), (1, 2), (2, 1), (4, 2), (2, 4), (4, 4), (1, 4)]

@@ -35,6 +35,8 @@ def run_gemm(dtype_in, dtype_out, la, lb, lc, m, n, k, a, b, c, alpha, beta, alg
         d0 = np.full(m * n, np.nan, dtype=np.float32)
     elif dtype_out == orc.I32:
         d0 = np.full(m * n, -123456789, dtype=np.int32)
+    elif dtype_out == orc.I8:
+        d0 = np.full(m * n, 0x55, dtype=np.int8)
     else:
         d0 = np.full(m * n, 0x7E00, dtype=np.uint16)
     d = to_device(d0)
@@ -76,6 +78,23 @@ def test_narrow_output_and_f32_type_combinations(dtype_in, dtype_out, tol, la, l
     got = run_gemm(dtype_in, dtype_out, la, lb, RM, m, n, k, a, b, c if beta else None, 1.5, beta, algo)
     want = orc.gemm(dtype_in, dtype_out, la, lb, RM, RM, m, n, k, a, b, c if beta else None, 1.5, beta)
     check(dtype_in, dtype_out, got, want, tol)
+
+
+@pytest.mark.parametrize("algo", ALGOS + [rw.GEMM_AUTO])
+@pytest.mark.parametrize("lc", [RM, CM])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (3.0, -2.0)])
+def test_int8_output_triple(algo, lc, alpha, beta):
+    """<int8, int8, int32> (test/gemm/gemm_common_test_params.hpp:51-56): 32-bit compute, C and D in
+    int8; the result keeps the low eight bits of alpha * acc + beta * c.  Bit-exact.  Entries are
+    small so that most results stay inside the int8 range and a lost bit anywhere shows."""
+    m, n, k = 256, 256, 256
+    rng = np.random.default_rng(61)
+    a = rng.integers(-3, 4, size=m * k, dtype=np.int8)
+    b = rng.integers(-3, 4, size=k * n, dtype=np.int8)
+    c = rng.integers(-128, 128, size=m * n, dtype=np.int8)
+    got = run_gemm(orc.I8, orc.I8, RM, CM, lc, m, n, k, a, b, c if beta else None, alpha, beta, algo)
+    want = orc.gemm(orc.I8, orc.I8, RM, CM, lc, lc, m, n, k, a, b, c if beta else None, alpha, beta)
+    assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} elements differ"
 
 
 # ---------------------------------------------------------------- config 1: simple_hgemm workload

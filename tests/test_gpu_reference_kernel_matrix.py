@@ -22,13 +22,15 @@ and 32 and the reference's problem sizes; inputs are -1, 0, 1 so results must eq
 
 tests/dropin/build_samples.py enumerates the cases and builds the executables
 on the development machine (where the reference checkout is); they travel with the tree.  Where
-they are absent the tests are skipped."""
+they are absent the tests fail (ROCWMMA_AMD_REQUIRE_DROPIN=0 skips them instead)."""
 import os
 import re
 import subprocess
 import sys
 
 import pytest
+
+from util import dropin_missing
 
 pytestmark = pytest.mark.gpu
 
@@ -43,7 +45,7 @@ BIN = os.path.join(HERE, "dropin", "_bin")
 def test_reference_cooperative_gemm_kernel_matrix(unit):
     exe = os.path.join(BIN, f"coop_gemm_matrix_{unit}")
     if not os.path.exists(exe):
-        pytest.skip("kernel-matrix executables not built on this machine (tests/dropin/build_samples.py)")
+        dropin_missing("kernel-matrix executables")
     expected = len(build_samples.coop_gemm_units()[unit][1])
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
     tail = res.stdout[-2000:]
@@ -63,7 +65,7 @@ def test_reference_cooperative_gemm_kernel_matrix(unit):
 def test_reference_unit_test_kernels(unit):
     exe = os.path.join(BIN, f"unit_kernels_{unit}")
     if not os.path.exists(exe):
-        pytest.skip("unit-kernel executables not built on this machine (tests/dropin/build_samples.py)")
+        dropin_missing("unit-kernel executables")
     expected = len(build_samples.unit_kernel_units()[unit][1])
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
     tail = res.stdout[-2000:]
@@ -81,7 +83,7 @@ def test_reference_unit_test_kernels(unit):
 def test_reference_dlrm_test_kernels():
     exe = os.path.join(BIN, "dlrm_kernels")
     if not os.path.exists(exe):
-        pytest.skip("DLRM kernel executable not built on this machine (tests/dropin/build_samples.py)")
+        dropin_missing("DLRM kernel executable")
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
     tail = res.stdout[-2000:]
     failed = [line for line in res.stdout.splitlines() if line.startswith("FAILED")]

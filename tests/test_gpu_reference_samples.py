@@ -3,11 +3,13 @@ headers by tests/dropin/build_samples.py, run and validate themselves (each samp
 GPU result with its own CPU code and prints PASSED or FAILED).
 
 The executables are built on the development machine (where the reference checkout is) and
-travel with the tree; where they are absent the tests are skipped."""
+travel with the tree; where they are absent the tests fail (ROCWMMA_AMD_REQUIRE_DROPIN=0 skips them instead)."""
 import os
 import subprocess
 
 import pytest
+
+from util import dropin_missing
 
 pytestmark = pytest.mark.gpu
 
@@ -23,7 +25,7 @@ SAMPLES = {"simple_hgemm": 1, "perf_hgemm": 1, "simple_sgemv": 1, "simple_dlrm":
 def test_reference_sample_runs_and_validates_itself(sample):
     exe = os.path.join(BIN, sample)
     if not os.path.exists(exe):
-        pytest.skip("sample executables not built on this machine (tests/dropin/build_samples.py)")
+        dropin_missing("sample executables")
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
     tail = res.stdout[-1500:]
     assert res.returncode == 0, tail

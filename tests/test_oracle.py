@@ -209,6 +209,25 @@ def test_gemm_int8_exact_against_int64():
     assert np.array_equal(d.reshape(m, n).astype(np.int64), want)
 
 
+def test_gemm_int8_output_keeps_low_byte_against_int64():
+    """<int8, int8, int32>: D = int8(alpha * acc + beta * c) keeps the low eight bits of the exact
+    integer result (two's complement), for the fast and the verbatim loop alike and in both C/D
+    layouts; the saturating alternative differs on this data, so the check has teeth."""
+    rng = np.random.default_rng(15)
+    m, n, k = 24, 40, 96
+    A = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    B = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    C = rng.integers(-128, 128, (m, n), dtype=np.int8)
+    exact = 3 * (A.astype(np.int64) @ B.astype(np.int64)) - 2 * C.astype(np.int64)
+    want = ((exact + 128) % 256 - 128).astype(np.int8)
+    assert not np.array_equal(want, np.clip(exact, -128, 127).astype(np.int8))
+    for lc in (RM, CM):
+        for naive in (False, True):
+            d = orc.gemm(orc.I8, orc.I8, RM, CM, lc, lc, m, n, k, A, _store(B, CM), _store(C, lc), 3, -2, naive=naive)
+            got = d.reshape(m, n) if lc == RM else d.reshape(n, m).T
+            assert np.array_equal(got, want)
+
+
 def test_gemm_accumulation_order_is_sequential_f32():
     """Pins 'one f32 accumulator, increasing h, separate multiply and add' against a
     pure-Python loop on a case where the order matters (large cancellation)."""

@@ -62,3 +62,18 @@ def tol_for(dtype_in):
     if dtype_in == orc.I8:
         return 0.0
     return 1e-3
+
+
+def dropin_missing(what):
+    """The drop-in executables are built where the reference checkout is (tests/dropin/build_samples.py) and
+    travel with the tree, so on a GPU box their absence is an error, not a reason to skip: a tree
+    without them would otherwise pass with the drop-in proof silently left out.
+    ROCWMMA_AMD_REQUIRE_DROPIN=0 turns the failure into a skip (a checkout without the reference)."""
+    import os
+
+    import pytest
+
+    msg = f"{what} not built (tests/dropin/build_samples.py, needs the reference checkout)"
+    if os.environ.get("ROCWMMA_AMD_REQUIRE_DROPIN", "1") == "0":
+        pytest.skip(msg)
+    pytest.fail(msg + "; set ROCWMMA_AMD_REQUIRE_DROPIN=0 to skip instead")
