@@ -15,7 +15,8 @@
  *     was launched.  The reference's hosts exit() on HIP errors (samples/common.hpp:34-46) and
  *     print "Unsupported size!" for shapes they reject (samples/simple_hgemm.cpp:144-149);
  *     here both become status codes;
- *   - no global mutable state: calls are re-entrant and thread safe.
+ *   - calls are re-entrant and thread safe; the only state the library keeps is a per-device cache
+ *     of immutable device properties (compute-unit count, architecture).
  */
 #ifndef ROCWMMA_AMD_H
 #define ROCWMMA_AMD_H
@@ -183,7 +184,7 @@ int rocwmma_amd_gemv(uint32_t    m,
  *            with Z = input[b] * input[b]^T.
  * Unlike the reference kernel this one needs no f32 m x m scratch (`acc`) and accepts any
  * m <= 32 (the reference GPU kernels need m % 16 == 0, test/dlrm/dlrm_kernel_base_impl.hpp:146-150).
- * k must be a multiple of 16 and at most 256; input must be 16-byte aligned.
+ * k must be 32, 64, 128 or 256; input and output must be 16-byte aligned.
  */
 int rocwmma_amd_dlrm_fwd(const void* input,
                          void*       output,

@@ -41,24 +41,21 @@ namespace rocwmma_amd
             return (row * (row - 1u)) / 2u + col;
         }
 
-        // Copies `halves` f16 values from LDS (16-byte aligned) to global (16-byte aligned),
-        // whole workgroup, 16-byte accesses with a 2-byte tail.
+        // Copies `halves` f16 values from LDS to global, whole workgroup.  `dst` is 2-byte aligned in
+        // general (rows of odd width); the caller stages the data at an LDS address congruent to `dst`
+        // modulo 16, so the 16-byte pieces are aligned on both sides and only the few halves in
+        // front of the first and behind the last whole piece move one by one.
         ROCWMMA_DEVICE inline void copyOut(float16_t* dst, const float16_t* ldsSrc, uint32_t halves)
         {
-            const uint32_t vecs = halves / 8u;
+            const uint32_t misalign = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst) & 15u) / 2u;
+            const uint32_t head     = min(halves, (8u - misalign) & 7u);
+            const uint32_t vecs     = (halves - head) / 8u;
             for(uint32_t i = threadIdx.x; i < vecs; i += blockDim.x)
-                reinterpret_cast<u32x4_t*>(dst)[i] = reinterpret_cast<const u32x4_t*>(ldsSrc)[i];
-            for(uint32_t i = vecs * 8u + threadIdx.x; i < halves; i += blockDim.x)
+                reinterpret_cast<u32x4_t*>(dst + head)[i] = reinterpret_cast<const u32x4_t*>(ldsSrc + head)[i];
+            for(uint32_t i = threadIdx.x; i < head; i += blockDim.x)
                 dst[i] = ldsSrc[i];
-        }
-
-        ROCWMMA_DEVICE inline void copyIn(float16_t* ldsDst, const float16_t* src, uint32_t halves)
-        {
-            const uint32_t vecs = halves / 8u;
-            for(uint32_t i = threadIdx.x; i < vecs; i += blockDim.x)
-                reinterpret_cast<u32x4_t*>(ldsDst)[i] = reinterpret_cast<const u32x4_t*>(src)[i];
-            for(uint32_t i = vecs * 8u + threadIdx.x; i < halves; i += blockDim.x)
-                ldsDst[i] = src[i];
+            for(uint32_t i = head + vecs * 8u + threadIdx.x; i < halves; i += blockDim.x)
+                dst[i] = ldsSrc[i];
         }
 
         // The feature rows of a workgroup's samples are contiguous in global memory
@@ -124,11 +121,14 @@ namespace rocwmma_amd
             const uint32_t width     = K + (m * (m - 1u)) / 2u;
             const uint32_t tileBytes = (((Samples - 1u) * m + kMaxM) * Tile::rowBytes + 1023u) & ~1023u;
             char*          ldsIn     = ldsRaw;
-            float16_t*     ldsOut    = reinterpret_cast<float16_t*>(ldsRaw + tileBytes);
+            const uint32_t sample0   = blockIdx.x * Samples;
+            // the output block of the workgroup's samples, staged at an LDS address congruent to its
+            // global address modulo 16 (see copyOut)
+            float16_t* const outBlock = output + static_cast<size_t>(sample0) * width;
+            float16_t*       ldsOut   = reinterpret_cast<float16_t*>(ldsRaw + tileBytes + (reinterpret_cast<uintptr_t>(outBlock) & 15u));
 
             const uint32_t lane    = threadIdx.x & 63u;
             const uint32_t wave    = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-            const uint32_t sample0 = blockIdx.x * Samples;
             const uint32_t nHere   = min(Samples, batch - sample0);
 
             // all feature rows of the workgroup's samples: one contiguous block
@@ -158,30 +158,52 @@ namespace rocwmma_amd
                     mma_sync(acc, fa[ks], applyTranspose(fa[ks]), acc);
 
                 float16_t* out = ldsOut + wave * width;
-                // bottom-MLP row: the lanes holding row 0 copy their operand registers
-                if(row == 0u)
+                // bottom-MLP row: the sample's first feature row, copied from the LDS tile by the whole
+                // wave (the output row starts on a 2-byte boundary only, so halves move one by one)
                 {
+                    const uint32_t   R0   = wave * m;
+                    const float16_t* row0 = reinterpret_cast<const float16_t*>(ldsIn + R0 * Tile::rowBytes);
+                    const uint32_t   swz0 = Tile::chunkSwizzle(R0);
 #pragma unroll
-                    for(uint32_t ks = 0; ks < KSteps; ++ks)
-#pragma unroll
-                        for(uint32_t j = 0; j < 8u; ++j)
-                            out[ks * 16u + kGroup * 8u + j] = fa[ks].x[j];
+                    for(uint32_t e = lane; e < K; e += 64u)
+                        out[e] = row0[(((e / 8u) ^ swz0) << 3) + e % 8u];
                 }
-                // strict lower triangle, row by row
+                // strict lower triangle, row by row.  Every lane writes all of its 16 values, those
+                // outside the triangle into a spare half behind the output block, so the writes issue
+                // back to back instead of one per branch.
+                const uint32_t rowStart = K + (row * (row - 1u)) / 2u;
+                const uint32_t spare    = (Samples - wave) * width + wave; // behind the last sample's row
 #pragma unroll
                 for(uint32_t e = 0; e < FragAcc::num_elements; ++e)
                 {
-                    const uint32_t r = AccMap::rowOf(e, lane);
                     const uint32_t c = AccMap::colOf(e, lane);
-                    if(r < m && c < r)
-                        out[K + trilIndex(r, c)] = static_cast<float16_t>(acc.x[e]);
+                    out[(row < m && c < row) ? rowStart + c : spare] = static_cast<float16_t>(acc.x[e]);
                 }
             }
             __syncthreads();
-            copyOut(output + static_cast<size_t>(sample0) * width, ldsOut, nHere * width);
+            copyOut(outBlock, ldsOut, nHere * width);
         }
 
         // ------------------------------------------------------------------ backward
+        // LDS staging of the gradient: the m x K result of a sample replaces its feature rows.  A lane
+        // writes runs of four columns of one row (8 bytes); the 32 lanes of a half-wave hold 32
+        // consecutive rows at the same column, which in a plain row-major stage are 32 addresses
+        // one row pitch apart: one bank.  The 8-byte units of LDS row R are therefore stored at unit
+        // position u ^ (R % units), and the write-out, which moves 16 bytes (two units whose positions
+        // differ in bit 0 only), reads them back and swaps the pair where R is odd.
+        template <uint32_t K>
+        struct GradStage
+        {
+            static constexpr uint32_t rowBytes = K * 2u;
+            static constexpr uint32_t units    = K / 4u; // 8-byte units per row
+            static constexpr uint32_t mask     = (units < 32u ? units : 32u) - 1u;
+
+            ROCWMMA_DEVICE static inline uint32_t unitOffset(uint32_t R, uint32_t unit)
+            {
+                return R * rowBytes + ((unit ^ (R & mask)) << 3);
+            }
+        };
+
         template <uint32_t K, uint32_t Samples>
         __global__ void __launch_bounds__(64 * Samples) dlrmBwdKernel(const float16_t* __restrict__ input,
                                                                            const float16_t* __restrict__ upstream,
@@ -192,6 +214,7 @@ namespace rocwmma_amd
         {
             constexpr uint32_t NBlocks = K / 32u; // 32-column blocks of the m x K result
             using Tile                 = FeatureTile<K>;
+            using Stage                = GradStage<K>;
             using FragG                = fragment<matrix_a, 32, 32, 16, float16_t, row_major>;
             using FragF                = fragment<matrix_b, 32, 32, 16, float16_t, row_major>;
             using FragAcc              = fragment<accumulator, 32, 32, 16, float32_t>;
@@ -208,18 +231,45 @@ namespace rocwmma_amd
             const uint32_t sample0 = blockIdx.x * Samples;
             const uint32_t nHere   = min(Samples, batch - sample0);
 
-            // Rows past the last sample are read as contraction rows >= m (multiplied by the zero
-            // columns of G): they must hold finite values, so clear everything behind the features
-            // first (the tail of the last partial copy is out of the buffer's bounds and reads zeros).
+            // features: direct copies, segment-swizzled for the transposing reads.  (Rows behind the
+            // last sample are never copied: whatever the LDS holds there only meets contraction indices
+            // >= m, which are masked out of the operand registers below.)
             const uint32_t featBytes = nHere * m * Tile::rowBytes;
-            for(uint32_t i = featBytes / 16u + threadIdx.x; i < tileBytes / 16u; i += blockDim.x)
-                reinterpret_cast<u32x4_t*>(ldsF)[i] = u32x4_t{0u, 0u, 0u, 0u};
-            // features: direct copies, segment-swizzled for the transposing reads
             Tile::template asyncLoad<true>(ldsF, input + static_cast<size_t>(sample0) * m * K, featBytes, wave, Samples, lane);
-            // upstream gradients (contiguous for the workgroup's samples)
-            copyIn(ldsUp, upstream + static_cast<size_t>(sample0) * width, nHere * width);
+            // upstream gradients (contiguous for the workgroup's samples): direct copies of 4 bytes per
+            // lane (the first sample of a workgroup has an even index, so the block starts on a 4-byte
+            // boundary whatever the row width).  An odd number of samples of odd width leaves two bytes
+            // behind the last whole word: no lane copies that word (nothing is read past the end of the
+            // caller's array), one lane moves the last half by hand.
+            {
+                const uint32_t        upBytes = nHere * width * 2u;
+                const uint32_t        whole   = upBytes & ~3u;
+                const float16_t*      upBlock = upstream + static_cast<size_t>(sample0) * width;
+                const lds::BufferRsrc rsrc
+                    = __builtin_amdgcn_make_buffer_rsrc(const_cast<float16_t*>(upBlock), 0, static_cast<int>(whole), 0x00020000);
+                for(uint32_t copy = wave; copy * 256u < whole; copy += Samples)
+                    if(copy * 256u + lane * 4u < whole)
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds::LdsPtr)(reinterpret_cast<char*>(ldsUp) + copy * 256u), 4,
+                                                                 static_cast<int>(copy * 256u + lane * 4u), 0, 0, 2 /* nt */);
+                if(whole != upBytes && threadIdx.x == 0u)
+                    ldsUp[whole / 2u] = upBlock[whole / 2u];
+            }
             lds::waitCopiesAndReads<0>();
             __syncthreads();
+
+            // bottom-MLP gradient = the first K entries of every upstream row; a row starts on a 2-byte
+            // boundary only, so it is read as halves.  Issued first: the stores drain under the arithmetic.
+            for(uint32_t i = threadIdx.x; i < nHere * (K / 8u); i += blockDim.x)
+            {
+                const uint32_t   s   = i / (K / 8u);
+                const uint32_t   c8  = i % (K / 8u);
+                const float16_t* src = ldsUp + s * width + c8 * 8u;
+                float16_t        tmp[8];
+#pragma unroll
+                for(uint32_t j = 0; j < 8u; ++j)
+                    tmp[j] = src[j];
+                reinterpret_cast<u32x4_t*>(mlpGrad + static_cast<size_t>(sample0 + s) * K)[c8] = *reinterpret_cast<u32x4_t*>(tmp);
+            }
 
             FragAcc acc[NBlocks];
             if(wave < nHere)
@@ -228,28 +278,35 @@ namespace rocwmma_amd
                 const uint32_t   kGroup = lane >> 5;
                 const float16_t* up     = ldsUp + wave * width;
 
-                // G operand: row `row`, columns ks*16 + kGroup*8 + j, rebuilt from the packed triangle
+                // G operand: row `row`, columns ks*16 + kGroup*8 + j, rebuilt from the packed triangle.
+                // Every lane reads all of its 16 entries (a harmless address where there is none) and
+                // selects afterwards, so the reads issue back to back instead of one per branch.
                 FragG fg[2];
+                // packed position of G(row, c): below the diagonal the row's entries are consecutive
+                // (tri(row) + c); above it entry (c, row) sits at tri(c) + row with tri(c + 1) = tri(c) + c
+                const uint32_t below = K + (row * (row - 1u)) / 2u;
 #pragma unroll
                 for(uint32_t ks = 0; ks < 2u; ++ks)
+                {
+                    const uint32_t c0    = ks * 16u + kGroup * 8u;
+                    uint32_t       above = K + (c0 * (c0 - 1u)) / 2u + row; // (c0 = 0: the product wraps to 0)
 #pragma unroll
                     for(uint32_t j = 0; j < 8u; ++j)
                     {
-                        const uint32_t c  = ks * 16u + kGroup * 8u + j;
-                        const uint32_t hi = row > c ? row : c;
-                        const uint32_t lo = row > c ? c : row;
-                        float16_t      g  = static_cast<float16_t>(0);
-                        if(hi < m && hi != lo)
-                            g = up[K + trilIndex(hi, lo)];
-                        fg[ks].x[j] = g;
+                        const uint32_t c     = c0 + j;
+                        const bool     there = (c > row ? c : row) < m && c != row;
+                        const float16_t g    = up[there ? (c < row ? below + c : above) : 0u];
+                        fg[ks].x[j]          = there ? g : static_cast<float16_t>(0);
+                        above += c;
                     }
+                }
 
                 // F operands: transposing reads, lane l gets column nb*32 + l%32 and contraction
                 // rows ks*16 + (l/32)*8 + 0..7 of this sample
                 const uint32_t group   = lane >> 4;
                 const uint32_t s16     = lane & 15u;
                 const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds::LdsPtr)ldsF));
-                FragF          ff[NBlocks][2];
+                uint32_t       ff[NBlocks][2][4]; // [block][k step][two halves per word]
 #pragma unroll
                 for(uint32_t nb = 0; nb < NBlocks; ++nb)
 #pragma unroll
@@ -262,27 +319,52 @@ namespace rocwmma_amd
                             const uint32_t seg  = nb * 2u + (group & 1u);
                             const uint32_t addr = ldsBase + R * Tile::rowBytes + ((seg ^ Tile::segmentSwizzle(R)) << 5)
                                                   + ((s16 & 3u) << 3);
-                            s16x4_t v;
+                            typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+                            u32x2_t v;
                             asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
-                            reinterpret_cast<s16x4_t*>(ff[nb][ks].x)[kk] = v;
+                            ff[nb][ks][2u * kk]      = v[0];
+                            ff[nb][ks][2u * kk + 1u] = v[1];
                         }
-                lds::waitReads();
-                __builtin_amdgcn_sched_barrier(0);
+                // Contraction rows >= m are the next sample's features (or stale LDS): G is zero there,
+                // but 0 * Inf and 0 * NaN are NaN, so those operand halves are cleared, which keeps
+                // the samples independent of one another as in the reference's CPU loops
+                // (test/reference_impl.hpp:121-179).  Word w of step ks holds contraction indices
+                // ks*16 + (l/32)*8 + 2w, + 1.
+                uint32_t keep[2][4];
+#pragma unroll
+                for(uint32_t ks = 0; ks < 2u; ++ks)
+#pragma unroll
+                    for(uint32_t w = 0; w < 4u; ++w)
+                    {
+                        const uint32_t c0 = ks * 16u + kGroup * 8u + 2u * w;
+                        keep[ks][w]       = (c0 < m ? 0x0000FFFFu : 0u) | (c0 + 1u < m ? 0xFFFF0000u : 0u);
+                    }
+                // the wait also makes the registers written by the inline assembly valid for what follows
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
                 for(uint32_t nb = 0; nb < NBlocks; ++nb)
                 {
                     fill_fragment(acc[nb], 0.0f);
 #pragma unroll
                     for(uint32_t ks = 0; ks < 2u; ++ks)
-                        mma_sync(acc[nb], fg[ks], ff[nb][ks], acc[nb]);
+                    {
+                        FragF f;
+#pragma unroll
+                        for(uint32_t w = 0; w < 4u; ++w)
+                        {
+                            // (the "+v" ties each operand word to a point behind the wait)
+                            asm volatile("" : "+v"(ff[nb][ks][w]));
+                            reinterpret_cast<uint32_t*>(f.x)[w] = ff[nb][ks][w] & keep[ks][w];
+                        }
+                        mma_sync(acc[nb], fg[ks], f, acc[nb]);
+                    }
                 }
             }
             __syncthreads(); // every wave is done reading features (its own and its neighbour's rows)
 
             if(wave < nHere)
             {
-                // this sample's feature rows become the staging buffer of its gradient (m x K, row-major)
-                float16_t* stage = reinterpret_cast<float16_t*>(ldsF) + wave * m * K;
+                // this sample's feature rows become the staging buffer of its gradient (m x K)
 #pragma unroll
                 for(uint32_t nb = 0; nb < NBlocks; ++nb)
 #pragma unroll
@@ -293,27 +375,30 @@ namespace rocwmma_amd
                         const uint32_t c  = nb * 32u + AccMap::colOf(e0, lane);
                         if(r < m)
                         {
-                            float16_t* p = stage + r * K + c;
+                            float16_t h[4];
 #pragma unroll
                             for(uint32_t j = 0; j < 4u; ++j)
-                                p[j] = static_cast<float16_t>(acc[nb].x[e0 + j]);
+                                h[j] = static_cast<float16_t>(acc[nb].x[e0 + j]);
+                            typedef uint32_t u32x2_t __attribute__((ext_vector_type(2), may_alias));
+                            *reinterpret_cast<u32x2_t*>(ldsF + Stage::unitOffset(wave * m + r, c / 4u)) = *reinterpret_cast<u32x2_t*>(h);
                         }
                     }
             }
             __syncthreads();
 
-            // coalesced write-out: gradients of all samples are one contiguous block
-            copyOut(grad + static_cast<size_t>(sample0) * m * K, reinterpret_cast<const float16_t*>(ldsF), nHere * m * K);
-            for(uint32_t i = threadIdx.x; i < nHere * (K / 8u); i += blockDim.x)
+            // coalesced write-out: gradients of all samples are one contiguous block of 16-byte pieces
             {
-                const uint32_t   s   = i / (K / 8u);
-                const uint32_t   c8  = i % (K / 8u);
-                const float16_t* src = ldsUp + s * width + c8 * 8u; // only 2-byte aligned in general
-                float16_t        tmp[8];
-#pragma unroll
-                for(uint32_t j = 0; j < 8u; ++j)
-                    tmp[j] = src[j];
-                reinterpret_cast<u32x4_t*>(mlpGrad + static_cast<size_t>(sample0 + s) * K)[c8] = *reinterpret_cast<u32x4_t*>(tmp);
+                constexpr uint32_t chunksPerRow = K / 8u;
+                u32x4_t*           dst          = reinterpret_cast<u32x4_t*>(grad + static_cast<size_t>(sample0) * m * K);
+                for(uint32_t q = threadIdx.x; q < nHere * m * chunksPerRow; q += blockDim.x)
+                {
+                    const uint32_t R = q / chunksPerRow, ch = q % chunksPerRow;
+                    const uint32_t s = R & Stage::mask;
+                    u32x4_t        v = *reinterpret_cast<const u32x4_t*>(ldsF + R * Stage::rowBytes + ((ch ^ (s >> 1)) << 4));
+                    if(s & 1u)
+                        v = u32x4_t{v[2], v[3], v[0], v[1]};
+                    dst[q] = v;
+                }
             }
         }
 
@@ -338,7 +423,9 @@ namespace rocwmma_amd
         int launchFwdS(const void* input, void* output, uint32_t m, uint32_t batch, hipStream_t stream)
         {
             const uint32_t width  = K + (m * (m - 1u)) / 2u;
-            const uint32_t lds    = tileBytesFor<K, Samples>(m) + ((Samples * width * 2u + 15u) & ~15u);
+            // (+ 32: the output staging starts at the output block's global address modulo 16, and a spare
+            // half per wave follows the block)
+            const uint32_t lds    = tileBytesFor<K, Samples>(m) + ((Samples * width * 2u + 15u) & ~15u) + 32u;
             const uint32_t grid   = (batch + Samples - 1u) / Samples;
             auto           kernel = dlrmFwdKernel<K, Samples>;
             if(int rc = optInLds(kernel, lds))
@@ -353,7 +440,8 @@ namespace rocwmma_amd
                        hipStream_t stream)
         {
             const uint32_t width  = K + (m * (m - 1u)) / 2u;
-            const uint32_t lds    = tileBytesFor<K, Samples>(m) + ((Samples * width * 2u + 15u) & ~15u);
+            // (the upstream block arrives as whole 256-byte copies)
+            const uint32_t lds    = tileBytesFor<K, Samples>(m) + ((Samples * width * 2u + 255u) & ~255u);
             const uint32_t grid   = (batch + Samples - 1u) / Samples;
             auto           kernel = dlrmBwdKernel<K, Samples>;
             if(int rc = optInLds(kernel, lds))

@@ -104,3 +104,23 @@ def test_backward_is_linear_and_forward_is_symmetric_at_large_batch():
               np.array_equal(f2[:, k + 1], f1[:, k + 0]),   # new Z[2,0] = F1.F0 = old Z[1,0]
               np.array_equal(f2[:, k + 2], f1[:, k + 2])]   # Z[2,1] is symmetric under the swap
     assert checks == [True, True, True]
+
+
+@pytest.mark.parametrize("b", [4, 9])
+def test_backward_samples_are_independent_of_non_finite_neighbours(b):
+    """The backward kernel contracts over 32 feature rows of a sample's LDS tile; with m < 32 the rows
+    behind the m-th belong to the next sample.  G is zero there, but 0 * NaN is NaN: a NaN or Inf in
+    sample s + 1 must leave the gradient of sample s untouched, as in the reference's CPU loops,
+    which never read another sample (test/reference_impl.hpp:121-179)."""
+    m, k = 27, 128
+    width = k + m * (m - 1) // 2
+    inp = uniform_bits(71, orc.F16, b * m * k).reshape(b, m, k).copy()
+    up = uniform_bits(72, orc.F16, b * width)
+    clean, _ = gpu_bwd(inp, up, m, k, b)
+    poisoned = inp.copy()
+    poisoned[1::2, :, :] = 0x7E00  # every odd sample: all NaN
+    poisoned[1::2, 0, 1] = 0x7C00  # and an Inf
+    grad, _ = gpu_bwd(poisoned, up, m, k, b)
+    assert np.array_equal(grad[0::2], clean[0::2])
+    wgrad, _ = orc.dlrm_bwd(poisoned, up, m, k, b)
+    assert np.array_equal(np.isnan(orc.decode(orc.F16, grad.reshape(-1))), np.isnan(orc.decode(orc.F16, wgrad.reshape(-1))))
