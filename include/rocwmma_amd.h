@@ -21,6 +21,7 @@
 #ifndef ROCWMMA_AMD_H
 #define ROCWMMA_AMD_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -147,6 +148,51 @@ int rocwmma_amd_gemm_ex(int         algo,
                         float       alpha,
                         float       beta,
                         void*       stream);
+
+/*
+ * D = alpha * A * B + beta * C with the tile count balanced over the compute units ("stream-K").
+ *
+ * Same arguments and semantics as rocwmma_amd_gemm.  The plain kernel runs one 256 x 256 tile per
+ * workgroup, in rounds of one tile per compute unit, so a tile count that is not a multiple of the
+ * unit count leaves units idle in the last round (m = 4096, n = 14336: 896 tiles = 3.5 rounds on
+ * 256 units; 3072^3: 144 tiles).  Here one persistent workgroup per unit takes whole tiles plus an
+ * equal share of the K range of the remaining ones; tiles shared by several workgroups are summed
+ * through `workspace`, in a fixed order (results are reproducible; I32 results are exact, F32 results
+ * differ from rocwmma_amd_gemm's only in how partial sums are rounded).
+ * The reference has no counterpart: its GEMM hosts launch plain 2-D grids
+ * (samples/perf_hgemm.cpp:810-812).
+ *
+ * Types: F16 / BF16 inputs with F32 C/D in every layout pair; I8 -> I32 and E4M3 / E5M2 -> F32 with
+ * row-major A and col-major B.  m and n multiples of 256, k a multiple of 128 bytes' worth of
+ * elements; other shapes return ROCWMMA_AMD_UNSUPPORTED_SHAPE (use rocwmma_amd_gemm).
+ * workspace: device memory, 256-byte aligned, at least rocwmma_amd_gemm_streamk_workspace_size()
+ * bytes (64 MiB + 1.25 KiB on a 256-unit device); contents need not be initialised and are not
+ * preserved.  Two calls that use the same workspace must not overlap in time.
+ * The call enqueues two kernels on `stream` (a small one that clears the flags, then the GEMM).
+ */
+size_t rocwmma_amd_gemm_streamk_workspace_size(void);
+
+int rocwmma_amd_gemm_streamk(int         dtype_in,
+                             int         dtype_out,
+                             int         layout_a,
+                             int         layout_b,
+                             int         layout_c,
+                             uint32_t    m,
+                             uint32_t    n,
+                             uint32_t    k,
+                             const void* a,
+                             uint32_t    lda,
+                             const void* b,
+                             uint32_t    ldb,
+                             const void* c,
+                             uint32_t    ldc,
+                             void*       d,
+                             uint32_t    ldd,
+                             float       alpha,
+                             float       beta,
+                             void*       workspace,
+                             size_t      workspace_bytes,
+                             void*       stream);
 
 /*
  * Skinny GEMV / GEMM:  Y = alpha * A * X + beta * Y,  in place on Y.

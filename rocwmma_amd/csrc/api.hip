@@ -5,6 +5,7 @@
 #include <atomic>
 #include <cmath>
 #include <cstring>
+#include <utility>
 
 namespace rocwmma_amd
 {
@@ -88,6 +89,21 @@ namespace rocwmma_amd
         int flip(int layout)
         {
             return layout == ROCWMMA_AMD_ROW_MAJOR ? ROCWMMA_AMD_COL_MAJOR : ROCWMMA_AMD_ROW_MAJOR;
+        }
+
+        // The blocked kernels write row-major C/D; a column-major result is the row-major result of
+        // the transposed problem D^T = B^T * A^T.
+        void transposeForColMajorC(GemmArgs& g, int& layoutA, int& layoutB)
+        {
+            if(g.layoutC != ROCWMMA_AMD_COL_MAJOR)
+                return;
+            std::swap(g.m, g.n);
+            std::swap(g.a, g.b);
+            std::swap(g.lda, g.ldb);
+            const int la = flip(layoutB), lb = flip(layoutA);
+            layoutA      = la;
+            layoutB      = lb;
+            g.layoutC    = ROCWMMA_AMD_ROW_MAJOR;
         }
     } // namespace
 } // namespace rocwmma_amd
@@ -184,22 +200,9 @@ int rocwmma_amd_gemm_ex(int         algo,
     }
     if(algo != ROCWMMA_AMD_GEMM_WAVE_TILE)
     {
-        // The blocked kernel writes row-major C/D; a column-major result is the row-major
-        // result of the transposed problem D^T = B^T * A^T.
         GemmArgs blocked = args;
         int      la = layout_a, lb = layout_b;
-        if(layout_c == ROCWMMA_AMD_COL_MAJOR)
-        {
-            blocked.m       = n;
-            blocked.n       = m;
-            blocked.a       = b;
-            blocked.b       = a;
-            blocked.lda     = ldb;
-            blocked.ldb     = lda;
-            la              = flip(layout_b);
-            lb              = flip(layout_a);
-            blocked.layoutC = ROCWMMA_AMD_ROW_MAJOR;
-        }
+        transposeForColMajorC(blocked, la, lb);
         rc = launchGemmBlocked(dtype_in, dtype_out, la, lb, blocked, asStream(stream), algo == ROCWMMA_AMD_GEMM_BLOCKED_256);
         if(rc == ROCWMMA_AMD_OK || algo == ROCWMMA_AMD_GEMM_BLOCKED || algo == ROCWMMA_AMD_GEMM_BLOCKED_256)
             return rc;
@@ -207,6 +210,46 @@ int rocwmma_amd_gemm_ex(int         algo,
             return rc;
     }
     return launchGemmWaveTile(dtype_in, dtype_out, layout_a, layout_b, args, asStream(stream));
+}
+
+size_t rocwmma_amd_gemm_streamk_workspace_size(void)
+{
+    return streamKWorkspaceBytes(computeUnits());
+}
+
+int rocwmma_amd_gemm_streamk(int         dtype_in,
+                             int         dtype_out,
+                             int         layout_a,
+                             int         layout_b,
+                             int         layout_c,
+                             uint32_t    m,
+                             uint32_t    n,
+                             uint32_t    k,
+                             const void* a,
+                             uint32_t    lda,
+                             const void* b,
+                             uint32_t    ldb,
+                             const void* c,
+                             uint32_t    ldc,
+                             void*       d,
+                             uint32_t    ldd,
+                             float       alpha,
+                             float       beta,
+                             void*       workspace,
+                             size_t      workspace_bytes,
+                             void*       stream)
+{
+    int rc = checkGemm(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, lda, b, ldb, c, ldc, d, ldd, alpha, beta);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(!workspace)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    GemmArgs args{m, n, k, a, b, c, d, lda, ldb, c ? ldc : ldd, ldd, alpha, beta, layout_c};
+    int      la = layout_a, lb = layout_b;
+    transposeForColMajorC(args, la, lb);
+    return launchGemmStreamK(dtype_in, dtype_out, la, lb, args, workspace, workspace_bytes, asStream(stream));
 }
 
 int rocwmma_amd_gemm(int         dtype_in,

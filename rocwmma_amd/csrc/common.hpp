@@ -3,6 +3,7 @@
 #define ROCWMMA_AMD_CSRC_COMMON_HPP
 
 #include <atomic>
+#include <cstddef>
 #include <cstdint>
 #include <hip/hip_runtime.h>
 
@@ -87,6 +88,12 @@ namespace rocwmma_amd
     int launchGemmBlocked(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream,
                           bool forceLargeTile = false);
     int launchGemmSkinny(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
+    // Stream-K: the 256 x 256 tiling with the tile count balanced over persistent workgroups.  The
+    // workspace holds one slot of raw accumulators per workgroup plus flags (streamKWorkspaceBytes).
+    constexpr uint32_t kStreamKSlotBytes = 256u * 256u * 4u;
+    size_t streamKWorkspaceBytes(uint32_t workgroups);
+    int    launchGemmStreamK(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, void* workspace,
+                             size_t workspaceBytes, hipStream_t stream);
 
 } // namespace rocwmma_amd
 

@@ -1,28 +1,6 @@
-// Blocked GEMM for gfx950: D = alpha * A * B + beta * C, C/D row-major.
-//
-// The workload of the reference's perf_hgemm sample (gemm_rocwmma_d,
-// samples/perf_hgemm.cpp:518-714: macro tile per workgroup, wave tile of MFMA blocks per wave,
-// two LDS buffers, next K slab prefetched while the current one is multiplied), re-tiled and
-// re-plumbed for CDNA4:
-//
-//   reference (gfx9 params)                      this kernel
-//   macro tile 128 x 128 x 16, 4 waves           256 x 256 x (64 bytes of K) x 4-stage LDS ring, 8 waves
-//                                                (two per SIMD: one keeps the matrix pipe fed
-//                                                while the other waits at a barrier)
-//   wave tile 2 x 2 blocks of 32x32x16 (2 MFMA)  2 x 4 blocks of 32x32, one wide-K MFMA per step
-//   global -> VGPR -> shuffle -> LDS             global -> LDS directly (global_load_lds_dwordx4)
-//   LDS -> VGPR -> shuffle (AOS<->SOA)           swizzled ds_read_b128, or ds_read_b64_tr_b16
-//                                                for operands whose K is not contiguous
-//   2 LDS buffers, wait + barrier per step       copies 3 stages ahead, one bare barrier per stage
-//   8 MFMA between barriers                      16 MFMA (128 passes) per wave between barriers
-//   C read / D written in fragment layout       C staged through LDS (full-row non-temporal
-//                                                copies), D written in fragment layout
-//   grid (m/128, n/128)                          1-D grid, tiles dealt to XCDs in L2-friendly patches
-//                                                (9 % faster than the plain order at 8192^3)
-//
-// Column-major C/D is handled by the caller as the transposed problem (D^T = B^T A^T).
-#include "common.hpp"
-#include <rocwmma/rocwmma_lds.hpp>
+// Blocked GEMM for gfx950, one macro tile per workgroup: kernel, tile ladder and dispatch.  The device
+// side (configuration, LDS pipeline, epilogue) is in gemm_blocked_core.hpp.
+#include "gemm_blocked_core.hpp"
 
 using namespace rocwmma;
 
@@ -30,712 +8,25 @@ namespace rocwmma_amd
 {
     namespace
     {
-        constexpr uint32_t kXcds = 8; // MI355X: 8 accelerator complex dies, one L2 each
-
-        template <typename InT_,
-                  typename OutT_,
-                  typename CompT_,
-                  bool     AKMajor_, // A row-major  (K contiguous)
-                  bool     BKMajor_, // B col-major  (K contiguous)
-                  uint32_t WavesM_,
-                  uint32_t WavesN_,
-                  uint32_t BlocksM_,
-                  uint32_t BlocksN_,
-                  uint32_t Stages_       = 4u, // LDS ring depth
-                  uint32_t WavesPerSimd_ = 1u, // waves per SIMD: sizes the register budget, and no more become resident
-                  uint32_t BlockEdge_    = 32u> // MFMA block edge: 32 (32x32xK) or 16 (16x16x2K)
-        struct BlockedConfig
-        {
-            using InT   = InT_;
-            using OutT  = OutT_;
-            using CompT = CompT_;
-
-            static constexpr bool     AKMajor = AKMajor_;
-            static constexpr bool     BKMajor = BKMajor_;
-            static constexpr uint32_t WavesM  = WavesM_;
-            static constexpr uint32_t WavesN  = WavesN_;
-            static constexpr uint32_t BlocksM = BlocksM_;
-            static constexpr uint32_t BlocksN = BlocksN_;
-            static constexpr uint32_t Waves   = WavesM * WavesN;
-            static constexpr uint32_t Threads = Waves * 64u;
-            static constexpr uint32_t Block   = BlockEdge_; // MFMA edge
-            static constexpr uint32_t WaveM   = BlocksM * Block;
-            static constexpr uint32_t WaveN   = BlocksN * Block;
-            static constexpr uint32_t MacroM  = WavesM * WaveM;
-            static constexpr uint32_t MacroN  = WavesN * WaveN;
-            // bytes of K per pipeline stage: 64 in the ring of four, 128 (whole lines of a K-contiguous
-            // operand) in the ring of two
-            static constexpr uint32_t StageKB = Stages_ == 2u ? 128u : 64u;
-            static constexpr uint32_t MacroK  = StageKB / sizeof(InT); // K elements per stage
-
-            // Fragments of one MFMA step.  BlockK = K of the widest single instruction.
-            static constexpr uint32_t KPack      = detail::maxKPack(detail::packClassOf<InT>());
-            static constexpr uint32_t BlockK     = KPack * (64u / Block); // 2 (32-wide) or 4 (16-wide) lane groups along K
-            static constexpr uint32_t KPackBytes = KPack * sizeof(InT);
-            static constexpr uint32_t KSteps     = MacroK / BlockK; // MFMA steps per stage (1 or 2)
-
-            using FragA   = fragment<matrix_a, Block, Block, BlockK, InT, row_major>;
-            using FragB   = fragment<matrix_b, Block, Block, BlockK, InT, col_major>;
-            using FragAcc = fragment<accumulator, Block, Block, BlockK, CompT>;
-            using FragC   = fragment<accumulator, Block, Block, BlockK, OutT, row_major>;
-
-            using TileA = std::conditional_t<AKMajor, lds::KMajorTile<MacroM, StageKB>, lds::DimMajorTile<MacroM, StageKB / 2u>>;
-            using TileB = std::conditional_t<BKMajor, lds::KMajorTile<MacroN, StageKB>, lds::DimMajorTile<MacroN, StageKB / 2u>>;
-
-            static constexpr uint32_t BytesA     = MacroM * StageKB;
-            static constexpr uint32_t BytesB     = MacroN * StageKB;
-            static constexpr uint32_t StageBytes = BytesA + BytesB;
-            static constexpr uint32_t Stages     = Stages_; // ring of K stages in LDS
-            static constexpr uint32_t WavesPerSimd = WavesPerSimd_;
-            static constexpr uint32_t LdsBytes   = Stages * StageBytes;
-            static constexpr uint32_t CopiesA    = BytesA / 1024u / Waves; // direct copies per wave per stage
-            static constexpr uint32_t CopiesB    = BytesB / 1024u / Waves;
-            static constexpr uint32_t Copies     = CopiesA + CopiesB;
-            // LDS read instructions per MFMA step: b128 reads per block (K-major) or two transposing b64 reads
-            static constexpr uint32_t ReadsA       = BlocksM * (AKMajor ? KPackBytes / 16u : 2u);
-            static constexpr uint32_t ReadsB       = BlocksN * (BKMajor ? KPackBytes / 16u : 2u);
-            static constexpr uint32_t ReadsPerStep = ReadsA + ReadsB;
-            static constexpr uint32_t MfmasPerStep = BlocksM * BlocksN;
-            // beta * C operand staged through LDS in the epilogue, in groups of Block rows by
-            // GroupBlocks blocks (256- or 512-byte rows), two group buffers per wave
-            static constexpr uint32_t GroupBlocks
-                = (WaveN == 128u && 2u * Block * 128u * sizeof(OutT) * Waves <= LdsBytes) ? 128u / Block : 64u / Block;
-            static constexpr bool StagedC = sizeof(OutT) == 4u && WaveN % 64u == 0u
-                                            && BlocksM * (BlocksN / GroupBlocks) >= 2u
-                                            && 2u * Block * GroupBlocks * Block * sizeof(OutT) * Waves <= LdsBytes;
-
-            static_assert(Block == 32u || Block == 16u, "MFMA blocks are 32 or 16 wide");
-            static_assert(Block == 32u || KPackBytes == 16u, "16-wide blocks: 16 bytes of K per lane (16-bit types, int8)");
-            static_assert(AKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
-            static_assert(BKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
-            static_assert(TileA::bytes == BytesA && TileB::bytes == BytesB, "stage geometry mismatch");
-            static_assert(BytesA % (1024u * Waves) == 0u && BytesB % (1024u * Waves) == 0u,
-                          "a stage must split into whole-wave copies evenly");
-            static_assert((Stages - 1u) * Copies < 64u, "too many copies in flight for vmcnt");
-            static_assert(Stages != 2u || KSteps == 2u, "the ring of two runs two MFMA steps per stage");
-            static_assert(LdsBytes <= Constants::AMDGCN_LDS_MAX_SIZE_BYTES, "macro tile does not fit the LDS");
-            // the dim-major tile's swizzle looks at K row bits 0..3: a wave's copies must all start
-            // on the same K row modulo 16
-            static_assert((AKMajor || (Waves * TileA::rowsPerCopy) % 16u == 0u)
-                              && (BKMajor || (Waves * TileB::rowsPerCopy) % 16u == 0u),
-                          "wave pool too small for the dim-major tile");
-            // the K-major tile's swizzle looks at row bits 0..3 likewise
-            static_assert((!AKMajor || (Waves * TileA::rowsPerCopy) % 16u == 0u)
-                              && (!BKMajor || (Waves * TileB::rowsPerCopy) % 16u == 0u),
-                          "wave pool too small for the K-major tile");
-        };
-
-        // Deals the 1-D grid to tiles so that the workgroups resident on one XCD (ids congruent
-        // mod 8 land on the same XCD) form a compact patch of the tile grid and share A / B
-        // panels through that XCD's L2.
-        ROCWMMA_DEVICE inline void tileOfWorkgroup(uint32_t wg, uint32_t tilesM, uint32_t tilesN, uint32_t& tm, uint32_t& tn)
-        {
-            const uint32_t total = tilesM * tilesN;
-            uint32_t       id    = wg;
-            if(total % kXcds == 0u)
-                id = (wg % kXcds) * (total / kXcds) + wg / kXcds;
-            // panels of 4 tile rows, walked column by column: the 32 workgroups an XCD runs at a
-            // time cover 4 x 8 tiles (measured: 1 % faster than 8 x 4, 5 % faster than 16 x 2)
-            constexpr uint32_t panel    = 4u;
-            const uint32_t     perPanel = panel * tilesN;
-            const uint32_t     panelIdx = id / perPanel;
-            const uint32_t     firstRow = panelIdx * panel;
-            const uint32_t     rowsHere = (tilesM - firstRow) < panel ? (tilesM - firstRow) : panel;
-            const uint32_t     inPanel  = id - panelIdx * perPanel;
-            tm                          = firstRow + inPanel % rowsHere;
-            tn                          = inPanel / rowsHere;
-        }
-
-        // Scheduling hint: within the current scheduling region, issue `Mfmas` matrix instructions
-        // with `Reads` LDS reads and `Copies` global -> LDS copies spread evenly between them.
-        template <uint32_t Mfmas, uint32_t Reads, uint32_t Copies>
-        ROCWMMA_DEVICE ROCWMMA_INLINE void scheduleInterleaved()
-        {
-            constexpr uint32_t Div = Mfmas > 0u ? Mfmas : 1u; // (an empty group: the loop does not run)
-#pragma unroll
-            for(uint32_t j = 0; j < Mfmas; ++j)
-            {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
-                const uint32_t r = ((j + 1u) * Reads) / Div - (j * Reads) / Div;
-                const uint32_t c = ((j + 1u) * Copies) / Div - (j * Copies) / Div;
-                if(r == 1u)
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
-                else if(r == 2u)
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                else if(r > 2u)
-                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-                if(c == 1u)
-                    __builtin_amdgcn_sched_group_barrier(0x010, 1, 0); // VMEM
-                else if(c >= 2u)
-                    __builtin_amdgcn_sched_group_barrier(0x010, 2, 0);
-            }
-        }
-
-        // Main loop schedule (per wave; S = 4 LDS stages of 64 bytes of K, F0/F1 = fragment
-        // register sets of the first / last MFMA step of a stage):
-        //
-        //   prologue : copies for stages 0..2 in flight; wait for stage 0; barrier; read F0(0)
-        //   iteration i:
-        //       issue copies of stage i+3 (into the ring slot everybody finished reading at
-        //         the barrier of iteration i-1)
-        //       [two-step stages] read F1(i) while the MFMAs of F0(i) run
-        //       wait: stage i+1 landed (copies of stages i+2, i+3 may stay in flight) and own
-        //         LDS reads returned;  barrier
-        //       read F0(i+1) while the MFMAs of the last step of stage i run
-        //
-        // So every LDS read has a full MFMA step (16 instructions, 512 cycles) to return, every
-        // global -> LDS copy has almost three iterations, and the barrier is the only
-        // synchronisation per stage.
         template <typename Cfg>
         __global__ void __launch_bounds__(Cfg::Threads) __attribute__((amdgpu_waves_per_eu(Cfg::WavesPerSimd, Cfg::WavesPerSimd)))
         gemmBlockedKernel(uint32_t                   m,
-                                                                           uint32_t                   n,
-                                                                           uint32_t                   k,
-                                                                           typename Cfg::InT const*   a,
-                                                                           typename Cfg::InT const*   b,
-                                                                           typename Cfg::OutT const*  c,
-                                                                           typename Cfg::OutT*        d,
-                                                                           uint32_t                   lda,
-                                                                           uint32_t                   ldb,
-                                                                           uint32_t                   ldc,
-                                                                           uint32_t                   ldd,
-                                                                           typename Cfg::CompT        alpha,
-                                                                           typename Cfg::CompT        beta)
+                          uint32_t                   n,
+                          uint32_t                   k,
+                          typename Cfg::InT const*   a,
+                          typename Cfg::InT const*   b,
+                          typename Cfg::OutT const*  c,
+                          typename Cfg::OutT*        d,
+                          uint32_t                   lda,
+                          uint32_t                   ldb,
+                          uint32_t                   ldc,
+                          uint32_t                   ldd,
+                          typename Cfg::CompT        alpha,
+                          typename Cfg::CompT        beta)
         {
-            using InT   = typename Cfg::InT;
-            using OutT  = typename Cfg::OutT;
-            using CompT = typename Cfg::CompT;
-            using TileA = typename Cfg::TileA;
-            using TileB = typename Cfg::TileB;
-
-            extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
-
-            const uint32_t lane  = threadIdx.x & 63u;
-            const uint32_t wave  = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave uniform
-            const uint32_t waveM = wave / Cfg::WavesN;
-            const uint32_t waveN = wave % Cfg::WavesN;
-
             uint32_t tm, tn;
             tileOfWorkgroup(blockIdx.x, m / Cfg::MacroM, n / Cfg::MacroN, tm, tn);
-            const uint32_t row0 = tm * Cfg::MacroM;
-            const uint32_t col0 = tn * Cfg::MacroN;
-
-            // Global sources: uniform tile pointer + uniform per-copy offset + per-lane offset
-            const uint32_t ldaB = lda * sizeof(InT);
-            const uint32_t ldbB = ldb * sizeof(InT);
-            const char*    aSrc = reinterpret_cast<const char*>(a)
-                               + static_cast<size_t>(row0) * (Cfg::AKMajor ? ldaB : static_cast<uint32_t>(sizeof(InT)));
-            const char* bSrc = reinterpret_cast<const char*>(b)
-                               + static_cast<size_t>(col0) * (Cfg::BKMajor ? ldbB : static_cast<uint32_t>(sizeof(InT)));
-            const size_t   aStep    = TileA::stageStep(ldaB);
-            const size_t   bStep    = TileB::stageStep(ldbB);
-            const uint32_t aLaneOff = TileA::laneSourceOffset(lane, wave, ldaB);
-            const uint32_t bLaneOff = TileB::laneSourceOffset(lane, wave, ldbB);
-
-            // A stage is copied in two halves (the A operand, then the B operand) so that each
-            // MFMA phase of an iteration carries half of the copy instructions.
-            // advance == false leaves the source on the stage just copied (used to re-copy the last
-            // stage instead of running past the end of the operand)
-            auto issueA = [&](uint32_t slot, bool advance = true) {
-                char*                 ldsA = ldsRaw + slot * Cfg::StageBytes;
-                const lds::BufferRsrc src  = lds::makeSource(aSrc);
-#pragma unroll
-                for(uint32_t i = 0; i < Cfg::CopiesA; ++i)
-                {
-                    const uint32_t copy = i * Cfg::Waves + wave;
-                    lds::asyncCopy16(ldsA + copy * 1024u, src, aLaneOff, TileA::copySourceOffset(copy, ldaB));
-                }
-                aSrc += advance ? aStep : size_t{0};
-            };
-            auto issueB = [&](uint32_t slot, bool advance = true) {
-                char*                 ldsB = ldsRaw + slot * Cfg::StageBytes + Cfg::BytesA;
-                const lds::BufferRsrc src  = lds::makeSource(bSrc);
-#pragma unroll
-                for(uint32_t i = 0; i < Cfg::CopiesB; ++i)
-                {
-                    const uint32_t copy = i * Cfg::Waves + wave;
-                    lds::asyncCopy16(ldsB + copy * 1024u, src, bLaneOff, TileB::copySourceOffset(copy, ldbB));
-                }
-                bSrc += advance ? bStep : size_t{0};
-            };
-            auto issueStage = [&](uint32_t slot, bool advance = true) {
-                issueA(slot, advance);
-                issueB(slot, advance);
-            };
-
-            struct Frags
-            {
-                typename Cfg::FragA a[Cfg::BlocksM];
-                typename Cfg::FragB b[Cfg::BlocksN];
-            };
-
-            auto readFrags = [&](Frags& f, uint32_t slot, uint32_t ks) {
-                const char* ldsA = ldsRaw + slot * Cfg::StageBytes;
-                const char* ldsB = ldsA + Cfg::BytesA;
-#pragma unroll
-                for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
-                {
-                    if constexpr(Cfg::Block == 32u)
-                        TileA::template readBlock32<Cfg::KPackBytes>(f.a[i].x, ldsA, waveM * Cfg::WaveM + i * Cfg::Block, ks, lane);
-                    else
-                        TileA::template readBlock16<Cfg::KPackBytes>(f.a[i].x, ldsA, waveM * Cfg::WaveM + i * Cfg::Block, ks, lane);
-                }
-#pragma unroll
-                for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
-                {
-                    if constexpr(Cfg::Block == 32u)
-                        TileB::template readBlock32<Cfg::KPackBytes>(f.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, ks, lane);
-                    else
-                        TileB::template readBlock16<Cfg::KPackBytes>(f.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, ks, lane);
-                }
-            };
-
-            typename Cfg::FragAcc acc[Cfg::BlocksM][Cfg::BlocksN];
-#pragma unroll
-            for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
-#pragma unroll
-                for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
-                    fill_fragment(acc[i][j], static_cast<CompT>(0));
-
-            auto multiply = [&](Frags const& f) {
-#pragma unroll
-                for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
-#pragma unroll
-                    for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
-                        mma_sync(acc[i][j], f.a[i], f.b[j], acc[i][j]);
-            };
-
-            constexpr uint32_t S      = Cfg::Stages;
-            const uint32_t     stages = k / Cfg::MacroK; // >= S - 1 (checked by the host)
-
-            if constexpr(S == 2u)
-            {
-                // Ring of two stages of 128 bytes of K (two MFMA steps each).  A phase multiplies one
-                // step while it reads the fragments of the next; the barrier in the middle of an
-                // iteration is where stage i has been read completely and stage i+1 has landed, so
-                // the copies of stage i+2 go out right behind it, into stage i's slot, and have the
-                // two phases up to the next barrier to land.  Past the end of K the loop copies the
-                // last stage again and reads fragments nobody multiplies, so its body is uniform.
-                issueStage(0u, 1u < stages);
-                issueStage(1u, 2u < stages);
-                lds::waitCopiesAndReads<Cfg::Copies>(); // stage 0 has landed
-                lds::barrier();
-                Frags f0, f1;
-                readFrags(f0, 0u, 0u);
-                for(uint32_t i = 0; i < stages; ++i)
-                {
-                    if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
-                    {
-                        lds::waitReads(); // transposing reads of the previous phase
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    readFrags(f1, i % 2u, 1u);
-                    multiply(f0);
-                    scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
-                    __builtin_amdgcn_sched_barrier(0);
-                    lds::waitCopiesAndReads<0u>(); // stage i+1 has landed, stage i is in registers
-                    lds::barrier();
-                    __builtin_amdgcn_sched_barrier(0);
-                    issueStage(i % 2u, i + 3u < stages);
-                    readFrags(f0, (i + 1u) % 2u, 0u);
-                    multiply(f1);
-                    scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
-                    scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::Copies>();
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
-                lds::barrier();
-            }
-            else if constexpr(Cfg::KSteps == 2u)
-            {
-                // Prologue
-#pragma unroll
-                for(uint32_t s = 0; s < S - 1u; ++s)
-                    issueStage(s);
-                lds::waitCopiesAndReads<(S - 2u) * Cfg::Copies>();
-                lds::barrier();
-                Frags f0, f1;
-                readFrags(f0, 0u, 0u);
-
-                // Steady state: a new stage is issued every iteration
-                uint32_t i = 0;
-                for(; i + (S - 1u) < stages; ++i)
-                {
-                    if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
-                    {
-                        lds::waitReads(); // fragments read during the previous phase
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    issueA((i + S - 1u) % S);
-                    readFrags(f1, i % S, 1u);
-                    multiply(f0);
-                    // LDS reads ride on the first half of the MFMAs (so they are back at the
-                    // barrier), the copies on the second half, two MFMAs per copy
-                    scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
-                    scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::CopiesA>();
-                    __builtin_amdgcn_sched_barrier(0); // nothing moves across the synchronisation point
-                    // stage i+1 has landed once only stage i+2 and the A half of stage i+3 are in flight
-                    lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies + Cfg::CopiesA>();
-                    lds::barrier();
-                    __builtin_amdgcn_sched_barrier(0);
-                    issueB((i + S - 1u) % S);
-                    readFrags(f0, (i + 1u) % S, 0u);
-                    multiply(f1);
-                    scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
-                    scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::CopiesB>();
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                // Drain: nothing left to issue; the remaining stages are already in flight
-                for(; i < stages; ++i)
-                {
-                    const bool more = i + 1u < stages;
-                    if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
-                    {
-                        lds::waitReads();
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    readFrags(f1, i % S, 1u);
-                    multiply(f0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    lds::waitCopiesAndReads<0u>();
-                    lds::barrier();
-                    __builtin_amdgcn_sched_barrier(0);
-                    if(more)
-                        readFrags(f0, (i + 1u) % S, 0u);
-                    multiply(f1);
-                }
-            }
-            else
-            {
-                // One MFMA step per stage (wide fp8): a phase multiplies stage s (fragments read
-                // during the previous phase) while it reads the fragments of stage s+1 and issues
-                // the copies of stage s+3; the wait + barrier closing the phase makes stage s+2
-                // visible.  Two phases per loop trip so the fragment sets swap without copies.
-                // Every phase issues a stage, so the loop body and its wait counts are uniform:
-                // past the end of K the last stage is copied again into a ring slot nobody reads.
-                static_assert(Cfg::KSteps == 1u, "one MFMA step per stage");
-                Frags f0, f1;
-                // Transposing LDS reads are inline assembly, which the scheduling hints cannot
-                // place: with a dim-major B (two such reads for each of its 8 blocks) the phase is laid
-                // out by hand, one column of blocks at a time (the reads of that column of the next
-                // stage, then its MFMAs): 5 % faster than leaving the reads in front of the MFMAs.  With
-                // only A dim-major (4 blocks) the compiler's placement is 1 % better and is kept.
-                auto phaseByColumns = [&](Frags const& cur, Frags& nxt, uint32_t slot) {
-                    const char* ldsA = ldsRaw + slot * Cfg::StageBytes;
-                    const char* ldsB = ldsA + Cfg::BytesA;
-                    static_assert(Cfg::Block == 16u || Cfg::KSteps != 1u || Cfg::BKMajor,
-                                  "one-step stages with a dim-major B use 16-wide blocks");
-                    if constexpr(Cfg::Block == 16u)
-                    {
-                        static_assert(Cfg::BlocksM <= Cfg::BlocksN, "the A blocks are read along with the first B columns");
-#pragma unroll
-                        for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
-                        {
-                            TileB::template readBlock16<Cfg::KPackBytes>(nxt.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, 0u, lane);
-                            if(j < Cfg::BlocksM)
-                                TileA::template readBlock16<Cfg::KPackBytes>(nxt.a[j].x, ldsA, waveM * Cfg::WaveM + j * Cfg::Block, 0u, lane);
-#pragma unroll
-                            for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
-                                mma_sync(acc[i][j], cur.a[i], cur.b[j], acc[i][j]);
-                            __builtin_amdgcn_sched_barrier(0);
-                        }
-                    }
-                };
-#define ROCWMMA_AMD_PHASE(STAGE, CUR, NXT, READ)                                                         \
-    do                                                                                                  \
-    {                                                                                                   \
-        issueStage(((STAGE) + S - 1u) % S, (STAGE) + S < stages);                                       \
-        if constexpr(Cfg::BKMajor)                                                                      \
-        {                                                                                               \
-            if(READ)                                                                                    \
-                readFrags(NXT, ((STAGE) + 1u) % S, 0u);                                                 \
-            multiply(CUR);                                                                              \
-            scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();                       \
-            scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::Copies>();         \
-        }                                                                                               \
-        else                                                                                            \
-            phaseByColumns(CUR, NXT, ((STAGE) + 1u) % S);                                               \
-        __builtin_amdgcn_sched_barrier(0);                                                              \
-        lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies>();                                              \
-        lds::barrier();                                                                                 \
-        __builtin_amdgcn_sched_barrier(0);                                                              \
-    } while(0)
-
-#pragma unroll
-                for(uint32_t s = 0; s < S - 1u; ++s)
-                    issueStage(s, s + 1u < stages);
-                lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies>(); // stages 0 and 1 have landed
-                lds::barrier();
-                readFrags(f0, 0u, 0u);
-                if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
-                {
-                    lds::waitReads(); // the transposing reads are outside the compiler's tracking
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                uint32_t s = 0;
-                for(; s + 1u < stages; s += 2u)
-                {
-                    ROCWMMA_AMD_PHASE(s, f0, f1, true);
-                    // (past the last stage this reads a ring slot whose content nobody multiplies:
-                    // an unconditional phase body keeps the instruction interleave intact)
-                    ROCWMMA_AMD_PHASE(s + 1u, f1, f0, true);
-                }
-                if(s < stages)
-                    multiply(f0);
-                lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
-                lds::barrier();
-#undef ROCWMMA_AMD_PHASE
-            }
-
-            // Epilogue: D = alpha * acc + beta * C, one row of blocks (BlocksN blocks) at a time,
-            // 16-byte accesses per lane.  Every block of a group has registers of its own, so
-            // the stores of a group issue back to back (a store whose data registers are about
-            // to be overwritten holds up the instruction stream until it has read them), and
-            // the C blocks of the next two groups are in flight while a group is finished.
-            const uint32_t wRow        = row0 + waveM * Cfg::WaveM;
-            const uint32_t wCol        = col0 + waveN * Cfg::WaveN;
-            // Plain stores: the 32-byte pieces a store instruction writes per row are merged into
-            // full lines in the L2.  Non-temporal stores bypass that merge and were 3-5x slower
-            // (4096 x 14336 x 256 int8: 157-277 us against 58 us).
-            // (accumulator layout: lane l owns runs of 4 consecutive columns of row l % Block;
-            // 32-wide blocks: 4 runs at columns 8 r + 4 (l / 32); 16-wide blocks: 1 run at 4 (l / 16))
-            constexpr uint32_t Runs     = Cfg::Block == 32u ? 4u : 1u; // runs per block per lane
-            const uint32_t     accRow   = lane & (Cfg::Block - 1u);
-            const uint32_t     accGroup = lane / Cfg::Block; // 0..1 or 0..3
-            auto storeBlock = [&](OutT* dst, auto const& f, uint32_t ld) {
-                typedef uint32_t Words __attribute__((ext_vector_type(sizeof(OutT))));
-#pragma unroll
-                for(uint32_t r = 0; r < Runs; ++r)
-                {
-                    Words v;
-                    __builtin_memcpy(&v, f.x + 4u * r, sizeof(v));
-                    *reinterpret_cast<Words*>(dst + static_cast<size_t>(accRow) * ld + 8u * r + 4u * accGroup) = v;
-                }
-            };
-            // 16-bit outputs with 16-wide blocks: a lane's run is only 8 bytes, a store instruction would
-            // write 32-byte pieces.  Two neighbouring blocks are handled together: v_permlane16_swap
-            // exchanges the second block's run of a lane in an even 16-lane row with the first block's
-            // run of its partner in the next row, after which every lane owns 8 consecutive columns
-            // (even rows: of the first block, odd rows: of the second) and moves 16 bytes; an
-            // instruction then covers 64 contiguous bytes per matrix row.  The exchange is its own
-            // inverse, so C is read the same way.
-            constexpr bool PairIO = Cfg::Block == 16u && sizeof(OutT) == 2u && Cfg::BlocksN % 2u == 0u;
-            const uint32_t pairCol = (accGroup & 1u) * 16u + 4u * (accGroup & 2u);
-            auto           swapPair = [](auto& fx, auto& fy) {
-                uint32_t x[2], y[2];
-                __builtin_memcpy(x, fx.x, 8);
-                __builtin_memcpy(y, fy.x, 8);
-#pragma unroll
-                for(uint32_t w = 0; w < 2u; ++w)
-                {
-                    auto r = __builtin_amdgcn_permlane16_swap(x[w], y[w], false, false);
-                    x[w]   = r[0];
-                    y[w]   = r[1];
-                }
-                __builtin_memcpy(fx.x, x, 8);
-                __builtin_memcpy(fy.x, y, 8);
-            };
-            auto storePair = [&](OutT* dst, auto& fx, auto& fy, uint32_t ld) {
-                swapPair(fx, fy);
-                typedef uint32_t Words __attribute__((ext_vector_type(4)));
-                Words            v;
-                __builtin_memcpy(&v, fx.x, 8);
-                __builtin_memcpy(reinterpret_cast<char*>(&v) + 8, fy.x, 8);
-                *reinterpret_cast<Words*>(dst + static_cast<size_t>(accRow) * ld + pairCol) = v;
-            };
-            auto loadPair = [&](auto& fx, auto& fy, const OutT* src, uint32_t ld) {
-                typedef uint32_t Words __attribute__((ext_vector_type(4)));
-                const Words      v = *reinterpret_cast<const Words*>(src + static_cast<size_t>(accRow) * ld + pairCol);
-                __builtin_memcpy(fx.x, &v, 8);
-                __builtin_memcpy(fy.x, reinterpret_cast<const char*>(&v) + 8, 8);
-                swapPair(fx, fy);
-            };
-            auto           blockOffset = [&](uint32_t bi, uint32_t bj, uint32_t ld) {
-                return static_cast<size_t>(wRow + bi * Cfg::Block) * ld + wCol + bj * Cfg::Block;
-            };
-            if(beta != static_cast<CompT>(0))
-            {
-                if constexpr(Cfg::StagedC)
-                {
-                    // C reaches the accumulator layout through LDS: whole-wave direct copies
-                    // fetch full rows of a 32-row group of GroupBlocks blocks (read in the
-                    // accumulator layout straight from global memory, an instruction would touch
-                    // 32 rows for 32 bytes each, at half the rate).  Row r is stored with its
-                    // 16-byte chunks XOR-swizzled by r % 16 so that the 16 rows a quarter-wave
-                    // reads at one chunk position fall into distinct bank groups.  The main-loop
-                    // ring is free by now and every wave owns two group buffers in it.
-                    constexpr uint32_t GB          = Cfg::GroupBlocks;
-                    constexpr uint32_t RowBytes    = GB * Cfg::Block * sizeof(OutT); // 256 or 512
-                    constexpr uint32_t GroupBytes  = Cfg::Block * RowBytes;
-                    constexpr uint32_t RowChunks   = RowBytes / 16u;
-                    constexpr uint32_t RowsPerCopy = 1024u / RowBytes;
-                    constexpr uint32_t CopiesC     = GroupBytes / 1024u;
-                    constexpr uint32_t StoresD     = GB * Runs; // 16-byte stores per group
-                    constexpr uint32_t GroupsPerRow = Cfg::BlocksN / GB;
-                    constexpr uint32_t NG          = Cfg::BlocksM * GroupsPerRow;
-                    static_assert((RowBytes == 256u || RowBytes == 512u) && 2u * GroupBytes * Cfg::Waves <= Cfg::LdsBytes
-                                      && NG >= 2u,
-                                  "C staging geometry");
-                    char*          myLds  = ldsRaw + wave * (2u * GroupBytes);
-                    const char*    cWave  = reinterpret_cast<const char*>(c + static_cast<size_t>(wRow) * ldc + wCol);
-                    const size_t   ldcB   = static_cast<size_t>(ldc) * sizeof(OutT);
-                    const uint32_t cpRow  = lane / RowChunks; // row inside a copy
-                    const uint32_t chunk  = lane % RowChunks; // chunk position inside the LDS row
-                    auto           copyGroup = [&](uint32_t gi) {
-                        const uint32_t bi = gi / GroupsPerRow, bj0 = (gi % GroupsPerRow) * GB;
-#pragma unroll
-                        for(uint32_t i = 0; i < CopiesC; ++i)
-                        {
-                            const uint32_t r = RowsPerCopy * i + cpRow;
-                            lds::asyncCopy16Streaming(myLds + (gi % 2u) * GroupBytes + i * 1024u,
-                                                      cWave + (bi * Cfg::Block + r) * ldcB + bj0 * Cfg::Block * sizeof(OutT)
-                                                          + ((chunk ^ (r & 15u)) << 4));
-                        }
-                    };
-                    const uint32_t rdRow  = accRow;
-                    const uint32_t rdBase = rdRow * RowBytes;
-                    copyGroup(0u);
-                    copyGroup(1u);
-#pragma unroll
-                    for(uint32_t gi = 0; gi < NG; ++gi)
-                    {
-                        const uint32_t bi = gi / GroupsPerRow, bj0 = (gi % GroupsPerRow) * GB;
-                        // vector-memory operations younger than this group's copies: the next
-                        // group's copies and the stores of the two previous groups
-                        if(gi == 0u)
-                            lds::waitCopiesAndReads<CopiesC>();
-                        else if(gi == 1u)
-                            lds::waitCopiesAndReads<(NG > 2u ? CopiesC : 0u) + StoresD>();
-                        else if(gi + 1u < NG)
-                            lds::waitCopiesAndReads<CopiesC + 2u * StoresD>();
-                        else
-                            lds::waitCopiesAndReads<2u * StoresD>();
-                        asm volatile("" ::: "memory");
-                        typename Cfg::FragC io[GB];
-#pragma unroll
-                        for(uint32_t bj = 0; bj < GB; ++bj)
-#pragma unroll
-                            for(uint32_t r = 0; r < Runs; ++r)
-                            {
-                                // logical chunk of this run: block bj holds Block / 4 chunks per row
-                                const uint32_t g = bj * (Cfg::Block / 4u) + 2u * r + accGroup;
-                                detail::copyBytes<16u>(io[bj].x + 4u * r,
-                                                       myLds + (gi % 2u) * GroupBytes + rdBase + ((g ^ (rdRow & 15u)) << 4));
-                            }
-                        if(gi + 2u < NG)
-                        {
-                            lds::waitReads(); // the buffer is overwritten next
-                            asm volatile("" ::: "memory");
-                            copyGroup(gi + 2u);
-                        }
-#pragma unroll
-                        for(uint32_t bj = 0; bj < GB; ++bj)
-                        {
-#pragma unroll
-                            for(uint32_t e = 0; e < io[bj].num_elements; ++e)
-                                acc[bi][bj0 + bj].x[e] = alpha * acc[bi][bj0 + bj].x[e] + beta * static_cast<CompT>(io[bj].x[e]);
-                        }
-                        // (results replace the accumulators: every store has registers of its own)
-#pragma unroll
-                        for(uint32_t bj = 0; bj < GB; ++bj)
-                            storeBlock(d + blockOffset(bi, bj0 + bj, ldd), acc[bi][bj0 + bj], ldd);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-                else
-                {
-                typename Cfg::FragC fc[2][Cfg::BlocksN];
-                auto                loadGroup = [&](uint32_t bi) {
-                    if constexpr(PairIO)
-                    {
-#pragma unroll
-                        for(uint32_t bj = 0; bj < Cfg::BlocksN; bj += 2u)
-                            loadPair(fc[bi % 2u][bj], fc[bi % 2u][bj + 1u], c + blockOffset(bi, bj, ldc), ldc);
-                    }
-                    else
-                    {
-#pragma unroll
-                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                            load_matrix_sync(fc[bi % 2u][bj], c + blockOffset(bi, bj, ldc), ldc);
-                    }
-                };
-                loadGroup(0u);
-                if constexpr(Cfg::BlocksM > 1u)
-                    loadGroup(1u);
-#pragma unroll
-                for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
-                {
-#pragma unroll
-                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                    {
-                        auto& io = fc[bi % 2u][bj];
-#pragma unroll
-                        for(uint32_t e = 0; e < io.num_elements; ++e)
-                            io.x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e] + beta * static_cast<CompT>(io.x[e]));
-                    }
-                    if constexpr(PairIO)
-                    {
-#pragma unroll
-                        for(uint32_t bj = 0; bj < Cfg::BlocksN; bj += 2u)
-                            storePair(d + blockOffset(bi, bj, ldd), fc[bi % 2u][bj], fc[bi % 2u][bj + 1u], ldd);
-                    }
-                    else
-                    {
-#pragma unroll
-                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                            storeBlock(d + blockOffset(bi, bj, ldd), fc[bi % 2u][bj], ldd);
-                    }
-                    if(bi + 2u < Cfg::BlocksM)
-                        loadGroup(bi + 2u);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                }
-            }
-            else
-            {
-#pragma unroll
-                for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
-                {
-                    if constexpr(std::is_same<OutT, CompT>::value)
-                    {
-                        // results replace the accumulators, so no two stores share data registers
-#pragma unroll
-                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                        {
-#pragma unroll
-                            for(uint32_t e = 0; e < acc[bi][bj].num_elements; ++e)
-                                acc[bi][bj].x[e] = alpha * acc[bi][bj].x[e];
-                        }
-#pragma unroll
-                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                            storeBlock(d + blockOffset(bi, bj, ldd), acc[bi][bj], ldd);
-                    }
-                    else
-                    {
-                        typename Cfg::FragC fd[Cfg::BlocksN];
-#pragma unroll
-                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                        {
-#pragma unroll
-                            for(uint32_t e = 0; e < fd[bj].num_elements; ++e)
-                                fd[bj].x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e]);
-                        }
-                        if constexpr(PairIO)
-                        {
-#pragma unroll
-                            for(uint32_t bj = 0; bj < Cfg::BlocksN; bj += 2u)
-                                storePair(d + blockOffset(bi, bj, ldd), fd[bj], fd[bj + 1u], ldd);
-                        }
-                        else
-                        {
-#pragma unroll
-                            for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                                storeBlock(d + blockOffset(bi, bj, ldd), fd[bj], ldd);
-                        }
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
+            gemmTile<Cfg>(tm, tn, 0u, k / Cfg::MacroK, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
         }
 
         template <typename Cfg>
