@@ -54,7 +54,9 @@ typedef enum rocwmma_amd_status
     ROCWMMA_AMD_BAD_ALIGNMENT     = 4, /* pointer or leading dimension not 16-byte aligned   */
     ROCWMMA_AMD_BAD_LEADING_DIM   = 5, /* leading dimension smaller than the matrix extent   */
     ROCWMMA_AMD_NO_DEVICE         = 6, /* no gfx950 device is current                        */
-    ROCWMMA_AMD_LAUNCH_FAILED     = 7  /* hipGetLastError() reported a launch failure        */
+    ROCWMMA_AMD_LAUNCH_FAILED     = 7, /* hipGetLastError() reported a launch failure        */
+    ROCWMMA_AMD_SCRATCH_TOO_SMALL = 8  /* the library's static scratch cannot hold what this
+                                          device needs (rocwmma_amd_gemm_streamk_static)     */
 } rocwmma_amd_status;
 
 /* Which GEMM kernel family rocwmma_amd_gemm_ex runs. */
@@ -193,6 +195,38 @@ int rocwmma_amd_gemm_streamk(int         dtype_in,
                              void*       workspace,
                              size_t      workspace_bytes,
                              void*       stream);
+
+/*
+ * rocwmma_amd_gemm_streamk without a workspace argument and without any allocation: for callers that
+ * cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it).  It has no counterpart in the reference.  The workspace is a static device array inside
+ * the library: 64 MiB + 1.25 KiB, enough for devices of up to 256 compute units
+ * (ROCWMMA_AMD_SCRATCH_TOO_SMALL on larger ones), which every GPU the library runs on holds until
+ * the process ends.  The entry point calls no hipMalloc / hipFree and no allocating library routine;
+ * the flags in the scratch are cleared by a small kernel on `stream` in front of the GEMM.  All calls
+ * on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two
+ * threads) race, so serialise them, or give the overlapping ones workspaces of their own through
+ * rocwmma_amd_gemm_streamk.
+ */
+int rocwmma_amd_gemm_streamk_static(int         dtype_in,
+                                    int         dtype_out,
+                                    int         layout_a,
+                                    int         layout_b,
+                                    int         layout_c,
+                                    uint32_t    m,
+                                    uint32_t    n,
+                                    uint32_t    k,
+                                    const void* a,
+                                    uint32_t    lda,
+                                    const void* b,
+                                    uint32_t    ldb,
+                                    const void* c,
+                                    uint32_t    ldc,
+                                    void*       d,
+                                    uint32_t    ldd,
+                                    float       alpha,
+                                    float       beta,
+                                    void*       stream);
 
 /*
  * Skinny GEMV / GEMM:  Y = alpha * A * X + beta * Y,  in place on Y.

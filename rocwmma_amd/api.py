@@ -18,7 +18,7 @@ GEMM_AUTO, GEMM_WAVE_TILE, GEMM_BLOCKED, GEMM_BLOCKED_256 = 0, 1, 2, 3
 EXPORTS = [
     "rocwmma_amd_version", "rocwmma_amd_status_string", "rocwmma_amd_device_info", "rocwmma_amd_gemm",
     "rocwmma_amd_gemm_ex", "rocwmma_amd_gemv", "rocwmma_amd_dlrm_fwd", "rocwmma_amd_dlrm_bwd",
-    "rocwmma_amd_gemm_streamk", "rocwmma_amd_gemm_streamk_workspace_size",
+    "rocwmma_amd_gemm_streamk", "rocwmma_amd_gemm_streamk_workspace_size", "rocwmma_amd_gemm_streamk_static",
 ]
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
 _AUX_LIB_NAME = "librocwmma_amd_aux.so"
@@ -62,6 +62,8 @@ def library():
         L.rocwmma_amd_gemm_ex.restype = i
         L.rocwmma_amd_gemm_streamk.argtypes = gemm_args[:-1] + [vp, ctypes.c_size_t, vp]
         L.rocwmma_amd_gemm_streamk.restype = i
+        L.rocwmma_amd_gemm_streamk_static.argtypes = gemm_args
+        L.rocwmma_amd_gemm_streamk_static.restype = i
         L.rocwmma_amd_gemm_streamk_workspace_size.argtypes = []
         L.rocwmma_amd_gemm_streamk_workspace_size.restype = ctypes.c_size_t
         L.rocwmma_amd_gemv.argtypes = [u, u, u, vp, u, vp, u, vp, u, f, f, vp]
@@ -172,6 +174,20 @@ def gemm_streamk(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, 
                                             _ptr(b), ldb, _ptr(c), ldc, _ptr(d), ldd, alpha, beta, _ptr(workspace),
                                             workspace.numel() * workspace.element_size(), _stream())
     _check(rc, "gemm_streamk")
+    return d
+
+
+def gemm_streamk_static(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, b, c, d, alpha, beta,
+                        lda=None, ldb=None, ldc=None, ldd=None):
+    """rocwmma_amd_gemm_streamk_static on device tensors (the library's own scratch, no allocation)."""
+    lda = lda if lda is not None else (k if layout_a == ROW_MAJOR else m)
+    ldb = ldb if ldb is not None else (n if layout_b == ROW_MAJOR else k)
+    nat = n if layout_c == ROW_MAJOR else m
+    ldc = ldc if ldc is not None else nat
+    ldd = ldd if ldd is not None else nat
+    rc = library().rocwmma_amd_gemm_streamk_static(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, _ptr(a),
+                                                   lda, _ptr(b), ldb, _ptr(c), ldc, _ptr(d), ldd, alpha, beta, _stream())
+    _check(rc, "gemm_streamk_static")
     return d
 
 

@@ -137,6 +137,8 @@ const char* rocwmma_amd_status_string(int status)
         return "no gfx950 device is current";
     case ROCWMMA_AMD_LAUNCH_FAILED:
         return "kernel launch failed";
+    case ROCWMMA_AMD_SCRATCH_TOO_SMALL:
+        return "the library's static scratch is too small for this device";
     default:
         return "unknown status";
     }
@@ -250,6 +252,37 @@ int rocwmma_amd_gemm_streamk(int         dtype_in,
     int      la = layout_a, lb = layout_b;
     transposeForColMajorC(args, la, lb);
     return launchGemmStreamK(dtype_in, dtype_out, la, lb, args, workspace, workspace_bytes, asStream(stream));
+}
+
+int rocwmma_amd_gemm_streamk_static(int         dtype_in,
+                                    int         dtype_out,
+                                    int         layout_a,
+                                    int         layout_b,
+                                    int         layout_c,
+                                    uint32_t    m,
+                                    uint32_t    n,
+                                    uint32_t    k,
+                                    const void* a,
+                                    uint32_t    lda,
+                                    const void* b,
+                                    uint32_t    ldb,
+                                    const void* c,
+                                    uint32_t    ldc,
+                                    void*       d,
+                                    uint32_t    ldd,
+                                    float       alpha,
+                                    float       beta,
+                                    void*       stream)
+{
+    int rc = checkGemm(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, lda, b, ldb, c, ldc, d, ldd, alpha, beta);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    GemmArgs args{m, n, k, a, b, c, d, lda, ldb, c ? ldc : ldd, ldd, alpha, beta, layout_c};
+    int      la = layout_a, lb = layout_b;
+    transposeForColMajorC(args, la, lb);
+    return launchGemmStreamKStatic(dtype_in, dtype_out, la, lb, args, asStream(stream));
 }
 
 int rocwmma_amd_gemm(int         dtype_in,

@@ -94,6 +94,8 @@ namespace rocwmma_amd
     size_t streamKWorkspaceBytes(uint32_t workgroups);
     int    launchGemmStreamK(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, void* workspace,
                              size_t workspaceBytes, hipStream_t stream);
+    // the same on the library's own scratch (a static device array): allocates nothing
+    int    launchGemmStreamKStatic(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
 
 } // namespace rocwmma_amd
 

@@ -185,6 +185,43 @@ namespace rocwmma_amd
         }
     } // namespace
 
+    // ---- the library's own scratch, for callers that cannot allocate ---------------------------
+    // A workspace for devices of up to 256 compute units, held by every device the library runs on
+    // until the process ends.  Host code never uses the array's name as an address: the device
+    // address is asked for once per device (hipGetSymbolAddress) and kept.
+    namespace
+    {
+        constexpr uint32_t kScratchWorkgroups = 256u;
+        constexpr size_t   kScratchBytes = static_cast<size_t>(kScratchWorkgroups) * kStreamKSlotBytes + 1280u; // slots + 257 flag words
+        __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+        void* scratchOfCurrentDevice()
+        {
+            constexpr int             kMaxDevices = 64;
+            static std::atomic<void*> known[kMaxDevices];
+            int                       dev = 0;
+            if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+                return nullptr;
+            void* ptr = known[dev].load(std::memory_order_acquire);
+            if(ptr)
+                return ptr;
+            if(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr)
+                return nullptr;
+            known[dev].store(ptr, std::memory_order_release);
+            return ptr;
+        }
+    } // namespace
+
+    int launchGemmStreamKStatic(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream)
+    {
+        if(streamKWorkspaceBytes(computeUnits()) > kScratchBytes)
+            return ROCWMMA_AMD_SCRATCH_TOO_SMALL;
+        void* ptr = scratchOfCurrentDevice();
+        if(!ptr)
+            return ROCWMMA_AMD_LAUNCH_FAILED;
+        return launchGemmStreamK(dtypeIn, dtypeOut, layoutA, layoutB, g, ptr, kScratchBytes, stream);
+    }
+
     size_t streamKWorkspaceBytes(uint32_t workgroups)
     {
         // slots, then the flags and the time-out marker, rounded to 256 bytes
