@@ -90,6 +90,22 @@ namespace rocwmma
             __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0), vmcnt / expcnt untouched
         }
 
+        // Ties registers that inline-assembly LDS reads (DimMajorTile::readBlock16 / readBlock32) have
+        // written to this point of the program: call it right after the wait that covers those reads
+        // and before the values are used.  The reads are outside the compiler's dependency
+        // tracking; an empty asm statement that takes each register as an in-out operand makes every
+        // later use depend on a statement that cannot be moved in front of the wait.
+        template <typename T>
+        ROCWMMA_DEVICE ROCWMMA_INLINE void pinRegisters(T& value)
+        {
+            static_assert(sizeof(T) % 4u == 0u, "whole 32-bit registers");
+            typedef uint32_t word_t __attribute__((may_alias));
+            word_t* words = reinterpret_cast<word_t*>(&value);
+#pragma unroll
+            for(uint32_t i = 0; i < sizeof(T) / 4u; ++i)
+                asm volatile("" : "+v"(words[i]));
+        }
+
         // Bare workgroup barrier (no implied memory waits: pair it with waitCopiesAndReads).
         ROCWMMA_DEVICE ROCWMMA_INLINE void barrier()
         {
@@ -247,7 +263,8 @@ namespace rocwmma
             // The transposing reads are written as inline assembly on purpose: as compiler
             // intrinsics they are assumed to alias every direct-to-LDS copy in flight and get a
             // full vmcnt(0) wait in front of them, which serialises the copy pipeline.  The price
-            // is that the caller must call lds::waitReads() before the registers are consumed.
+            // is that the caller must call lds::waitReads() (or another wait that covers LDS reads)
+            // and then lds::pinRegisters() on the destination before the registers are consumed.
             template <uint32_t KPackBytes = 16u>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
                 readBlock32(void* regs, const char* ldsTile, uint32_t dim0, uint32_t ks, uint32_t lane)

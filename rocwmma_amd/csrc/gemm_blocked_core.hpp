@@ -405,6 +405,24 @@ namespace rocwmma_amd
                 }
             };
 
+            // Fragments of a dim-major operand come from inline-assembly transposing reads: after the wait
+            // that covers those reads, their registers are tied to that point of the program.
+            auto pinFrags = [&](Frags& f) {
+                if constexpr(!Cfg::AKMajor)
+                {
+#pragma unroll
+                    for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
+                        lds::pinRegisters(f.a[i].x);
+                }
+                if constexpr(!Cfg::BKMajor)
+                {
+#pragma unroll
+                    for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
+                        lds::pinRegisters(f.b[j].x);
+                }
+                (void)f;
+            };
+
             typename Cfg::FragAcc acc[Cfg::BlocksM][Cfg::BlocksN];
 #pragma unroll
             for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
@@ -442,6 +460,7 @@ namespace rocwmma_amd
                     if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
                     {
                         lds::waitReads(); // transposing reads of the previous phase
+                        pinFrags(f0);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                     readFrags(f1, i % 2u, 1u);
@@ -449,6 +468,7 @@ namespace rocwmma_amd
                     scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                     __builtin_amdgcn_sched_barrier(0);
                     lds::waitCopiesAndReads<0u>(); // stage i+1 has landed, stage i is in registers
+                    pinFrags(f1);
                     lds::barrier();
                     __builtin_amdgcn_sched_barrier(0);
                     issueStage(i % 2u, i + 3u < stages);
@@ -479,6 +499,7 @@ namespace rocwmma_amd
                     if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
                     {
                         lds::waitReads(); // fragments read during the previous phase
+                        pinFrags(f0);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                     issueA((i + S - 1u) % S);
@@ -491,6 +512,7 @@ namespace rocwmma_amd
                     __builtin_amdgcn_sched_barrier(0); // nothing moves across the synchronisation point
                     // stage i+1 has landed once only stage i+2 and the A half of stage i+3 are in flight
                     lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies + Cfg::CopiesA>();
+                    pinFrags(f1);
                     lds::barrier();
                     __builtin_amdgcn_sched_barrier(0);
                     issueB((i + S - 1u) % S);
@@ -507,12 +529,14 @@ namespace rocwmma_amd
                     if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
                     {
                         lds::waitReads();
+                        pinFrags(f0);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                     readFrags(f1, i % S, 1u);
                     multiply(f0);
                     __builtin_amdgcn_sched_barrier(0);
                     lds::waitCopiesAndReads<0u>();
+                    pinFrags(f1);
                     lds::barrier();
                     __builtin_amdgcn_sched_barrier(0);
                     if(more)
@@ -572,6 +596,7 @@ namespace rocwmma_amd
             phaseByColumns(CUR, NXT, ((STAGE) + 1u) % S);                                               \
         __builtin_amdgcn_sched_barrier(0);                                                              \
         lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies>();                                              \
+        pinFrags(NXT);                                                                                  \
         lds::barrier();                                                                                 \
         __builtin_amdgcn_sched_barrier(0);                                                              \
     } while(0)
@@ -585,6 +610,7 @@ namespace rocwmma_amd
                 if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
                 {
                     lds::waitReads(); // the transposing reads are outside the compiler's tracking
+                    pinFrags(f0);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 uint32_t s = 0;
