@@ -73,6 +73,27 @@ namespace rocwmma_amd
             return launchStatus();
         }
 
+        // The 4-wave configurations come with either LDS pipeline.  With at most one workgroup per
+        // compute unit a launch is one round of latency-bound workgroups, and the ring of four 64-byte
+        // stages (copies three stages ahead) hides more of it: 128 x 14336 x 4096 int8 25.8 against 29.7 us,
+        // 2048^3 f16 24 against 27 us.  With more workgroups than compute units the units stream operands
+        // all the time, the L2 request rate limits them, and the ring of two 128-byte stages (whole-line
+        // requests) wins: 512 x 14336 x 4096 int8 51 -> 44 us, f16 with a row-major B 101 -> 85 us,
+        // 192 x 14336 x 4096 f16 (64 x 64 tiles) 74 -> 56 us.  Results are identical bit for bit.
+        template <typename Ring4, typename Ring2>
+        int launchByRounds(GemmArgs const& g, hipStream_t stream)
+        {
+            static_assert(Ring4::MacroM == Ring2::MacroM && Ring4::MacroN == Ring2::MacroN, "same tiling");
+            if(g.m % Ring4::MacroM == 0u && g.n % Ring4::MacroN == 0u
+               && (g.m / Ring4::MacroM) * (g.n / Ring4::MacroN) > computeUnits())
+            {
+                const int rc = launchCfg<Ring2>(g, stream);
+                if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE) // (K not in whole 128-byte stages)
+                    return rc;
+            }
+            return launchCfg<Ring4>(g, stream);
+        }
+
         // Tile ladder: the 256 x 256 macro tile when the problem divides into enough of them to occupy
         // at least half of the compute units, else 128 x 128; when that gives at most one tile per two
         // compute units (few token rows against a wide weight matrix), 128 x 64 tiles double the
@@ -97,6 +118,9 @@ namespace rocwmma_amd
             // tiles than compute units then ran in whole rounds: 512 x 14336 x 4096 f16 90 -> 77 us,
             // 256 x 14336 x 4096 fp8 36 -> 30 us)
             using Small  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2, 4, 2>;
+            // the same tiles on the ring of two 128-byte stages, for more than one workgroup per
+            // compute unit (see launchByRounds)
+            using Small2 = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2, 2, 2>;
             // (a 256 x 256 tiling that covers less than half of the compute units loses to 128 x 128
             // tiles: 2048^3 f16 47 -> 24 us, 1024^3 30 -> 9 us, 512 x 14336 x 4096 int8 51 -> 42 us;
             // from 144 tiles on 256 units the large tile wins again)
@@ -149,7 +173,7 @@ namespace rocwmma_amd
                 }
             }
             {
-                int rc = launchCfg<Small>(g, stream);
+                int rc = launchByRounds<Small, Small2>(g, stream);
                 if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
                     return rc;
             }
@@ -157,8 +181,9 @@ namespace rocwmma_amd
             // (K-contiguous operands only: the dim-major LDS tile is at least 128 wide)
             if constexpr(AK && BK)
             {
-                using Tiny = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 1, 4, 4>;
-                return launchCfg<Tiny>(g, stream);
+                using Tiny  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 1, 4, 4>;
+                using Tiny2 = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 1, 2, 4>;
+                return launchByRounds<Tiny, Tiny2>(g, stream);
             }
             else
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;

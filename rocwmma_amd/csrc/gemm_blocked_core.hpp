@@ -117,7 +117,7 @@ namespace rocwmma_amd
             static_assert(BytesA % (1024u * Waves) == 0u && BytesB % (1024u * Waves) == 0u,
                           "a stage must split into whole-wave copies evenly");
             static_assert((Stages - 1u) * Copies < 64u, "too many copies in flight for vmcnt");
-            static_assert(Stages != 2u || KSteps == 2u, "the ring of two runs two MFMA steps per stage");
+            static_assert(Stages != 2u || KSteps == 2u || KSteps == 4u, "the ring of two runs two or four MFMA steps per stage");
             static_assert(LdsBytes <= Constants::AMDGCN_LDS_MAX_SIZE_BYTES, "macro tile does not fit the LDS");
             // the dim-major tile's swizzle looks at K row bits 0..3: a wave's copies must all start
             // on the same K row modulo 16
@@ -443,37 +443,42 @@ namespace rocwmma_amd
 
             if constexpr(S == 2u)
             {
-                // Ring of two stages of 128 bytes of K (two MFMA steps each).  A phase multiplies one
-                // step while it reads the fragments of the next; the barrier in the middle of an
-                // iteration is where stage i has been read completely and stage i+1 has landed, so
+                // Ring of two stages of 128 bytes of K (two or four MFMA steps each).  A phase multiplies
+                // one step while it reads the fragments of the next; the barrier in front of a stage's
+                // last phase is where stage i has been read completely and stage i+1 has landed, so
                 // the copies of stage i+2 go out right behind it, into stage i's slot, and have the
-                // two phases up to the next barrier to land.  Past the end of K the loop copies the
+                // phases up to the next barrier to land.  Past the end of K the loop copies the
                 // last stage again and reads fragments nobody multiplies, so its body is uniform.
                 issueStage(0u, 1u < stages);
                 issueStage(1u, 2u < stages);
                 lds::waitCopiesAndReads<Cfg::Copies>(); // stage 0 has landed
                 lds::barrier();
-                Frags f0, f1;
-                readFrags(f0, 0u, 0u);
+                constexpr uint32_t N = Cfg::KSteps; // MFMA steps per stage: 2 or 4 (even: the fragment sets alternate)
+                Frags              f[2];
+                readFrags(f[0], 0u, 0u);
                 for(uint32_t i = 0; i < stages; ++i)
                 {
-                    if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
+#pragma unroll
+                    for(uint32_t ks = 0; ks + 1u < N; ++ks)
                     {
-                        lds::waitReads(); // transposing reads of the previous phase
-                        pinFrags(f0);
+                        if constexpr(!Cfg::AKMajor || !Cfg::BKMajor)
+                        {
+                            lds::waitReads(); // transposing reads of the previous phase
+                            pinFrags(f[ks & 1u]);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        readFrags(f[(ks + 1u) & 1u], i % 2u, ks + 1u);
+                        multiply(f[ks & 1u]);
+                        scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    readFrags(f1, i % 2u, 1u);
-                    multiply(f0);
-                    scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
-                    __builtin_amdgcn_sched_barrier(0);
                     lds::waitCopiesAndReads<0u>(); // stage i+1 has landed, stage i is in registers
-                    pinFrags(f1);
+                    pinFrags(f[(N - 1u) & 1u]);
                     lds::barrier();
                     __builtin_amdgcn_sched_barrier(0);
                     issueStage(i % 2u, i + 3u < stages);
-                    readFrags(f0, (i + 1u) % 2u, 0u);
-                    multiply(f1);
+                    readFrags(f[0], (i + 1u) % 2u, 0u);
+                    multiply(f[(N - 1u) & 1u]);
                     scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                     scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::Copies>();
                     __builtin_amdgcn_sched_barrier(0);

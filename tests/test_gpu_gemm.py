@@ -366,6 +366,28 @@ def test_blocked_kernel_tile_ladder(dtype_in, m, n):
     check(dtype_in, out, got, want, tol_for(dtype_in))
 
 
+@pytest.mark.parametrize("la,lb", [(RM, CM), (CM, RM), (RM, RM)])
+@pytest.mark.parametrize("dtype_in,m,n,k", [(orc.F16, 2176, 2176, 448), (orc.F16, 1088, 1088, 320), (orc.I8, 2176, 2304, 640),
+                                            (orc.E4M3, 1088, 1216, 384), (orc.BF16, 2176, 2176, 96)])
+def test_blocked_kernel_more_workgroups_than_compute_units(dtype_in, m, n, k, la, lb):
+    """128 x 128 and 64 x 64 tilings with more tiles than a 256-unit device has compute units run on the
+    ring of two 128-byte K stages (with K in whole stages; the last case, K = 96, stays on the ring of
+    four); an odd number of stages and every layout pair the types allow."""
+    if dtype_in in (orc.I8, orc.E4M3) and (la, lb) != (RM, CM):
+        pytest.skip("8-bit operands: the blocked kernel takes the K-contiguous pairing only")
+    if (m % 128 != 0) and (la, lb) != (RM, CM):
+        pytest.skip("64 x 64 tiles: K-contiguous operands only")
+    if dtype_in in (orc.E4M3,):
+        a, b = normal_fp8_bits(81, dtype_in, m * k), normal_fp8_bits(82, dtype_in, k * n)
+    else:
+        a, b = uniform_bits(81, dtype_in, m * k), uniform_bits(82, dtype_in, k * n)
+    out = OUT_OF[dtype_in]
+    c = uniform_bits(83, out, m * n)
+    got = run_gemm(dtype_in, out, la, lb, RM, m, n, k, a, b, c, 1.0, 1.0, rw.GEMM_BLOCKED)
+    want = orc.gemm(dtype_in, out, la, lb, RM, RM, m, n, k, a, b, c, 1.0, 1.0)
+    check(dtype_in, out, got, want, tol_for(dtype_in))
+
+
 @pytest.mark.parametrize("m,n,k", [(16, 352, 2048), (16, 14336, 4096), (32, 352, 2048), (32, 352, 4096),
                                    (48, 1040, 1536), (80, 352, 4096), (112, 352, 1024)])
 @pytest.mark.parametrize("dtype_in", [orc.F16, orc.BF16])
