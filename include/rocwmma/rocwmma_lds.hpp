@@ -56,6 +56,15 @@ namespace rocwmma
             return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7FFFFFFF, 0x00020000);
         }
 
+        // The same with the window ending at `end` (one past the last readable byte; at most 2 GiB
+        // from `base`): copies of bytes beyond it read nothing and store zeros.
+        ROCWMMA_DEVICE ROCWMMA_INLINE BufferRsrc makeSource(const void* base, const void* end)
+        {
+            const ptrdiff_t left  = static_cast<const char*>(end) - static_cast<const char*>(base);
+            const int       bytes = left <= 0 ? 0 : (left > 0x7FFFFFFF ? 0x7FFFFFFF : static_cast<int>(left));
+            return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+        }
+
         ROCWMMA_DEVICE ROCWMMA_INLINE void asyncCopy16(void* ldsBase, BufferRsrc src, uint32_t laneOffset, uint32_t waveOffset)
         {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(

@@ -25,14 +25,14 @@ namespace rocwmma_amd
                           typename Cfg::CompT        beta)
         {
             uint32_t tm, tn;
-            tileOfWorkgroup(blockIdx.x, m / Cfg::MacroM, n / Cfg::MacroN, tm, tn);
-            gemmTile<Cfg>(tm, tn, 0u, k / Cfg::MacroK, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
+            tileOfWorkgroup(blockIdx.x, ceilDiv(m, Cfg::MacroM), ceilDiv(n, Cfg::MacroN), tm, tn);
+            gemmTile<Cfg>(tm, tn, 0u, k / Cfg::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
         }
 
         template <typename Cfg>
         int launchCfg(GemmArgs const& g, hipStream_t stream)
         {
-            if(g.m % Cfg::MacroM != 0u || g.n % Cfg::MacroN != 0u || g.k % Cfg::MacroK != 0u
+            if((!Cfg::Edges && (g.m % Cfg::MacroM != 0u || g.n % Cfg::MacroN != 0u)) || g.k % Cfg::MacroK != 0u
                || g.k < (Cfg::Stages - 1u) * Cfg::MacroK)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             // a stage's copies address their source inside a 2 GiB window from the stage origin
@@ -51,7 +51,7 @@ namespace rocwmma_amd
                                    static_cast<int>(Cfg::LdsBytes))
                != hipSuccess)
                 return ROCWMMA_AMD_LAUNCH_FAILED;
-            const uint32_t tiles = (g.m / Cfg::MacroM) * (g.n / Cfg::MacroN);
+            const uint32_t tiles = ceilDiv(g.m, Cfg::MacroM) * ceilDiv(g.n, Cfg::MacroN);
             hipLaunchKernelGGL(kernel,
                                dim3(tiles),
                                dim3(Cfg::Threads),
@@ -84,8 +84,7 @@ namespace rocwmma_amd
         int launchByRounds(GemmArgs const& g, hipStream_t stream)
         {
             static_assert(Ring4::MacroM == Ring2::MacroM && Ring4::MacroN == Ring2::MacroN, "same tiling");
-            if(g.m % Ring4::MacroM == 0u && g.n % Ring4::MacroN == 0u
-               && (g.m / Ring4::MacroM) * (g.n / Ring4::MacroN) > computeUnits())
+            if(ceilDiv(g.m, Ring4::MacroM) * ceilDiv(g.n, Ring4::MacroN) > computeUnits())
             {
                 const int rc = launchCfg<Ring2>(g, stream);
                 if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE) // (K not in whole 128-byte stages)
@@ -183,10 +182,15 @@ namespace rocwmma_amd
             {
                 using Tiny  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 1, 4, 4>;
                 using Tiny2 = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 1, 2, 4>;
-                return launchByRounds<Tiny, Tiny2>(g, stream);
+                int rc      = launchByRounds<Tiny, Tiny2>(g, stream);
+                if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                    return rc;
             }
-            else
-                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            // any other multiples of 16: 128 x 128 tiles, the last row and column of tiles partly
+            // filled (the wave-tile kernel, which these shapes used to fall to, is 2-3x slower)
+            using Edge  = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2, 4, 2, 32, true>;
+            using Edge2 = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2, 2, 2, 32, true>;
+            return launchByRounds<Edge, Edge2>(g, stream);
         }
 
         template <typename InT, typename OutT, typename CompT>

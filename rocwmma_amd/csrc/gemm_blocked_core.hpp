@@ -48,7 +48,8 @@ namespace rocwmma_amd
                   uint32_t BlocksN_,
                   uint32_t Stages_       = 4u, // LDS ring depth
                   uint32_t WavesPerSimd_ = 1u, // waves per SIMD: sizes the register budget, and no more become resident
-                  uint32_t BlockEdge_    = 32u> // MFMA block edge: 32 (32x32xK) or 16 (16x16x2K)
+                  uint32_t BlockEdge_    = 32u, // MFMA block edge: 32 (32x32xK) or 16 (16x16x2K)
+                  bool     Edges_        = false> // M and N need not fill whole macro tiles (multiples of 16 do)
         struct BlockedConfig
         {
             using InT   = InT_;
@@ -57,6 +58,10 @@ namespace rocwmma_amd
 
             static constexpr bool     AKMajor = AKMajor_;
             static constexpr bool     BKMajor = BKMajor_;
+            // Partly filled tiles at the lower and right edges of C/D: operand reads past a matrix end
+            // are cut off by the buffer bounds (rows and columns beyond the problem only ever meet
+            // results beyond it), C reads and D stores are masked lane by lane.
+            static constexpr bool     Edges   = Edges_;
             static constexpr uint32_t WavesM  = WavesM_;
             static constexpr uint32_t WavesN  = WavesN_;
             static constexpr uint32_t BlocksM = BlocksM_;
@@ -105,7 +110,7 @@ namespace rocwmma_amd
             // GroupBlocks blocks (256- or 512-byte rows), two group buffers per wave
             static constexpr uint32_t GroupBlocks
                 = (WaveN == 128u && 2u * Block * 128u * sizeof(OutT) * Waves <= LdsBytes) ? 128u / Block : 64u / Block;
-            static constexpr bool StagedC = sizeof(OutT) == 4u && WaveN % 64u == 0u
+            static constexpr bool StagedC = !Edges && sizeof(OutT) == 4u && WaveN % 64u == 0u
                                             && BlocksM * (BlocksN / GroupBlocks) >= 2u
                                             && 2u * Block * GroupBlocks * Block * sizeof(OutT) * Waves <= LdsBytes;
 
@@ -299,6 +304,9 @@ namespace rocwmma_amd
                                                     uint32_t                   tn,
                                                     uint32_t                   stage0,
                                                     uint32_t                   stages,
+                                                    uint32_t                   m, // problem size: used by
+                                                    uint32_t                   n, // configurations with edge
+                                                    uint32_t                   k, // tiles only
                                                     typename Cfg::InT const*   a,
                                                     typename Cfg::InT const*   b,
                                                     typename Cfg::OutT const*  c,
@@ -340,6 +348,11 @@ namespace rocwmma_amd
                                + static_cast<size_t>(row0) * (Cfg::AKMajor ? ldaB : static_cast<uint32_t>(sizeof(InT)));
             const char* bSrc = reinterpret_cast<const char*>(b)
                                + static_cast<size_t>(col0) * (Cfg::BKMajor ? ldbB : static_cast<uint32_t>(sizeof(InT)));
+            // one past the last byte of each operand (edge tiles: the buffer bounds end there)
+            const char* const aEnd = reinterpret_cast<const char*>(a)
+                                     + (static_cast<size_t>((Cfg::AKMajor ? m : k) - 1u) * lda + (Cfg::AKMajor ? k : m)) * sizeof(InT);
+            const char* const bEnd = reinterpret_cast<const char*>(b)
+                                     + (static_cast<size_t>((Cfg::BKMajor ? n : k) - 1u) * ldb + (Cfg::BKMajor ? k : n)) * sizeof(InT);
             const size_t   aStep    = TileA::stageStep(ldaB);
             const size_t   bStep    = TileB::stageStep(ldbB);
             aSrc += aStep * stage0; // (the whole K range starts at stage 0)
@@ -353,7 +366,7 @@ namespace rocwmma_amd
             // stage instead of running past the end of the operand)
             auto issueA = [&](uint32_t slot, bool advance = true) {
                 char*                 ldsA = ldsRaw + slot * Cfg::StageBytes;
-                const lds::BufferRsrc src  = lds::makeSource(aSrc);
+                const lds::BufferRsrc src  = Cfg::Edges ? lds::makeSource(aSrc, aEnd) : lds::makeSource(aSrc);
 #pragma unroll
                 for(uint32_t i = 0; i < Cfg::CopiesA; ++i)
                 {
@@ -364,7 +377,7 @@ namespace rocwmma_amd
             };
             auto issueB = [&](uint32_t slot, bool advance = true) {
                 char*                 ldsB = ldsRaw + slot * Cfg::StageBytes + Cfg::BytesA;
-                const lds::BufferRsrc src  = lds::makeSource(bSrc);
+                const lds::BufferRsrc src  = Cfg::Edges ? lds::makeSource(bSrc, bEnd) : lds::makeSource(bSrc);
 #pragma unroll
                 for(uint32_t i = 0; i < Cfg::CopiesB; ++i)
                 {
@@ -657,14 +670,38 @@ namespace rocwmma_amd
             constexpr uint32_t Runs     = Cfg::Block == 32u ? 4u : 1u; // runs per block per lane
             const uint32_t     accRow   = lane & (Cfg::Block - 1u);
             const uint32_t     accGroup = lane / Cfg::Block; // 0..1 or 0..3
-            auto storeBlock = [&](OutT* dst, auto const& f, uint32_t ld) {
+            // (edge tiles: a lane's run of four columns of one row is inside the problem or outside it
+            // as a whole, N being a multiple of 16)
+            auto inside = [&](uint32_t bi, uint32_t bj, uint32_t r) {
+                return wRow + bi * Cfg::Block + accRow < m && wCol + bj * Cfg::Block + 8u * r + 4u * accGroup < n;
+            };
+            auto storeBlock = [&](uint32_t bi, uint32_t bj, auto const& f) {
                 typedef uint32_t Words __attribute__((ext_vector_type(sizeof(OutT))));
+                OutT* dst = d + static_cast<size_t>(wRow + bi * Cfg::Block) * ldd + wCol + bj * Cfg::Block;
 #pragma unroll
                 for(uint32_t r = 0; r < Runs; ++r)
                 {
                     Words v;
                     __builtin_memcpy(&v, f.x + 4u * r, sizeof(v));
-                    *reinterpret_cast<Words*>(dst + static_cast<size_t>(accRow) * ld + 8u * r + 4u * accGroup) = v;
+                    if(!Cfg::Edges || inside(bi, bj, r))
+                        *reinterpret_cast<Words*>(dst + static_cast<size_t>(accRow) * ldd + 8u * r + 4u * accGroup) = v;
+                }
+            };
+            auto loadBlockC = [&](uint32_t bi, uint32_t bj, auto& f) {
+                const OutT* src = c + static_cast<size_t>(wRow + bi * Cfg::Block) * ldc + wCol + bj * Cfg::Block;
+                if constexpr(!Cfg::Edges)
+                    load_matrix_sync(f, src, ldc);
+                else
+                {
+                    typedef uint32_t Words __attribute__((ext_vector_type(sizeof(OutT))));
+#pragma unroll
+                    for(uint32_t r = 0; r < Runs; ++r)
+                    {
+                        Words v = {};
+                        if(inside(bi, bj, r))
+                            v = *reinterpret_cast<const Words*>(src + static_cast<size_t>(accRow) * ldc + 8u * r + 4u * accGroup);
+                        __builtin_memcpy(f.x + 4u * r, &v, sizeof(v));
+                    }
                 }
             };
             // 16-bit outputs with 16-wide blocks: a lane's run is only 8 bytes, a store instruction would
@@ -674,7 +711,7 @@ namespace rocwmma_amd
             // (even rows: of the first block, odd rows: of the second) and moves 16 bytes; an
             // instruction then covers 64 contiguous bytes per matrix row.  The exchange is its own
             // inverse, so C is read the same way.
-            constexpr bool PairIO = Cfg::Block == 16u && sizeof(OutT) == 2u && Cfg::BlocksN % 2u == 0u;
+            constexpr bool PairIO = !Cfg::Edges && Cfg::Block == 16u && sizeof(OutT) == 2u && Cfg::BlocksN % 2u == 0u;
             const uint32_t pairCol = (accGroup & 1u) * 16u + 4u * (accGroup & 2u);
             auto           swapPair = [](auto& fx, auto& fy) {
                 uint32_t x[2], y[2];
@@ -793,7 +830,7 @@ namespace rocwmma_amd
                         // (results replace the accumulators: every store has registers of its own)
 #pragma unroll
                         for(uint32_t bj = 0; bj < GB; ++bj)
-                            storeBlock(d + blockOffset(bi, bj0 + bj, ldd), acc[bi][bj0 + bj], ldd);
+                            storeBlock(bi, bj0 + bj, acc[bi][bj0 + bj]);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
@@ -811,7 +848,7 @@ namespace rocwmma_amd
                     {
 #pragma unroll
                         for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                            load_matrix_sync(fc[bi % 2u][bj], c + blockOffset(bi, bj, ldc), ldc);
+                            loadBlockC(bi, bj, fc[bi % 2u][bj]);
                     }
                 };
                 loadGroup(0u);
@@ -838,7 +875,7 @@ namespace rocwmma_amd
                     {
 #pragma unroll
                         for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                            storeBlock(d + blockOffset(bi, bj, ldd), fc[bi % 2u][bj], ldd);
+                            storeBlock(bi, bj, fc[bi % 2u][bj]);
                     }
                     if(bi + 2u < Cfg::BlocksM)
                         loadGroup(bi + 2u);
@@ -863,7 +900,7 @@ namespace rocwmma_amd
                         }
 #pragma unroll
                         for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                            storeBlock(d + blockOffset(bi, bj, ldd), acc[bi][bj], ldd);
+                            storeBlock(bi, bj, acc[bi][bj]);
                     }
                     else
                     {
@@ -885,7 +922,7 @@ namespace rocwmma_amd
                         {
 #pragma unroll
                             for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
-                                storeBlock(d + blockOffset(bi, bj, ldd), fd[bj], ldd);
+                                storeBlock(bi, bj, fd[bj]);
                         }
                     }
                     __builtin_amdgcn_sched_barrier(0);

@@ -46,7 +46,7 @@ namespace rocwmma_amd
                           uint32_t                   wholeRounds)
         {
             const uint32_t workgroups = gridDim.x;
-            const uint32_t tilesM = m / Cfg::MacroM, tilesN = n / Cfg::MacroN;
+            const uint32_t tilesM = m / Cfg::MacroM, tilesN = n / Cfg::MacroN; // (whole tiles: checked by the host)
             const uint32_t stagesPerTile = k / Cfg::MacroK;
             const uint32_t roundTiles    = wholeRounds * workgroups; // tile ids [0, roundTiles): one per workgroup and round
             const uint32_t splitTiles    = tilesM * tilesN - roundTiles; // tile ids behind them: shared by K range
@@ -75,7 +75,7 @@ namespace rocwmma_amd
                 const uint32_t count  = min(stagesPerTile - stage0, uEnd - u);
                 tileOf(roundTiles + u / stagesPerTile, tm, tn);
                 sk.mySlot = range;
-                gemmTile<Cfg, TilePart::Contributor>(tm, tn, stage0, count, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, sk);
+                gemmTile<Cfg, TilePart::Contributor>(tm, tn, stage0, count, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, sk);
                 u += count;
                 __syncthreads(); // the next tile's copies reuse the LDS
             }
@@ -83,7 +83,7 @@ namespace rocwmma_amd
             for(uint32_t r = 0; r < wholeRounds; ++r)
             {
                 tileOf(r * workgroups + blockIdx.x, tm, tn);
-                gemmTile<Cfg>(tm, tn, 0u, stagesPerTile, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, sk);
+                gemmTile<Cfg>(tm, tn, 0u, stagesPerTile, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, sk);
                 __syncthreads();
             }
             // 3. the rest of the range: whole split tiles, then a part that starts at K = 0
@@ -92,7 +92,7 @@ namespace rocwmma_amd
                 const uint32_t count = min(stagesPerTile, uEnd - u);
                 tileOf(roundTiles + u / stagesPerTile, tm, tn);
                 if(count == stagesPerTile)
-                    gemmTile<Cfg>(tm, tn, 0u, stagesPerTile, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, sk);
+                    gemmTile<Cfg>(tm, tn, 0u, stagesPerTile, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, sk);
                 else
                 {
                     // the parts behind this one: the ranges that start before the tile ends
@@ -101,7 +101,7 @@ namespace rocwmma_amd
                     sk.slotCount           = 0u;
                     while(sk.firstSlot + sk.slotCount < workgroups && rangeStart(sk.firstSlot + sk.slotCount) < tileEnd)
                         ++sk.slotCount;
-                    gemmTile<Cfg, TilePart::Owner>(tm, tn, 0u, count, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, sk);
+                    gemmTile<Cfg, TilePart::Owner>(tm, tn, 0u, count, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, sk);
                 }
                 u += count;
                 __syncthreads();

@@ -388,6 +388,45 @@ def test_blocked_kernel_more_workgroups_than_compute_units(dtype_in, m, n, k, la
     check(dtype_in, out, got, want, tol_for(dtype_in))
 
 
+@pytest.mark.parametrize("la,lb,lc", [(RM, CM, RM), (CM, RM, RM), (RM, RM, CM), (CM, CM, RM)])
+@pytest.mark.parametrize("dtype_in,dtype_out,m,n,k", [
+    (orc.F16, orc.F32, 144, 208, 256), (orc.F16, orc.F32, 2064, 2192, 192), (orc.F16, orc.F16, 400, 16, 128),
+    (orc.BF16, orc.BF16, 16, 400, 320), (orc.I8, orc.I32, 272, 1040, 512), (orc.I8, orc.I8, 1936, 2320, 256),
+    (orc.E4M3, orc.F32, 656, 48, 384), (orc.E5M2, orc.F32, 2160, 2064, 256)])
+def test_blocked_kernel_partly_filled_edge_tiles(dtype_in, dtype_out, m, n, k, la, lb, lc):
+    """M and N that are multiples of 16 but not of 64 run on 128 x 128 tiles whose last row and column
+    are partly filled (operand reads beyond a matrix end cut off by the buffer bounds, C reads and D
+    stores masked); one and many tiles, more tiles than compute units, with and without beta.  D is
+    allocated to size and framed by a guard region that must stay untouched."""
+    import torch
+
+    if dtype_in in (orc.I8, orc.E4M3, orc.E5M2) and (la, lb) != (RM, CM):
+        pytest.skip("8-bit operands: the blocked kernel takes the K-contiguous pairing only")
+    if dtype_in in (orc.E4M3, orc.E5M2):
+        a, b = normal_fp8_bits(85, dtype_in, m * k), normal_fp8_bits(86, dtype_in, k * n)
+    elif dtype_in == orc.I8 and dtype_out == orc.I8:
+        rng = np.random.default_rng(85)
+        a, b = rng.integers(-3, 4, m * k, dtype=np.int8), rng.integers(-3, 4, k * n, dtype=np.int8)
+    else:
+        a, b = uniform_bits(85, dtype_in, m * k), uniform_bits(86, dtype_in, k * n)
+    c = uniform_bits(87, dtype_out, m * n)
+    tol = 4e-3 if dtype_out == orc.BF16 else tol_for(dtype_in)
+    np_out = orc.storage_dtype(dtype_out)
+    guard = 4096
+    for alpha, beta in [(1.0, 0.0), (2.0, -1.0)]:
+        frame = np.zeros(m * n + 2 * guard, dtype=np_out)
+        frame[:] = 0x55 if np_out != np.float32 else 12345.0
+        dev = to_device(frame)
+        d = dev[guard:guard + m * n]
+        rw.gemm(dtype_in, dtype_out, la, lb, lc, m, n, k, to_device(a), to_device(b), to_device(c), d, alpha, beta,
+                algo=rw.GEMM_BLOCKED)
+        torch.cuda.synchronize()
+        host = to_host(dev, np_out)
+        assert np.array_equal(host[:guard], frame[:guard]) and np.array_equal(host[-guard:], frame[-guard:]), "wrote outside D"
+        want = orc.gemm(dtype_in, dtype_out, la, lb, lc, lc, m, n, k, a, b, c, alpha, beta)
+        check(dtype_in, dtype_out, host[guard:guard + m * n], want, tol)
+
+
 @pytest.mark.parametrize("m,n,k", [(16, 352, 2048), (16, 14336, 4096), (32, 352, 2048), (32, 352, 4096),
                                    (48, 1040, 1536), (80, 352, 4096), (112, 352, 1024)])
 @pytest.mark.parametrize("dtype_in", [orc.F16, orc.BF16])
