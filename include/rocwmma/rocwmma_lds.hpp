@@ -18,7 +18,7 @@
 //
 //   KMajorTile   -- one operand row per LDS row (row-major A / col-major B).
 //   DimMajorTile -- one K index per LDS row of Dim elements (col-major A / row-major B),
-//                   16-bit elements only.
+//                   16-bit elements; DimMajorTile8 is its 8-bit twin (ds_read_b64_tr_b8).
 #ifndef ROCWMMA_LDS_HPP
 #define ROCWMMA_LDS_HPP
 
@@ -321,6 +321,106 @@ namespace rocwmma
                     asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
                     reinterpret_cast<s16x4*>(regs)[kk] = v;
                 }
+            }
+        };
+
+
+        // ---------------------------------------------------------------------------------
+        // Dim-major stage of 8-bit elements (int8, fp8): KRows LDS rows (one per K index) of Dim bytes,
+        // cut into 16-byte segments; segment s of K row k lives at segment position s ^ swz(k).
+        //
+        // ds_read_b64_tr_b8, found by reading a table of byte ids back: within each group of 16 lanes,
+        // result lane t receives, as its byte j (0..7), byte t % 8 of the 8 bytes that lane
+        // 2 j + t / 8 of the group addressed.  With lanes 2 j and 2 j + 1 pointing at the two halves of
+        // 16 consecutive elements of K row k0 + j, lane t ends up with element t of the K rows
+        // k0 .. k0 + 7: a transposed 8 x 16 block, eight consecutive K values per lane.
+        //
+        // A group's read touches 8 K rows at one segment; rows are Dim bytes apart (a multiple of 128), so
+        // swz must spread the rows of one read, and of the two lane groups served together (K rows 16
+        // apart for 16-wide blocks), over distinct 16-byte bank groups: the low K bits, and bit 4 above them.
+        // ---------------------------------------------------------------------------------
+        template <uint32_t Dim, uint32_t KRows>
+        struct DimMajorTile8
+        {
+            static_assert(Dim == 128u || Dim == 256u, "tile rows of 128 or 256 bytes");
+            static_assert(KRows == 64u || KRows == 128u, "stages of 64 or 128 K rows");
+            static constexpr uint32_t kRows       = KRows;
+            static constexpr uint32_t rowBytes    = Dim;
+            static constexpr uint32_t bytes       = kRows * rowBytes;
+            static constexpr uint32_t copies      = bytes / 1024u;
+            static constexpr uint32_t slotsPerRow = rowBytes / 16u; // 8 or 16 segments
+            static constexpr uint32_t rowsPerCopy = 64u / slotsPerRow; // 8 or 4 K rows per whole-wave copy
+
+            // (128-byte rows: two K rows share a 256-byte bank window, so K bit 0 already separates them)
+            ROCWMMA_HOST_DEVICE static constexpr uint32_t swz(uint32_t k)
+            {
+                return Dim == 128u ? (((k >> 1) & 3u) | (((k >> 4) & 1u) << 2)) : ((k & 7u) | (((k >> 4) & 1u) << 3));
+            }
+            ROCWMMA_HOST_DEVICE static constexpr uint32_t offset(uint32_t k, uint32_t seg)
+            {
+                return k * rowBytes + ((seg ^ swz(k)) << 4);
+            }
+            // Source byte offset of `lane` inside a copy issued by wave `wave` of a pool whose size times
+            // rowsPerCopy is a multiple of 32 (so k % 32 is the same for all of a wave's copies).
+            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t laneSourceOffset(uint32_t lane, uint32_t wave, uint32_t ldBytes)
+            {
+                const uint32_t kInCopy = lane / slotsPerRow;
+                const uint32_t pos     = lane % slotsPerRow;
+                const uint32_t k       = wave * rowsPerCopy + kInCopy; // only k % 32 matters
+                return kInCopy * ldBytes + ((pos ^ swz(k)) << 4);
+            }
+            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t copySourceOffset(uint32_t copy, uint32_t ldBytes)
+            {
+                return copy * rowsPerCopy * ldBytes;
+            }
+            ROCWMMA_DEVICE static ROCWMMA_INLINE size_t stageStep(uint32_t ldBytes)
+            {
+                return static_cast<size_t>(kRows) * ldBytes;
+            }
+
+            // One transposing read: the lane's group reads K rows k0 .. k0 + 7 of the 16 elements that
+            // start at dim16 (a multiple of 16); the lane receives element dim16 + lane % 16.
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void
+                read8(uint32_t (&out)[2], uint32_t ldsBase, uint32_t k0, uint32_t dim16, uint32_t lane)
+            {
+                typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+                const uint32_t s    = lane & 15u;
+                const uint32_t k    = k0 + (s >> 1);
+                const uint32_t addr = ldsBase + offset(k, dim16 >> 4) + ((s & 1u) << 3);
+                u32x2_t        v;
+                asm volatile("ds_read_b64_tr_b8 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+                out[0] = v[0];
+                out[1] = v[1];
+            }
+
+            // Operand of one 16-wide MFMA block with 16 K values per lane (v_mfma_i32_16x16x64_i8):
+            // lane l ends up with dim = dim0 + l % 16 and k = 64 ks + (l / 16) * 16 + 0..15.
+            // As for the 16-bit tile, the caller waits for the reads and pins the registers before use.
+            template <uint32_t KPackBytes>
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void
+                readBlock16(void* regs, const char* ldsTile, uint32_t dim0, uint32_t ks, uint32_t lane)
+            {
+                static_assert(KPackBytes == 16u, "16-wide blocks of 8-bit types take 16 bytes of K per lane");
+                const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsPtr)ldsTile));
+                const uint32_t kBase   = ks * 64u + (lane >> 4) * 16u;
+#pragma unroll
+                for(uint32_t kk = 0; kk < 2u; ++kk)
+                    read8(reinterpret_cast<uint32_t(*)[2]>(regs)[kk], ldsBase, kBase + 8u * kk, dim0, lane);
+            }
+
+            // Operand of one 32-wide MFMA block: lane l ends up with dim = dim0 + l % 32 and
+            // k = KPackBytes * (2 ks + l / 32) + 0 .. KPackBytes - 1 (16 for v_mfma_i32_32x32x32_i8, 32 for
+            // v_mfma_f32_32x32x64_f8f6f4).
+            template <uint32_t KPackBytes>
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void
+                readBlock32(void* regs, const char* ldsTile, uint32_t dim0, uint32_t ks, uint32_t lane)
+            {
+                const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsPtr)ldsTile));
+                const uint32_t kBase   = KPackBytes * (2u * ks + (lane >> 5));
+                const uint32_t dim16   = dim0 + (lane & 16u);
+#pragma unroll
+                for(uint32_t kk = 0; kk < KPackBytes / 8u; ++kk)
+                    read8(reinterpret_cast<uint32_t(*)[2]>(regs)[kk], ldsBase, kBase + 8u * kk, dim16, lane);
             }
         };
 

@@ -210,10 +210,15 @@ namespace rocwmma_amd
         template <typename InT, typename OutT, typename CompT>
         int pickLayout8(int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream, bool big)
         {
-            // 8-bit operands: only the K-contiguous pairing (row-major A, col-major B)
-            if(layoutA == ROCWMMA_AMD_ROW_MAJOR && layoutB == ROCWMMA_AMD_COL_MAJOR)
+            const bool ak = layoutA == ROCWMMA_AMD_ROW_MAJOR;
+            const bool bk = layoutB == ROCWMMA_AMD_COL_MAJOR;
+            if(ak && bk)
                 return pickTile<InT, OutT, CompT, true, true>(g, stream, big);
-            return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            if(ak && !bk)
+                return pickTile<InT, OutT, CompT, true, false>(g, stream, big);
+            if(!ak && bk)
+                return pickTile<InT, OutT, CompT, false, true>(g, stream, big);
+            return pickTile<InT, OutT, CompT, false, false>(g, stream, big);
         }
     } // namespace
 

@@ -89,8 +89,12 @@ namespace rocwmma_amd
             using FragAcc = fragment<accumulator, Block, Block, BlockK, CompT>;
             using FragC   = fragment<accumulator, Block, Block, BlockK, OutT, row_major>;
 
-            using TileA = std::conditional_t<AKMajor, lds::KMajorTile<MacroM, StageKB>, lds::DimMajorTile<MacroM, StageKB / 2u>>;
-            using TileB = std::conditional_t<BKMajor, lds::KMajorTile<MacroN, StageKB>, lds::DimMajorTile<MacroN, StageKB / 2u>>;
+            // (a dim-major tile holds one K index per LDS row: StageKB / sizeof(InT) rows)
+            template <uint32_t Dim>
+            using DimTile = std::conditional_t<sizeof(InT) == 2u, lds::DimMajorTile<Dim, StageKB / 2u>,
+                                               lds::DimMajorTile8<(Dim == 128u || Dim == 256u) ? Dim : 128u, StageKB>>;
+            using TileA = std::conditional_t<AKMajor, lds::KMajorTile<MacroM, StageKB>, DimTile<MacroM>>;
+            using TileB = std::conditional_t<BKMajor, lds::KMajorTile<MacroN, StageKB>, DimTile<MacroN>>;
 
             static constexpr uint32_t BytesA     = MacroM * StageKB;
             static constexpr uint32_t BytesB     = MacroN * StageKB;
@@ -102,8 +106,9 @@ namespace rocwmma_amd
             static constexpr uint32_t CopiesB    = BytesB / 1024u / Waves;
             static constexpr uint32_t Copies     = CopiesA + CopiesB;
             // LDS read instructions per MFMA step: b128 reads per block (K-major) or two transposing b64 reads
-            static constexpr uint32_t ReadsA       = BlocksM * (AKMajor ? KPackBytes / 16u : 2u);
-            static constexpr uint32_t ReadsB       = BlocksN * (BKMajor ? KPackBytes / 16u : 2u);
+            static constexpr uint32_t TrReads      = KPackBytes / 8u; // transposing 8-byte reads per operand
+            static constexpr uint32_t ReadsA       = BlocksM * (AKMajor ? KPackBytes / 16u : TrReads);
+            static constexpr uint32_t ReadsB       = BlocksN * (BKMajor ? KPackBytes / 16u : TrReads);
             static constexpr uint32_t ReadsPerStep = ReadsA + ReadsB;
             static constexpr uint32_t MfmasPerStep = BlocksM * BlocksN;
             // beta * C operand staged through LDS in the epilogue, in groups of Block rows by
@@ -116,8 +121,9 @@ namespace rocwmma_amd
 
             static_assert(Block == 32u || Block == 16u, "MFMA blocks are 32 or 16 wide");
             static_assert(Block == 32u || KPackBytes == 16u, "16-wide blocks: 16 bytes of K per lane (16-bit types, int8)");
-            static_assert(AKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
-            static_assert(BKMajor || sizeof(InT) == 2, "transposing LDS reads exist for 16-bit types only");
+            static_assert(sizeof(InT) == 2u || sizeof(InT) == 1u, "16-bit and 8-bit operands");
+            static_assert(sizeof(InT) == 2u || ((AKMajor || MacroM == 128u || MacroM == 256u) && (BKMajor || MacroN == 128u || MacroN == 256u)),
+                          "dim-major tiles of 8-bit operands are 128 or 256 wide");
             static_assert(TileA::bytes == BytesA && TileB::bytes == BytesB, "stage geometry mismatch");
             static_assert(BytesA % (1024u * Waves) == 0u && BytesB % (1024u * Waves) == 0u,
                           "a stage must split into whole-wave copies evenly");
@@ -126,8 +132,9 @@ namespace rocwmma_amd
             static_assert(LdsBytes <= Constants::AMDGCN_LDS_MAX_SIZE_BYTES, "macro tile does not fit the LDS");
             // the dim-major tile's swizzle looks at K row bits 0..3: a wave's copies must all start
             // on the same K row modulo 16
-            static_assert((AKMajor || (Waves * TileA::rowsPerCopy) % 16u == 0u)
-                              && (BKMajor || (Waves * TileB::rowsPerCopy) % 16u == 0u),
+            // (the 8-bit tile's looks at K row bit 4 as well)
+            static_assert((AKMajor || (Waves * TileA::rowsPerCopy) % (sizeof(InT) == 2u ? 16u : 32u) == 0u)
+                              && (BKMajor || (Waves * TileB::rowsPerCopy) % (sizeof(InT) == 2u ? 16u : 32u) == 0u),
                           "wave pool too small for the dim-major tile");
             // the K-major tile's swizzle looks at row bits 0..3 likewise
             static_assert((!AKMajor || (Waves * TileA::rowsPerCopy) % 16u == 0u)
@@ -580,8 +587,6 @@ namespace rocwmma_amd
                 auto phaseByColumns = [&](Frags const& cur, Frags& nxt, uint32_t slot) {
                     const char* ldsA = ldsRaw + slot * Cfg::StageBytes;
                     const char* ldsB = ldsA + Cfg::BytesA;
-                    static_assert(Cfg::Block == 16u || Cfg::KSteps != 1u || Cfg::BKMajor,
-                                  "one-step stages with a dim-major B use 16-wide blocks");
                     if constexpr(Cfg::Block == 16u)
                     {
                         static_assert(Cfg::BlocksM <= Cfg::BlocksN, "the A blocks are read along with the first B columns");
@@ -602,7 +607,7 @@ namespace rocwmma_amd
     do                                                                                                  \
     {                                                                                                   \
         issueStage(((STAGE) + S - 1u) % S, (STAGE) + S < stages);                                       \
-        if constexpr(Cfg::BKMajor)                                                                      \
+        if constexpr(Cfg::BKMajor || Cfg::Block != 16u)                                                 \
         {                                                                                               \
             if(READ)                                                                                    \
                 readFrags(NXT, ((STAGE) + 1u) % S, 0u);                                                 \

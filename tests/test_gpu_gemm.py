@@ -160,6 +160,23 @@ def test_8bit_types_other_layouts_wave_tile(dtype_in, la, lb):
     check(dtype_in, out, got, want, tol_for(dtype_in))
 
 
+@pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3, orc.E5M2])
+@pytest.mark.parametrize("la,lb", [(RM, RM), (CM, CM), (CM, RM)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 512), (512, 768, 384), (2176, 2304, 640), (128, 384, 320), (64, 192, 256),
+                                   (1040, 912, 448)])
+def test_8bit_types_other_layouts_blocked(dtype_in, la, lb, m, n, k):
+    """8-bit operands whose K index is not the contiguous one go through transposing LDS reads:
+    the 256-wide tile, the 128-wide tiles in both ring depths, 64-wide tiles and partly filled edge tiles.
+    Random operands, so a lane or byte that lands in the wrong place shows."""
+    a = uniform_bits(43, orc.I8, m * k) if dtype_in == orc.I8 else normal_fp8_bits(43, dtype_in, m * k)
+    b = uniform_bits(44, orc.I8, k * n) if dtype_in == orc.I8 else normal_fp8_bits(44, dtype_in, k * n)
+    out = OUT_OF[dtype_in]
+    c = uniform_bits(45, out, m * n)
+    got = run_gemm(dtype_in, out, la, lb, RM, m, n, k, a, b, c, 1.0, 1.0, rw.GEMM_BLOCKED)
+    want = orc.gemm(dtype_in, out, la, lb, RM, RM, m, n, k, a, b, c, 1.0, 1.0)
+    check(dtype_in, out, got, want, tol_for(dtype_in))
+
+
 @pytest.mark.parametrize("algo", ALGOS)
 @pytest.mark.parametrize("dtype_in", [orc.F16, orc.BF16, orc.E4M3, orc.E5M2, orc.I8])
 def test_exact_integer_pattern_is_bit_exact(dtype_in, algo):
