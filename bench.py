@@ -42,7 +42,8 @@ FP8_BLOCKED_SHAPE = "fp8_32x32x64"  # the matrix instruction of the blocked kern
 # no longer matches is reported as null.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 KERNEL_SOURCES = {
-    "gemm_blocked": ["rocwmma_amd/csrc/gemm_blocked.hip", "include/rocwmma/rocwmma_lds.hpp"],
+    "gemm_blocked": ["rocwmma_amd/csrc/gemm_blocked.hip", "rocwmma_amd/csrc/gemm_blocked_core.hpp",
+                     "include/rocwmma/rocwmma_lds.hpp"],
 }
 
 
@@ -66,6 +67,29 @@ def measured_traffic(key, family):
     return rec.get("bytes")
 
 
+def record_traffic(spec):
+    """--record-traffic KEY:FAMILY:FETCH_KIB:WRITE_KIB:COPY_FETCH_KIB:COPY_WRITE_KIB -- store what a pair of
+    rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE: per-dispatch averages of the kernel, in the counters' own
+    units) read for case KEY, scaled by what the same counters read for the 1 GiB copy of --calibrate-copy,
+    together with the digest of the kernel sources it was measured on."""
+    key, family, fetch, write, cfetch, cwrite = spec.split(":")
+    gib_kib = float(1 << 20)
+    f_factor, w_factor = gib_kib / float(cfetch), gib_kib / float(cwrite)
+    byts = (float(fetch) * f_factor + float(write) * w_factor) * 1024.0
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        table = {}
+    table[key] = {"bytes": round(byts), "fetch_size": float(fetch), "write_size": float(write),
+                  "fetch_factor": round(f_factor, 3), "write_factor": round(w_factor, 3),
+                  "sources_digest": sources_digest(family)}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(table, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(json.dumps({key: table[key]}))
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -79,6 +103,10 @@ def parse_args():
     ap.add_argument("--shapes", action="store_true",
                     help="also time GEMM shapes below the headline size, one per kernel / tile configuration "
                          "(extra.shapes in the JSON line)")
+    ap.add_argument("--no-ceiling", action="store_true",
+                    help="skip the MFMA-only ceiling loops and the all-zero-operand run (counter runs)")
+    ap.add_argument("--record-traffic", default=None, metavar="KEY:FAMILY:FETCH:WRITE:COPY_FETCH:COPY_WRITE",
+                    help="no GPU work: rewrite the entry of profiles/traffic.json for one case from counter readings")
     ap.add_argument("--only", default=None,
                     help="run one case only: a headline case such as f16_rc (dtype_{r|c}{r|c} = A,B layout) or an "
                          "extra case by its JSON key (gemm_fp8_m4096, gemv_8192x8192_n8, ...): for profiling")
@@ -143,6 +171,9 @@ HEADLINE_TAGS = [f"{d}_{a}{b}" for d in ("f16", "bf16") for a in "rc" for b in "
 
 def main():
     args = parse_args()
+    if args.record_traffic:
+        record_traffic(args.record_traffic)
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
               "--gpus must be 1", file=sys.stderr)
@@ -243,7 +274,7 @@ def main():
     # instruction, on this operand distribution and on all-zero operands, and the dominant kernel on
     # all-zero operands: the gap between the two operand patterns is the device's power management,
     # not the kernel's schedule.
-    if not args.only or args.only == dom:
+    if (not args.only or args.only == dom) and not args.no_ceiling:
         ceiling = run_ceiling(rw, torch, dev, gen, [dom_dtype] if args.only else None)
         key = f"{dom_dtype}_16x16x32"
         dom_case = next(c for c in cases if c[0] == dom)
