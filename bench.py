@@ -475,6 +475,29 @@ def run_extras(rw, torch, dev, gen, only=None):
                                                "us_graph_replay": None if msg is None else round(msg * 1e3, 2),
                                                "note": "back-to-back launches, launch-latency bound"}
 
+    # A GEMM written against the public fragment API only (the reference's perf_hgemm data flow: cooperative
+    # global reads, LDS slabs, mma_sync), 8192^3 f16 -> f32.  A col-major / B row-major makes every global
+    # and LDS access a dim-major fragment access; A row / B col are K-contiguous in global memory.
+    for tag, la_, lb_ in (("cr", CM, RM), ("rc", RM, CM)):
+        key = f"public_api_gemm_f16_{tag}_8192"
+        if not wanted(key):
+            continue
+        sz = 8192
+        Ap = (torch.rand(sz * sz, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        Bp = (torch.rand(sz * sz, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        Cp = torch.rand(sz * sz, device=dev, generator=gen) * 2 - 1
+        Dp = torch.empty(sz * sz, device=dev)
+
+        def fnp():
+            rw.selftest_coop_gemm(la_, lb_, sz, sz, sz, Ap, Bp, Cp, Dp, 1.0, 1.0)
+
+        fnp()
+        ms = event_ms(fnp, 3, torch)
+        out[key] = {"ms": round(ms, 3), "tflops": round(2.0 * sz ** 3 / ms / 1e9, 1),
+                    "note": "fragment API only (load/store_matrix_coop_sync, applyDataLayout, applyTranspose, mma_sync); "
+                            "32x32x16 blocks, 128 x 128 macro tile, single LDS buffer"}
+        del Ap, Bp, Cp, Dp
+
     # config 3: N = 14336, K = 4096, M in {16, 128, 4096}; int8 and e4m3, A row / B col.  The weight
     # matrix (56 MiB) would stay in the 256 MiB Infinity Cache between launches, so the timed loop
     # rotates over 5 weight buffers (280 MiB); the cache-resident time is reported beside it.

@@ -3,8 +3,12 @@
 // A fragment is a sequence of "items": for input fragments an item is one MFMA operand
 // (kpack elements contiguous in K, see fragment_map.hpp); for accumulators an item is a run
 // of four consecutive columns of one row (a single element for 64-bit accumulators).  Items whose elements are contiguous in memory
-// (K-contiguous operands; row-major accumulators) move as one 2..32-byte vector access,
-// the others element by element.
+// (K-contiguous operands; row-major accumulators) move as one 2..32-byte vector access.
+// Input items of 16 bytes per lane whose K index is NOT the contiguous one (col-major matrix_a,
+// row-major matrix_b) also move as 16-byte vectors: every lane accesses one memory row (16 bytes along
+// the contiguous dimension, one K index) and a transpose inside groups of 8 lanes (16-bit elements) or
+// 16 lanes (8-bit elements) converts between that and the register order (see LaneTranspose).
+// Everything else moves element by element.
 //
 // The same walk serves the cooperative API.  Wave w of a pool of W waves owns the fragment's
 // register elements [w * size / W, (w + 1) * size / W) and keeps them at their ordinary
@@ -20,7 +24,8 @@
 // opaque_load.hpp:65-159, opaque_store.hpp:56-135, coop_load.hpp:43-218, coop_store.hpp:43-217.)
 //
 // Alignment contract: a vector access of B bytes needs its address aligned to min(B, 16).
-// That holds when the tile origin and the leading dimension are multiples of 16 bytes.
+// That holds when the tile origin and the leading dimension are multiples of 16 bytes (in either
+// orientation: the dim-major vector path reads 16 bytes along the contiguous dimension).
 #ifndef ROCWMMA_FRAGMENT_IO_HPP
 #define ROCWMMA_FRAGMENT_IO_HPP
 
@@ -53,6 +58,152 @@ namespace rocwmma
             }
         }
 
+
+        // ---- transposes across lanes -----------------------------------------------------
+        // Four registers (16 bytes) per lane.  transpose8x8Halves: inside every group of 8 consecutive
+        // lanes, lane r holds row r of an 8 x 8 matrix of 16-bit elements; afterwards lane c holds column c.
+        // transpose16x16Bytes: the same for 16 x 16 bytes in groups of 16 lanes.  Both are their own
+        // inverse.  Each is a butterfly: stage b swaps bit b of the lane index with bit b of the element
+        // index, i.e. a lane keeps the elements whose bit b equals its own and trades the others with lane
+        // ^ (1 << b).  Whole registers are traded with DPP row shifts whose bank mask picks the receiving
+        // half of the lanes (distances 4 and 8), or with a quad permute and selects (distance 2 inside a
+        // quad); halves and bytes of registers with a quad permute followed by v_perm_b32.
+        // (rocWMMA reaches the same end with its AOS <-> SOA register transforms, reference
+        // library/include/rocwmma/internal/transforms.hpp and io_layout.hpp:160-226.)
+        struct LaneTranspose
+        {
+            static constexpr int QuadXor1 = 0xB1; // quad_perm:[1,0,3,2]
+            static constexpr int QuadXor2 = 0x4E; // quad_perm:[2,3,0,1]
+            static constexpr int RowShl4 = 0x104, RowShr4 = 0x114, RowShl8 = 0x108, RowShr8 = 0x118;
+
+            template <int Ctrl, int BankMask>
+            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t dpp(uint32_t keep, uint32_t src)
+            {
+                return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(
+                    static_cast<int>(keep), static_cast<int>(src), Ctrl, 0xF, BankMask, false));
+            }
+
+            // registers (a, b) <-> (c, d) between lanes `Shift` apart: the lower lane of a pair ends up
+            // with the upper lane's (a, b) in its (c, d); the upper lane with the lower lane's (c, d) in
+            // its (a, b).  LowerBanks: the banks (groups of 4 lanes of a row of 16) of the lower lanes.
+            template <int Shl, int Shr, int LowerBanks>
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void
+                tradeRegisters(uint32_t& a, uint32_t& b, uint32_t& c, uint32_t& d)
+            {
+                const uint32_t nc = dpp<Shl, LowerBanks>(c, a);
+                const uint32_t nd = dpp<Shl, LowerBanks>(d, b);
+                const uint32_t na = dpp<Shr, 0xF & ~LowerBanks>(a, c);
+                const uint32_t nb = dpp<Shr, 0xF & ~LowerBanks>(b, d);
+                a = na, b = nb, c = nc, d = nd;
+            }
+
+            // value of lane `QuadPerm(lane)` for every lane (nothing kept: no tie to an old register)
+            template <int QuadPerm>
+            ROCWMMA_DEVICE static ROCWMMA_INLINE uint32_t quad(uint32_t src)
+            {
+                return static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(src), QuadPerm, 0xF, 0xF, true));
+            }
+
+            // halves or bytes of every register (which ones: the v_perm_b32 selectors of the lower and the
+            // upper lane) between the lanes of a quad that differ in `LaneBit`
+            template <int QuadPerm, uint32_t LaneBit, uint32_t LowerSel, uint32_t UpperSel>
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void tradeWithinRegisters(uint32_t (&x)[4], uint32_t lane)
+            {
+                const uint32_t sel = (lane & LaneBit) ? UpperSel : LowerSel;
+#pragma unroll
+                for(uint32_t d = 0; d < 4u; ++d)
+                {
+                    x[d] = __builtin_amdgcn_perm(quad<QuadPerm>(x[d]), x[d], sel);
+                }
+            }
+
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void transpose8x8Halves(uint32_t (&x)[4], uint32_t lane)
+            {
+                // element bit 2 = register bit 1, lane bit 2: lanes 0-3 and 8-11 of a row are the lower ones
+                tradeRegisters<RowShl4, RowShr4, 0x5>(x[0], x[1], x[2], x[3]);
+                // element bit 1 = register bit 0, lane bit 1 (inside a quad)
+                // (written so that each select can take its permuted operand as a DPP source)
+                const bool     upper = (lane & 2u) != 0u;
+                const uint32_t p0 = quad<QuadXor2>(x[0]), p1 = quad<QuadXor2>(x[1]);
+                const uint32_t p2 = quad<QuadXor2>(x[2]), p3 = quad<QuadXor2>(x[3]);
+                x[0] = upper ? p1 : x[0];
+                x[1] = upper ? x[1] : p0;
+                x[2] = upper ? p3 : x[2];
+                x[3] = upper ? x[3] : p2;
+                // element bit 0 = half of a register, lane bit 0
+                tradeWithinRegisters<QuadXor1, 1u, 0x05040100u, 0x03020706u>(x, lane);
+            }
+
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void transpose16x16Bytes(uint32_t (&x)[4], uint32_t lane)
+            {
+                tradeRegisters<RowShl8, RowShr8, 0x3>(x[0], x[1], x[2], x[3]); // byte bit 3, lane bit 3
+                tradeRegisters<RowShl4, RowShr4, 0x5>(x[0], x[2], x[1], x[3]); // byte bit 2, lane bit 2
+                tradeWithinRegisters<QuadXor2, 2u, 0x05040100u, 0x03020706u>(x, lane); // byte bit 1, lane bit 1
+                tradeWithinRegisters<QuadXor1, 1u, 0x06020400u, 0x03070105u>(x, lane); // byte bit 0, lane bit 0
+            }
+        };
+
+        // ---- LDS reads that transpose ------------------------------------------------------
+        // True when the generic pointer points into LDS (folds to a constant wherever the compiler has
+        // inferred the address space, which is the usual case after inlining).  The answer is taken from
+        // the first active lane, so a branch on it is a scalar branch: every lane of a wave passes the same
+        // tile pointer, but the compiler cannot always see that, and the transposing LDS reads must not be
+        // reached under a lane mask (they execute whatever the mask says and would overwrite the
+        // destination registers of the other branch).
+        ROCWMMA_DEVICE ROCWMMA_INLINE bool isLdsPointer(const void* p)
+        {
+#if defined(__HIP_DEVICE_COMPILE__)
+            return __builtin_amdgcn_readfirstlane(
+                       static_cast<int>(__builtin_amdgcn_is_shared((const __attribute__((address_space(0))) void*)p)))
+                   != 0;
+#else
+            (void)p;
+            return false;
+#endif
+        }
+
+        // ds_read_b64_tr_b16: inside a group of 16 lanes, lane s addresses 8 bytes (4 consecutive dims
+        // (s % 4) * 4 .. + 3 of memory row s / 4); lane t receives dim t of the 4 rows.
+        // ds_read_b64_tr_b8: lane s addresses 8 bytes (dims (s % 2) * 8 .. + 7 of memory row s / 2); lane t
+        // receives dim t of the 8 rows.  Either way one read yields 8 bytes of consecutive K for one dim
+        // out of a block of 16 consecutive dims, which is the register order of input fragments.
+        template <typename DataT>
+        struct LdsTransposedRead
+        {
+            static constexpr uint32_t RowsPerRead = 8u / sizeof(DataT); // K indices per read: 4 or 8
+            static constexpr uint32_t LanesPerRow = 16u / RowsPerRead; // 4 or 2
+
+            // `block`: first of the 16 dims at the first K index; the lane receives dim lane % 16,
+            // Reads * RowsPerRead consecutive K indices.
+            template <uint32_t Reads>
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void read(DataT* reg, const DataT* block, uint32_t ld, uint32_t lane)
+            {
+#if defined(__HIP_DEVICE_COMPILE__)
+                const uint32_t s = lane & 15u;
+                const DataT*   p = block + (s / LanesPerRow) * ld + (s % LanesPerRow) * (16u / LanesPerRow);
+#pragma unroll
+                for(uint32_t r = 0; r < Reads; ++r)
+                {
+                    const DataT* q = p + r * RowsPerRead * ld;
+                    if constexpr(sizeof(DataT) == 2u)
+                    {
+                        typedef short s16x4 __attribute__((ext_vector_type(4)));
+                        const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)q);
+                        copyBytes<8u>(reg + r * RowsPerRead, &v);
+                    }
+                    else
+                    {
+                        typedef int i32x2 __attribute__((ext_vector_type(2)));
+                        const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)q);
+                        copyBytes<8u>(reg + r * RowsPerRead, &v);
+                    }
+                }
+#else
+                (void)reg, (void)block, (void)ld, (void)lane;
+#endif
+            }
+        };
+
         // ---- input fragments -------------------------------------------------------------
         // KContiguous: memory offset of (dim, k) is dim * ld + k  (matrix_a row_major,
         // matrix_b col_major); otherwise k * ld + dim.
@@ -61,6 +212,31 @@ namespace rocwmma
         {
             static constexpr uint32_t Items     = Map::nchunks;
             static constexpr uint32_t ItemElems = Map::kpack;
+
+            // Dim-major memory, whole items of 16-byte multiples per lane on 16- or 32-wide tiles: a group
+            // of GroupLanes lanes (one K run each, consecutive dims) covers GroupLanes K indices x 16 bytes
+            // of consecutive dims, which the lanes access as one memory row each.
+            static constexpr uint32_t GroupLanes = 16u / sizeof(DataT); // 8 (16-bit), 16 (8-bit)
+            static constexpr uint32_t Vectors
+                = (!KContiguous && (sizeof(DataT) == 2u || sizeof(DataT) == 1u) && Map::tile >= 16u
+                   && (Map::kpack * sizeof(DataT)) % 16u == 0u && Map::kpack % GroupLanes == 0u)
+                      ? Map::kpack / GroupLanes
+                      : 0u;
+
+            // Loads from LDS: transposing reads of 8 bytes (items of at least 8 bytes per lane).
+            static constexpr uint32_t LdsReads
+                = (!KContiguous && (sizeof(DataT) == 2u || sizeof(DataT) == 1u) && Map::tile >= 16u
+                   && (Map::kpack * sizeof(DataT)) % 8u == 0u)
+                      ? Map::kpack * sizeof(DataT) / 8u
+                      : 0u;
+
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void transposeGroup(uint32_t (&w)[4], uint32_t lane)
+            {
+                if constexpr(sizeof(DataT) == 2u)
+                    LaneTranspose::transpose8x8Halves(w, lane);
+                else
+                    LaneTranspose::transpose16x16Bytes(w, lane);
+            }
 
             // Elements [first, first + Count) of item `item`; the whole item is <ItemElems>(.., 0u, ..).
             template <uint32_t Count>
@@ -74,9 +250,31 @@ namespace rocwmma
                     copyBytes<Count * sizeof(DataT)>(reg, data + dim * ld + k);
                 else
                 {
+                    if constexpr(Count == ItemElems && LdsReads > 0u)
+                    {
+                        if(isLdsPointer(data))
+                        {
+                            LdsTransposedRead<DataT>::template read<LdsReads>(reg, data + k * ld + (dim - (lane & 15u)), ld, lane);
+                            return;
+                        }
+                    }
+                    if constexpr(Count == ItemElems && Vectors > 0u)
+                    {
 #pragma unroll
-                    for(uint32_t j = 0; j < Count; ++j)
-                        copyBytes<sizeof(DataT)>(reg + j, data + (k + j) * ld + dim);
+                        for(uint32_t v = 0; v < Vectors; ++v)
+                        {
+                            uint32_t w[4];
+                            copyBytes<16u>(w, data + (k + v * GroupLanes + (lane % GroupLanes)) * ld + (dim - lane % GroupLanes));
+                            transposeGroup(w, lane);
+                            copyBytes<16u>(reg + v * GroupLanes, w);
+                        }
+                    }
+                    else
+                    {
+#pragma unroll
+                        for(uint32_t j = 0; j < Count; ++j)
+                            copyBytes<sizeof(DataT)>(reg + j, data + (k + j) * ld + dim);
+                    }
                 }
             }
 
@@ -91,6 +289,22 @@ namespace rocwmma
                     copyBytes<Count * sizeof(DataT)>(data + dim * ld + k, reg);
                 else
                 {
+                    // (stores to LDS stay element-wise: 2-byte LDS writes cost less than the transpose)
+                    if constexpr(Count == ItemElems && Vectors > 0u)
+                    {
+                        if(!isLdsPointer(data))
+                        {
+#pragma unroll
+                            for(uint32_t v = 0; v < Vectors; ++v)
+                            {
+                                uint32_t w[4];
+                                copyBytes<16u>(w, reg + v * GroupLanes);
+                                transposeGroup(w, lane);
+                                copyBytes<16u>(data + (k + v * GroupLanes + (lane % GroupLanes)) * ld + (dim - lane % GroupLanes), w);
+                            }
+                            return;
+                        }
+                    }
 #pragma unroll
                     for(uint32_t j = 0; j < Count; ++j)
                         copyBytes<sizeof(DataT)>(data + (k + j) * ld + dim, reg + j);
