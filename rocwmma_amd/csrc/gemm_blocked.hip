@@ -29,6 +29,88 @@ namespace rocwmma_amd
             gemmTile<Cfg>(tm, tn, 0u, k / Cfg::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
         }
 
+        // Two tilings in one launch: the first `fullTiles` workgroups run Full tiles over the columns
+        // [0, nFull), the others Half tiles (same rows, half the columns) over the columns [nFull, n).
+        // Used when the Full tiles alone would leave the last round of workgroups at most half occupied.
+        template <typename Full, typename Half>
+        __global__ void __launch_bounds__(Full::Threads) __attribute__((amdgpu_waves_per_eu(Full::WavesPerSimd, Full::WavesPerSimd)))
+        gemmBlockedSplitTailKernel(uint32_t                   m,
+                                   uint32_t                   n,
+                                   uint32_t                   k,
+                                   typename Full::InT const*  a,
+                                   typename Full::InT const*  b,
+                                   typename Full::OutT const* c,
+                                   typename Full::OutT*       d,
+                                   uint32_t                   lda,
+                                   uint32_t                   ldb,
+                                   uint32_t                   ldc,
+                                   uint32_t                   ldd,
+                                   typename Full::CompT       alpha,
+                                   typename Full::CompT       beta,
+                                   uint32_t                   nFull,
+                                   uint32_t                   fullTiles)
+        {
+            // (The half tiles go last.  Putting half of them first, so that one half of the compute units
+            // runs half a tile ahead of the other and result writes overlap main loops, was 3-4 % slower.)
+            uint32_t tm, tn;
+            if(blockIdx.x < fullTiles)
+            {
+                tileOfWorkgroup(blockIdx.x, m / Full::MacroM, nFull / Full::MacroN, tm, tn);
+                gemmTile<Full>(tm, tn, 0u, k / Full::MacroK, m, nFull, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
+            }
+            else
+            {
+                const uint32_t nHalf = n - nFull;
+                tileOfWorkgroup(blockIdx.x - fullTiles, m / Half::MacroM, nHalf / Half::MacroN, tm, tn);
+                b += static_cast<size_t>(nFull) * (Half::BKMajor ? ldb : 1u);
+                gemmTile<Half>(tm, tn, 0u, k / Half::MacroK, m, nHalf, k, a, b, c == nullptr ? c : c + nFull, d + nFull, lda, ldb,
+                               ldc, ldd, alpha, beta, StreamKPart{});
+            }
+        }
+
+        // Launches Full tiles with the last tile columns cut into Half tiles when that fills the last
+        // round: T = q * units + r tiles with 0 < r <= units / 2 would otherwise end with a round that
+        // occupies at most half of the compute units for the time of a whole tile (4096 x 14336: 896 tiles
+        // on 256 units, 3.5 rounds).  Whole tile columns are cut, as many as fit into r.
+        template <typename Full, typename Half>
+        int launchSplitTail(GemmArgs const& g, hipStream_t stream)
+        {
+            static_assert(Full::MacroM == Half::MacroM && Full::MacroN == 2u * Half::MacroN && Full::MacroK == Half::MacroK
+                              && Full::Threads == Half::Threads && Full::Stages == Half::Stages
+                              && Full::WavesPerSimd == Half::WavesPerSimd && !Full::Edges && !Half::Edges,
+                          "half tiles: same rows, half the columns, same pipeline");
+            if(g.m % Full::MacroM != 0u || g.n % Full::MacroN != 0u || g.k % Full::MacroK != 0u
+               || g.k < (Full::Stages - 1u) * Full::MacroK)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            const uint32_t tilesM = g.m / Full::MacroM, tilesN = g.n / Full::MacroN, units = computeUnits();
+            const uint32_t total = tilesM * tilesN, rest = total % units;
+            const uint32_t cutColumns = rest / tilesM;
+            if(total < units || rest == 0u || 2u * rest > units || cutColumns == 0u)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            {
+                const uint64_t spanA = static_cast<uint64_t>(g.lda) * sizeof(typename Full::InT)
+                                       * (Full::AKMajor ? Full::MacroM : Full::MacroK);
+                const uint64_t spanB = static_cast<uint64_t>(g.ldb) * sizeof(typename Full::InT)
+                                       * (Full::BKMajor ? Full::MacroN : Full::MacroK);
+                if(spanA >= 0x7FFF0000ull || spanB >= 0x7FFF0000ull)
+                    return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            }
+            auto               kernel = gemmBlockedSplitTailKernel<Full, Half>;
+            constexpr uint32_t lds    = Full::LdsBytes > Half::LdsBytes ? Full::LdsBytes : Half::LdsBytes;
+            if(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   static_cast<int>(lds))
+               != hipSuccess)
+                return ROCWMMA_AMD_LAUNCH_FAILED;
+            const uint32_t nFull     = (tilesN - cutColumns) * Full::MacroN;
+            const uint32_t fullTiles = tilesM * (tilesN - cutColumns);
+            hipLaunchKernelGGL(kernel, dim3(fullTiles + 2u * cutColumns * tilesM), dim3(Full::Threads), lds, stream, g.m, g.n,
+                               g.k, static_cast<typename Full::InT const*>(g.a), static_cast<typename Full::InT const*>(g.b),
+                               static_cast<typename Full::OutT const*>(g.c), static_cast<typename Full::OutT*>(g.d), g.lda,
+                               g.ldb, g.ldc, g.ldd, static_cast<typename Full::CompT>(g.alpha),
+                               static_cast<typename Full::CompT>(g.beta), nFull, fullTiles);
+            return launchStatus();
+        }
+
         template <typename Cfg>
         int launchCfg(GemmArgs const& g, hipStream_t stream)
         {
@@ -123,10 +205,18 @@ namespace rocwmma_amd
             // (a 256 x 256 tiling that covers less than half of the compute units loses to 128 x 128
             // tiles: 2048^3 f16 47 -> 24 us, 1024^3 30 -> 9 us, 512 x 14336 x 4096 int8 51 -> 42 us;
             // from 144 tiles on 256 units the large tile wins again)
+            // the same rows and pipeline with half the columns, for the tiles of a last round that would be
+            // at most half full (launchSplitTail)
+            using BigHalf = std::conditional_t<Edge16,
+                                               BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 4, 4, 2, 2, 16>,
+                                               BlockedConfig<InT, OutT, CompT, AK, BK, 4, 2, 2, 2, 2, 2, 32>>;
             if(g.m % Big::MacroM == 0u && g.n % Big::MacroN == 0u
                && (forceLargeTile || 2u * (g.m / Big::MacroM) * (g.n / Big::MacroN) >= computeUnits()))
             {
-                int rc = launchCfg<Big>(g, stream);
+                int rc = forceLargeTile ? ROCWMMA_AMD_UNSUPPORTED_SHAPE : launchSplitTail<Big, BigHalf>(g, stream);
+                if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                    return rc;
+                rc = launchCfg<Big>(g, stream);
                 if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
                     return rc;
             }
