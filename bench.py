@@ -35,7 +35,7 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0, "i8": 5000.0}  # dense MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
-FP8_BLOCKED_SHAPE = "fp8_32x32x64"  # the matrix instruction of the blocked kernel's 256 x 256 fp8 configuration
+FP8_BLOCKED_SHAPE = "fp8_16x16x128"  # the matrix instruction of the blocked kernel's 256 x 256 fp8 configuration (A row / B col)
 # Bytes moved through the L2s per launch come from rocprofv3 counter runs of this file (counters cannot
 # be read from inside this process): profiles/traffic.json holds the figures of the committed counter
 # summaries together with a digest of the kernel sources they were taken on, and a figure whose digest

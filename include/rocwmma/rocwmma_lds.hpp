@@ -145,10 +145,18 @@ namespace rocwmma
         // (row parity, chunk position): swz = row bits 1..3 does that for both readers (the eight
         // even rows of a 16-row group get eight different XOR masks; of the two K chunks a group
         // touches, one goes with masks {0,1,6,7} and the other, differing in bit 0, with {2,3,4,5}).
-        template <uint32_t Dim, uint32_t RowBytes = 64u>
+        //
+        // Pairs = true (128-byte rows only) is the variant for 16-wide blocks that take 32 bytes of K per
+        // lane (v_mfma_f32_16x16x128_f8f6f4): lane l reads chunks 2 (l / 16) and 2 (l / 16) + 1 of row
+        // l % 16 in two instructions.  Lane bit 4 is then chunk bit 1 and is tied to row bits 2, 3 by the
+        // parity rule above, so the XOR mask must leave chunk bit 1 free of row bit 3 or of row bit 2:
+        // swz = (row bit 3, row bit 3, row bit 1) puts each of the two reads on 16 distinct bank groups
+        // (checked by enumeration; the mask of the general variant gives two-way conflicts here).
+        template <uint32_t Dim, uint32_t RowBytes = 64u, bool Pairs = false>
         struct KMajorTile
         {
             static_assert(RowBytes == 64u || RowBytes == 128u, "stage rows of 64 or 128 bytes");
+            static_assert(!Pairs || RowBytes == 128u, "the pair reader works on 128-byte rows");
             static constexpr uint32_t rowBytes    = RowBytes;
             static constexpr uint32_t chunks      = RowBytes / 16u;
             static constexpr uint32_t rowsPerCopy = 1024u / rowBytes; // 16 or 8
@@ -159,6 +167,8 @@ namespace rocwmma
             {
                 if constexpr(RowBytes == 64u)
                     return (0x78u >> ((row >> 1) & 6u)) & 3u; // 0, 2, 3, 1 for rows 0-3, 4-7, 8-11, 12-15
+                else if constexpr(Pairs)
+                    return (((row >> 3) & 1u) * 6u) | ((row >> 1) & 1u);
                 else
                     return (row >> 1) & 7u;
             }
@@ -210,10 +220,14 @@ namespace rocwmma
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
                 readBlock16(void* regs, const char* ldsTile, uint32_t row0, uint32_t ks, uint32_t lane)
             {
-                static_assert(KPackBytes == 16u, "16-wide blocks take 16 bytes of K per lane");
-                const uint32_t row = row0 + (lane & 15u);
-                *reinterpret_cast<detail::u32x4*>(regs)
-                    = *reinterpret_cast<const detail::u32x4*>(ldsTile + offset(row, ks * 4u + (lane >> 4)));
+                static_assert(KPackBytes == 16u || (KPackBytes == 32u && Pairs),
+                              "16-wide blocks take 16 bytes of K per lane, or 32 from the pair variant");
+                constexpr uint32_t perLane = KPackBytes / 16u;
+                const uint32_t     row     = row0 + (lane & 15u);
+#pragma unroll
+                for(uint32_t j = 0; j < perLane; ++j)
+                    reinterpret_cast<detail::u32x4*>(regs)[j] = *reinterpret_cast<const detail::u32x4*>(
+                        ldsTile + offset(row, (ks * 4u + (lane >> 4)) * perLane + j));
             }
         };
 

@@ -50,8 +50,9 @@ namespace rocwmma_amd
                                    uint32_t                   nFull,
                                    uint32_t                   fullTiles)
         {
-            // (The half tiles go last.  Putting half of them first, so that one half of the compute units
-            // runs half a tile ahead of the other and result writes overlap main loops, was 3-4 % slower.)
+            // (The half tiles go last.  Running half of them first, on half of the compute units of every
+            // XCD or on XCDs 0-3, so that one half of the device writes its results while the other is in
+            // its main loop, was 3-4 % slower either way.)
             uint32_t tm, tn;
             if(blockIdx.x < fullTiles)
             {
@@ -184,8 +185,10 @@ namespace rocwmma_amd
         {
             // 256 x 256 macro tile, 8 waves of 64 x 128.  16-bit and int8 operands use 16-wide blocks
             // (16x16x32 / 16x16x64 instructions: half the accumulator traffic per flop of the
-            // 32-wide forms, which is worth 5-7 % under the power cap); fp8 uses 32x32x64.
-            static constexpr bool Edge16 = sizeof(InT) == 2u || std::is_same<InT, int8_t>::value;
+            // 32-wide forms, which is worth 5-7 % under the power cap).
+            // fp8 with both operands K-contiguous uses 16x16x128 (its fragments streamed column by column:
+            // the matrix pipes sustain 6 % more on it than on 32x32x64, the kernel gains 1.5-3 %); the other fp8 layouts use 32x32x64.
+            static constexpr bool Edge16 = sizeof(InT) == 2u || std::is_same<InT, int8_t>::value || (AK && BK);
             // Ring of two stages of 128 bytes of K: a copy instruction then requests whole 128-byte lines
             // of a K-contiguous operand (half as many requests to the L2 as with 64-byte stage rows);
             // against the ring of four 64-byte stages 8192^3 runs 1-5 % faster for f16 / bf16 in every

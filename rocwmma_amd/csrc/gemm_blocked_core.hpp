@@ -93,8 +93,10 @@ namespace rocwmma_amd
             template <uint32_t Dim>
             using DimTile = std::conditional_t<sizeof(InT) == 2u, lds::DimMajorTile<Dim, StageKB / 2u>,
                                                lds::DimMajorTile8<(Dim == 128u || Dim == 256u) ? Dim : 128u, StageKB>>;
-            using TileA = std::conditional_t<AKMajor, lds::KMajorTile<MacroM, StageKB>, DimTile<MacroM>>;
-            using TileB = std::conditional_t<BKMajor, lds::KMajorTile<MacroN, StageKB>, DimTile<MacroN>>;
+            // (16-wide blocks with 32 bytes of K per lane, fp8 16x16x128: the K-major tile's pair reader)
+            static constexpr bool PairReads = Block == 16u && KPackBytes == 32u;
+            using TileA = std::conditional_t<AKMajor, lds::KMajorTile<MacroM, StageKB, PairReads>, DimTile<MacroM>>;
+            using TileB = std::conditional_t<BKMajor, lds::KMajorTile<MacroN, StageKB, PairReads>, DimTile<MacroN>>;
 
             static constexpr uint32_t BytesA     = MacroM * StageKB;
             static constexpr uint32_t BytesB     = MacroN * StageKB;
@@ -120,7 +122,9 @@ namespace rocwmma_amd
                                             && 2u * Block * GroupBlocks * Block * sizeof(OutT) * Waves <= LdsBytes;
 
             static_assert(Block == 32u || Block == 16u, "MFMA blocks are 32 or 16 wide");
-            static_assert(Block == 32u || KPackBytes == 16u, "16-wide blocks: 16 bytes of K per lane (16-bit types, int8)");
+            static_assert(Block == 32u || KPackBytes == 16u || (PairReads && AKMajor && BKMajor && Stages_ == 2u),
+                          "16-wide blocks: 16 bytes of K per lane (16-bit types, int8), or fp8 16x16x128 on K-contiguous "
+                          "operands in the ring of two");
             static_assert(sizeof(InT) == 2u || sizeof(InT) == 1u, "16-bit and 8-bit operands");
             static_assert(sizeof(InT) == 2u || ((AKMajor || MacroM == 128u || MacroM == 256u) && (BKMajor || MacroN == 128u || MacroN == 256u)),
                           "dim-major tiles of 8-bit operands are 128 or 256 wide");
@@ -128,7 +132,8 @@ namespace rocwmma_amd
             static_assert(BytesA % (1024u * Waves) == 0u && BytesB % (1024u * Waves) == 0u,
                           "a stage must split into whole-wave copies evenly");
             static_assert((Stages - 1u) * Copies < 64u, "too many copies in flight for vmcnt");
-            static_assert(Stages != 2u || KSteps == 2u || KSteps == 4u, "the ring of two runs two or four MFMA steps per stage");
+            static_assert(Stages != 2u || KSteps == 2u || KSteps == 4u || (KSteps == 1u && BlocksN % 2u == 0u),
+                          "the ring of two runs one (fragments streamed by columns), two or four MFMA steps per stage");
             static_assert(LdsBytes <= Constants::AMDGCN_LDS_MAX_SIZE_BYTES, "macro tile does not fit the LDS");
             // the dim-major tile's swizzle looks at K row bits 0..3: a wave's copies must all start
             // on the same K row modulo 16
@@ -461,7 +466,72 @@ namespace rocwmma_amd
             constexpr uint32_t S      = Cfg::Stages;
             // `stages` stages of K from stage0 on: >= S - 1 of them (checked by the host)
 
-            if constexpr(S == 2u)
+            if constexpr(S == 2u && Cfg::KSteps == 1u)
+            {
+                // Ring of two stages, one MFMA step per stage whose fragments would not fit the register
+                // file twice (fp8 16x16x128: 8 registers per block and operand).  The A fragments of a
+                // stage are held whole (and read one stage ahead into a second set); the B fragments
+                // stream through two column buffers: while column j is multiplied, column j + 1 is read.
+                // The barrier sits in front of the last column: by then the wave has read everything it
+                // needs from stage i (the last column's fragment arrived with the wait), stage i + 1 has
+                // landed, and the copies of stage i + 2 go out into stage i's slot.
+                static_assert(Cfg::AKMajor && Cfg::BKMajor, "streamed columns: K-contiguous operands");
+                issueStage(0u, 1u < stages);
+                issueStage(1u, 2u < stages);
+                lds::waitCopiesAndReads<Cfg::Copies>(); // stage 0 has landed
+                lds::barrier();
+                typename Cfg::FragA fa[2][Cfg::BlocksM];
+                typename Cfg::FragB fb[2];
+                auto readA = [&](typename Cfg::FragA(&dst)[Cfg::BlocksM], uint32_t slot) {
+                    const char* ldsA = ldsRaw + slot * Cfg::StageBytes;
+#pragma unroll
+                    for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+                        TileA::template readBlock16<Cfg::KPackBytes>(dst[bi].x, ldsA, waveM * Cfg::WaveM + bi * Cfg::Block, 0u, lane);
+                };
+                auto readB = [&](typename Cfg::FragB& dst, uint32_t slot, uint32_t bj) {
+                    const char* ldsB = ldsRaw + slot * Cfg::StageBytes + Cfg::BytesA;
+                    TileB::template readBlock16<Cfg::KPackBytes>(dst.x, ldsB, waveN * Cfg::WaveN + bj * Cfg::Block, 0u, lane);
+                };
+                auto column = [&](typename Cfg::FragA const(&a_)[Cfg::BlocksM], typename Cfg::FragB const& b_, uint32_t bj) {
+#pragma unroll
+                    for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+                        mma_sync(acc[bi][bj], a_[bi], b_, acc[bi][bj]);
+                };
+                constexpr uint32_t RB = Cfg::KPackBytes / 16u; // LDS reads per block
+                readA(fa[0], 0u);
+                readB(fb[0], 0u, 0u);
+                // (the A sets alternate with the stage parity; two stages per trip keep the indices static)
+                auto stage = [&](typename Cfg::FragA(&cur)[Cfg::BlocksM], typename Cfg::FragA(&nxt)[Cfg::BlocksM],
+                                 uint32_t slot, uint32_t ii) {
+#pragma unroll
+                        for(uint32_t bj = 0; bj + 1u < Cfg::BlocksN; ++bj)
+                        {
+                            readB(fb[(bj + 1u) & 1u], slot, bj + 1u);
+                            column(cur, fb[bj & 1u], bj);
+                            scheduleInterleaved<Cfg::BlocksM, RB, 0u>();
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        lds::waitCopiesAndReads<0u>(); // stage ii + 1 has landed, stage ii is in registers
+                        lds::barrier();
+                        __builtin_amdgcn_sched_barrier(0);
+                        issueStage(slot, ii + 3u < stages);
+                        readA(nxt, slot ^ 1u);
+                        readB(fb[0], slot ^ 1u, 0u);
+                        column(cur, fb[(Cfg::BlocksN - 1u) & 1u], Cfg::BlocksN - 1u);
+                        __builtin_amdgcn_sched_barrier(0);
+                };
+                uint32_t i = 0;
+                for(; i + 1u < stages; i += 2u)
+                {
+                    stage(fa[0], fa[1], 0u, i);
+                    stage(fa[1], fa[0], 1u, i + 1u);
+                }
+                if(i < stages)
+                    stage(fa[0], fa[1], 0u, i);
+                lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
+                lds::barrier();
+            }
+            else if constexpr(S == 2u)
             {
                 // Ring of two stages of 128 bytes of K (two or four MFMA steps each).  A phase multiplies
                 // one step while it reads the fragments of the next; the barrier in front of a stage's
