@@ -100,8 +100,10 @@ int rocwmma_amd_device_info(int* compute_units, int* clock_mhz, int* is_gfx950);
  * c may be NULL when beta == 0.  c may equal d.
  * Shapes: m and n multiples of 16, k a multiple of 32 bytes' worth of elements per row is the
  * minimum every kernel accepts (k % 16 == 0 for 16-bit types, k % 32 == 0 for 8-bit types);
- * the blocked kernel additionally needs whole macro tiles (multiples of 64) and is chosen
- * automatically, as are the weight-streaming kernels for up to 112 rows of A against a col-major B.
+ * the blocked kernel additionally needs k in whole 64-byte stages and at least three of them, takes every
+ * type in all four A/B layout pairs (m, n that do not fill whole tiles run on partly filled edge tiles)
+ * and is chosen automatically, as are the weight-streaming kernels for up to 112 rows of A against a
+ * col-major B.
  * One of those (48, 80, 96, 112 rows, or a 16-bit A too large for the LDS) runs as two launches on the
  * stream and adds its K slices into D with atomic adds: I32 results are exact, F32 results can differ
  * in the last bit from run to run.
@@ -128,8 +130,9 @@ int rocwmma_amd_gemm(int         dtype_in,
                      void*       stream);
 
 /* Same as rocwmma_amd_gemm with the kernel family forced (`algo` is a rocwmma_amd_gemm_algo).
- * ROCWMMA_AMD_GEMM_BLOCKED / _BLOCKED_256 return ROCWMMA_AMD_UNSUPPORTED_SHAPE when the shape does not
- * fill whole macro tiles, like the reference's perf_hgemm host (samples/perf_hgemm.cpp:735-765). */
+ * ROCWMMA_AMD_GEMM_BLOCKED returns ROCWMMA_AMD_UNSUPPORTED_SHAPE when k is not in whole stages, and
+ * _BLOCKED_256 when the shape does not fill whole 256 x 256 tiles, like the reference's perf_hgemm host
+ * (samples/perf_hgemm.cpp:735-765). */
 int rocwmma_amd_gemm_ex(int         algo,
                         int         dtype_in,
                         int         dtype_out,
