@@ -23,6 +23,7 @@ layouts) or one of the extra cases by its key in the JSON line (gemm_fp8_m4096, 
 gemv_8192x8192_n8, dlrm_bwd_b262144, ...).
 """
 import argparse
+import ctypes
 import hashlib
 import json
 import os
@@ -603,6 +604,53 @@ def run_extras(rw, torch, dev, gen, only=None):
                                                         "gbs_graph_replay": round(byts / msg / 1e6, 1),
                                                         "frac_hbm_graph_replay": round(byts / msg / 1e6 / PEAK_HBM_GBS, 4)})
         del Fs
+
+    # What plain streaming kernels reach on this device for the byte counts of the bandwidth-bound cases
+    # (one read-only / copy kernel, windows rotated through 2 GiB so that every launch reads from HBM):
+    # at tens of megabytes a launch is over before the memory system reaches the rate of a long stream.
+    if only is None or only == "stream_ceiling":
+        MiB = 1 << 20
+        src = torch.ones(2048 * MiB // 4, device=dev, dtype=torch.int32)
+        dst = torch.empty(2048 * MiB // 4, device=dev, dtype=torch.int32)
+        ceil = {}
+        for tag, mode, nbytes in (("read_56MiB", rw.STREAM_READ, 56 * MiB), ("read_128MiB", rw.STREAM_READ, 128 * MiB),
+                                  ("read_1792MiB", rw.STREAM_READ, 1792 * MiB), ("copy_1792MiB", rw.STREAM_COPY, 1792 * MiB)):
+            windows = max(1, (2048 * MiB) // nbytes)
+            state = {"i": 0}
+            # (raw addresses and the stream handle prepared up front: a launch of 10 us must not wait for Python)
+            srcs = [ctypes.c_void_p(src.data_ptr() + w * nbytes) for w in range(windows)]
+            dsts = [ctypes.c_void_p(dst.data_ptr() + w * nbytes) for w in range(windows)]
+            strm = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+            def fns():
+                w = state["i"] % windows
+                rw.bench_stream(mode, srcs[w], dsts[w], nbytes, strm)
+                state["i"] += 1
+
+            def fns_current_stream():
+                w = state["i"] % windows
+                rw.bench_stream(mode, srcs[w], dsts[w], nbytes)
+                state["i"] += 1
+
+            fns()
+            ms = event_ms(fns, iters, torch)
+            # launches of 10-20 us: replayed as one HIP graph as well, and the shorter of the two counts
+            msg = graph_ms(fns_current_stream, iters, torch) if (nbytes <= 128 * MiB and only is None) else None
+            best = ms if msg is None else min(ms, msg)
+            moved = nbytes * (2 if mode == rw.STREAM_COPY else 1)
+            ceil[tag] = {"ms": round(ms, 5), "ms_graph_replay": None if msg is None else round(msg, 5),
+                         "gbs": round(moved / best / 1e6, 1), "frac_hbm": round(moved / best / 1e6 / PEAK_HBM_GBS, 4)}
+        del src, dst
+        out["stream_ceiling"] = ceil
+        # the bandwidth-bound cases against the plain stream of the nearest size and kind
+        for key, ref in (("gemm_i8_m16", "read_56MiB"), ("gemm_fp8_m16", "read_56MiB"), ("gemm_i8_m128", "read_56MiB"),
+                         ("gemm_fp8_m128", "read_56MiB"), ("gemv_8192x8192_n1", "read_128MiB"),
+                         ("gemv_8192x8192_n4", "read_128MiB"), ("gemv_8192x8192_n8", "read_128MiB"),
+                         ("gemv_14336x4096_n1", "read_128MiB"), ("gemv_14336x4096_n4", "read_128MiB"),
+                         ("gemv_14336x4096_n8", "read_128MiB"), ("dlrm_fwd_b262144", "read_1792MiB"),
+                         ("dlrm_bwd_b262144", "copy_1792MiB")):
+            if key in out:
+                out[key]["frac_of_stream_ceiling"] = round(out[key]["gbs"] / ceil[ref]["gbs"], 4)
     return out
 
 

@@ -94,6 +94,15 @@ int rocwmma_amd_bench_mfma_ceiling(int         shape,
                                    double*     ops,
                                    void*       stream);
 
+/*
+ * Memory-stream ceiling probe: one plain kernel that reads (mode 0), writes (mode 1) or copies (mode 2)
+ * `bytes` bytes (a multiple of 32 KiB) with 16-byte accesses, 16 workgroups of 256 threads per compute
+ * unit.  mode 0 reads `src` (and needs 4 writable bytes at `dst`), mode 1 writes `dst`, mode 2 copies
+ * `src` to `dst`.  The bandwidth-bound workloads are priced against what this reaches for their byte
+ * counts on the same device.  Has no counterpart in the reference.
+ */
+int rocwmma_amd_bench_stream(int mode, const void* src, void* dst, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,7 +22,8 @@ EXPORTS = [
 ]
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
 _AUX_LIB_NAME = "librocwmma_amd_aux.so"
-AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_bench_mfma_ceiling"]
+AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_bench_mfma_ceiling",
+               "rocwmma_amd_bench_stream"]
 (MFMA_F16_16X16X32, MFMA_F16_32X32X16, MFMA_BF16_16X16X32, MFMA_BF16_32X32X16, MFMA_I8_16X16X64, MFMA_I8_32X32X32,
  MFMA_F8_16X16X128, MFMA_F8_32X32X64) = range(8)
 
@@ -98,6 +99,8 @@ def aux_library():
         L.rocwmma_amd_selftest_coop_gemm.restype = i
         L.rocwmma_amd_bench_mfma_ceiling.argtypes = [i, u, u, vp, vp, ctypes.POINTER(ctypes.c_double), vp]
         L.rocwmma_amd_bench_mfma_ceiling.restype = i
+        L.rocwmma_amd_bench_stream.argtypes = [i, vp, vp, ctypes.c_size_t, vp]
+        L.rocwmma_amd_bench_stream.restype = i
         _aux = L
     return _aux
 
@@ -130,7 +133,12 @@ def _stream():
 
 
 def _ptr(t):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    """Device tensor (its data pointer), raw address (int / c_void_p) or None."""
+    if t is None or isinstance(t, ctypes.c_void_p):
+        return t
+    if isinstance(t, int):
+        return ctypes.c_void_p(t)
+    return ctypes.c_void_p(t.data_ptr())
 
 
 def gemm_raw(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, lda, b, ldb, c, ldc, d, ldd,
@@ -221,6 +229,16 @@ def selftest_coop_gemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta):
     _check(aux_library().rocwmma_amd_selftest_coop_gemm(layout_a, layout_b, m, n, k, _ptr(a), _ptr(b), _ptr(c), _ptr(d),
                                                     alpha, beta, _stream()), "selftest_coop_gemm")
     return d
+
+
+STREAM_READ, STREAM_WRITE, STREAM_COPY = 0, 1, 2
+
+
+def bench_stream(mode, src, dst, nbytes, stream=None):
+    """Launches the memory-stream ceiling probe (plain read / write / copy of nbytes bytes); src / dst are
+    device tensors or raw addresses."""
+    _check(aux_library().rocwmma_amd_bench_stream(mode, _ptr(src), _ptr(dst), nbytes,
+                                                  stream if stream is not None else _stream()), "bench_stream")
 
 
 def bench_mfma_ceiling(shape, trips, waves_per_simd, operands, out):

@@ -13,6 +13,7 @@ namespace rocwmma_amd
                          const float* c, float* d, float alpha, float beta, hipStream_t stream);
     int benchMfmaCeiling(int shape, uint32_t trips, uint32_t wavesPerSimd, const void* operands, float* out, double* ops,
                          hipStream_t stream);
+    int benchStream(int mode, const void* src, void* dst, size_t bytes, hipStream_t stream);
 
     namespace
     {
@@ -94,6 +95,15 @@ int rocwmma_amd_bench_mfma_ceiling(int         shape,
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
     return benchMfmaCeiling(shape, trips, waves_per_simd, operands, out, ops, asStream(stream));
+}
+
+int rocwmma_amd_bench_stream(int mode, const void* src, void* dst, size_t bytes, void* stream)
+{
+    if((src && !aligned16(src)) || (dst && !aligned16(dst)))
+        return ROCWMMA_AMD_BAD_ALIGNMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return benchStream(mode, src, dst, bytes, asStream(stream));
 }
 
 } // extern "C"
