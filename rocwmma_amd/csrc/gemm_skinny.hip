@@ -43,7 +43,8 @@ namespace rocwmma_amd
                                                                               uint32_t    ldc,
                                                                               uint32_t    ldd,
                                                                               CompT       alpha,
-                                                                              CompT       beta)
+                                                                              CompT       beta,
+                                                                              uint32_t    rowsPerWg)
         {
             constexpr uint32_t E       = sizeof(InT); // bytes per element
             constexpr uint32_t kSkinnyK = kSkinnyKBytes / E; // K elements per fragment step
@@ -64,9 +65,16 @@ namespace rocwmma_amd
             const uint32_t wave   = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
             const uint32_t slice  = wave % kSkinnySlices;
             const uint32_t blk    = wave / kSkinnySlices;
-            const uint32_t nBlock = blockIdx.x * kSkinnyBlocks + blk; // block of 16 weight rows
-            const bool     live   = nBlock * 16u < n;
-            const uint32_t n0     = (live ? nBlock : 0u) * 16u; // idle waves shadow block 0, store nothing
+            // A workgroup owns rowsPerWg weight rows (a multiple of 8, at most 64: the host picks the count
+            // that spreads the rows most evenly over the compute units); block `blk` covers the next 16 of
+            // them, of which the last block of a workgroup may hold only 8 (its other lanes load and store
+            // nothing) or none.
+            const uint32_t first    = blockIdx.x * rowsPerWg + blk * 16u; // first weight row of this block
+            const uint32_t wgEnd    = min(blockIdx.x * rowsPerWg + rowsPerWg, n);
+            const uint32_t liveRows = first < wgEnd ? min(16u, wgEnd - first) : 0u;
+            const bool     live     = liveRows != 0u;
+            const uint32_t n0       = live ? first : 0u; // idle waves shadow block 0, store nothing
+            const bool     rowLive  = !live || (lane & 15u) < liveRows; // this lane's weight row exists
             const uint32_t kLen   = k / kSkinnySlices;
             const uint32_t kBeg   = slice * kLen;
 
@@ -94,9 +102,12 @@ namespace rocwmma_amd
             const InT*     bPtr = b + static_cast<size_t>(n0) * ldb + kBeg;
 
             auto loadB = [&](FragB(&fb)[Ahead], uint32_t kk) {
+                if(rowLive) // (lanes of rows beyond a half-filled block keep their zeros)
+                {
 #pragma unroll
-                for(uint32_t u = 0; u < Ahead; ++u)
-                    load_matrix_sync(fb[u], bPtr + kk + u * kSkinnyK, ldb);
+                    for(uint32_t u = 0; u < Ahead; ++u)
+                        load_matrix_sync(fb[u], bPtr + kk + u * kSkinnyK, ldb);
+                }
             };
             auto multiply = [&](FragB(&fb)[Ahead], uint32_t kk) {
 #pragma unroll
@@ -122,6 +133,9 @@ namespace rocwmma_amd
 
             // the first batch of weight fragments is requested before waiting for A
             FragB fb[Ahead];
+#pragma unroll
+            for(uint32_t u = 0; u < Ahead; ++u)
+                fill_fragment(fb[u], static_cast<InT>(0));
             loadB(fb, 0u);
             lds::waitCopiesAndReads<0>();
             __syncthreads();
@@ -153,6 +167,9 @@ namespace rocwmma_amd
                 const size_t row = i * 16u;
                 const size_t col = n0;
                 FragC        fc;
+                // (accumulator layout: a lane owns output columns 4 (lane / 16) .. + 3 of the block)
+                if(4u * (lane >> 4) >= liveRows)
+                    continue;
                 if(beta != static_cast<CompT>(0))
                 {
                     load_matrix_sync(fc, c + row * ldc + col, ldc);
@@ -180,11 +197,22 @@ namespace rocwmma_amd
                                       static_cast<int>(lds))
                       != hipSuccess)
                 return ROCWMMA_AMD_LAUNCH_FAILED;
-            const uint32_t nBlocks = g.n / 16u;
-            hipLaunchKernelGGL(kernel, dim3((nBlocks + kSkinnyBlocks - 1u) / kSkinnyBlocks), dim3(64u * kSkinnyWaves), lds,
+            // Weight rows per workgroup: 64, or fewer (a multiple of 8) when that spreads the rows more evenly:
+            // the kernel is bound by what one compute unit's L1 can request, so the busiest unit sets the time
+            // (14336 rows on 256 units: 224 workgroups of 64 rows leave 32 units idle, 256 of 56 rows do not).
+            const uint32_t units = computeUnits();
+            uint32_t       rows  = 16u * kSkinnyBlocks;
+            uint32_t       best  = ((g.n + rows - 1u) / rows + units - 1u) / units * rows;
+            for(uint32_t r = 16u * kSkinnyBlocks - 8u; r >= 32u; r -= 8u)
+            {
+                const uint32_t cost = ((g.n + r - 1u) / r + units - 1u) / units * r;
+                if(cost < best)
+                    best = cost, rows = r;
+            }
+            hipLaunchKernelGGL(kernel, dim3((g.n + rows - 1u) / rows), dim3(64u * kSkinnyWaves), lds,
                                stream, g.m, g.n, g.k, static_cast<InT const*>(g.a), static_cast<InT const*>(g.b),
                                static_cast<OutT const*>(g.c), static_cast<OutT*>(g.d), g.lda, g.ldb, g.ldc, g.ldd,
-                               static_cast<CompT>(g.alpha), static_cast<CompT>(g.beta));
+                               static_cast<CompT>(g.alpha), static_cast<CompT>(g.beta), rows);
             return launchStatus();
         }
 
