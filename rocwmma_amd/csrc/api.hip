@@ -195,7 +195,7 @@ int rocwmma_amd_gemm_ex(int         algo,
     if(algo == ROCWMMA_AMD_GEMM_AUTO && m <= 128u)
     {
         // few token rows against a wide 8-bit weight matrix: the weight-streaming kernels (<= 32 rows;
-        // 48, 80, 96, 112 rows with the K slices spread over workgroups)
+        // 48 rows with the K slices spread over workgroups)
         rc = launchGemmSkinny(dtype_in, dtype_out, layout_a, layout_b, args, asStream(stream));
         if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE && rc != ROCWMMA_AMD_UNSUPPORTED_TYPE)
             return rc;

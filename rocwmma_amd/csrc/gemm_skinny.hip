@@ -1,6 +1,6 @@
 // Skinny GEMM: D = alpha * A * B + beta * C for M <= 32 token rows against an N x K weight
 // matrix (8-bit or 16-bit A row-major, B col-major, 32-bit C/D row-major), and a K-sliced variant
-// further down for more token rows (up to 112) or when A does not fit the LDS whole.
+// further down for 48 token rows or when A does not fit the LDS whole.
 //
 // At these shapes (the reference's GEMM kernels, samples/perf_hgemm.cpp:518-714, need whole
 // 128-wide macro tiles in M and would leave most of the chip idle) the job is streaming the
@@ -217,7 +217,7 @@ namespace rocwmma_amd
         }
 
 
-        // ---- 48, 80, 96, 112 token rows: K slices over workgroups ------------------------------------
+        // ---- 48 token rows (and A too large for the LDS): K slices over workgroups ------------------
         // With more than 32 token rows A no longer fits the LDS whole, and the blocked kernel needs
         // whole 128-row tiles.  Here a workgroup keeps one K slice of A (at most 128 KiB)
         // in LDS and its 8 waves stream the same K slice of 32 weight rows each, so a compute
@@ -432,9 +432,11 @@ namespace rocwmma_amd
             // (n: the kernel that initialises D counts 4-element groups in 32 bits)
             if(g.m % 16u != 0u || g.m >= kSlicedMaxM || g.n % 16u != 0u || g.n > (1u << 24) || (g.k * E) % 1024u != 0u)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-            // 64 rows against a multiple of 64 columns: the blocked kernel's 64 x 64 tiles are as fast
-            // (24 against 25 us at 64 x 14336 x 4096), in one launch and without atomic adds
-            if(g.m % 64u == 0u && g.n % 64u == 0u)
+            // From 64 rows on the blocked kernel is as fast or faster, in one launch and without atomic adds
+            // (its 64 x 64 tiles at 64 rows: 21 against 21 us; its partly filled 128 x 128 tiles at 80, 96,
+            // 112 rows of int8 against 14336 x 4096: 25.5, 25.4, 26.4 us against 26.8, 29.0, 32.3 us here);
+            // 48 rows stay (20.8 against 24.6 us).
+            if(g.m >= 64u)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             // K slices: whole 1 KiB copies per row and whole batches of fragment steps per slice, the
             // A slice within 128 KiB of LDS; as few slices as fill the compute units
@@ -459,14 +461,6 @@ namespace rocwmma_amd
                 return launchSliced<InT, OutT, CompT, 2>(g, stream, slices);
             case 3:
                 return launchSliced<InT, OutT, CompT, 3>(g, stream, slices);
-            case 4:
-                return launchSliced<InT, OutT, CompT, 4>(g, stream, slices);
-            case 5:
-                return launchSliced<InT, OutT, CompT, 5>(g, stream, slices);
-            case 6:
-                return launchSliced<InT, OutT, CompT, 6>(g, stream, slices);
-            case 7:
-                return launchSliced<InT, OutT, CompT, 7>(g, stream, slices);
             default:
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             }
