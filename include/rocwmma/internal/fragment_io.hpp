@@ -11,15 +11,18 @@
 // Everything else moves element by element.
 //
 // The same walk serves the cooperative API.  Wave w of a pool of W waves owns the fragment's
-// register elements [w * size / W, (w + 1) * size / W) and keeps them at their ordinary
-// positions; the rest of its fragment is untouched.  With Items % W == 0 that is a run of whole
-// items; with more waves than items (W % Items == 0) an item is cut into W / Items equal
-// pieces.  Because the share is a range of register elements, a cooperative fragment may be
-// reinterpreted as another fragment type with the same element count (an LDS "register file"
-// view, say) and stored cooperatively with the same (w, W): every wave then writes what it
-// read, whatever the item sizes of the two types.  Other wave counts (3 waves, 4 items) fall
-// back to ceil(Items / W) whole items per wave, which agrees only between types with equal
-// item sizes.
+// elements [w * size / W, (w + 1) * size / W) (a blocked, not a strided, assignment) and keeps them in
+// its FIRST size / W register elements; the rest of its fragment is untouched.  With Items % W == 0 that
+// is a run of whole items; with more waves than items (W % Items == 0) an item is cut into W / Items
+// equal pieces.  Because a share is "the first size / W register elements <-> the w-th size / W-th of the
+// fragment", a cooperative fragment may be reinterpreted as another fragment type with the same element
+// count (an LDS "register file" view, say) and stored cooperatively with the same (w, W): every wave then
+// writes what it read, whatever the item sizes of the two types.  Other wave counts (3 waves, 4 items)
+// fall back to ceil(Items / W) whole items per wave, which agrees only between types with equal item
+// sizes.  Keeping a share at the front of the registers keeps every register index a compile-time
+// constant without any branch on the wave index (with shares at their ordinary positions, behind
+// "if (w == i)" branches, the reference's perf_hgemm sample ran three times slower: the compiler merged
+// the branches into one body with a computed register index and the fragments went to scratch memory).
 // (rocWMMA's engines for the same job: reference library/include/rocwmma/internal/
 // opaque_load.hpp:65-159, opaque_store.hpp:56-135, coop_load.hpp:43-218, coop_store.hpp:43-217.)
 //
@@ -217,15 +220,21 @@ namespace rocwmma
             // of GroupLanes lanes (one K run each, consecutive dims) covers GroupLanes K indices x 16 bytes
             // of consecutive dims, which the lanes access as one memory row each.
             static constexpr uint32_t GroupLanes = 16u / sizeof(DataT); // 8 (16-bit), 16 (8-bit)
+#ifndef ROCWMMA_AMD_DIM_MAJOR_VECTORS
+#define ROCWMMA_AMD_DIM_MAJOR_VECTORS 1
+#endif
+#ifndef ROCWMMA_AMD_DIM_MAJOR_LDS_TR
+#define ROCWMMA_AMD_DIM_MAJOR_LDS_TR 1
+#endif
             static constexpr uint32_t Vectors
-                = (!KContiguous && (sizeof(DataT) == 2u || sizeof(DataT) == 1u) && Map::tile >= 16u
+                = (ROCWMMA_AMD_DIM_MAJOR_VECTORS && !KContiguous && (sizeof(DataT) == 2u || sizeof(DataT) == 1u) && Map::tile >= 16u
                    && (Map::kpack * sizeof(DataT)) % 16u == 0u && Map::kpack % GroupLanes == 0u)
                       ? Map::kpack / GroupLanes
                       : 0u;
 
             // Loads from LDS: transposing reads of 8 bytes (items of at least 8 bytes per lane).
             static constexpr uint32_t LdsReads
-                = (!KContiguous && (sizeof(DataT) == 2u || sizeof(DataT) == 1u) && Map::tile >= 16u
+                = (ROCWMMA_AMD_DIM_MAJOR_LDS_TR && !KContiguous && (sizeof(DataT) == 2u || sizeof(DataT) == 1u) && Map::tile >= 16u
                    && (Map::kpack * sizeof(DataT)) % 8u == 0u)
                       ? Map::kpack * sizeof(DataT) / 8u
                       : 0u;
@@ -241,11 +250,10 @@ namespace rocwmma
             // Elements [first, first + Count) of item `item`; the whole item is <ItemElems>(.., 0u, ..).
             template <uint32_t Count>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
-                loadPart(DataT* x, uint32_t item, uint32_t first, const DataT* data, uint32_t ld, uint32_t lane)
+                loadPart(DataT* reg, uint32_t item, uint32_t first, const DataT* data, uint32_t ld, uint32_t lane)
             {
                 const uint32_t dim = Map::chunkDim(item, lane);
                 const uint32_t k   = Map::chunkK(item, lane) + first;
-                DataT*         reg = x + item * ItemElems + first;
                 if constexpr(KContiguous)
                     copyBytes<Count * sizeof(DataT)>(reg, data + dim * ld + k);
                 else
@@ -280,11 +288,10 @@ namespace rocwmma
 
             template <uint32_t Count>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
-                storePart(const DataT* x, uint32_t item, uint32_t first, DataT* data, uint32_t ld, uint32_t lane)
+                storePart(const DataT* reg, uint32_t item, uint32_t first, DataT* data, uint32_t ld, uint32_t lane)
             {
                 const uint32_t dim = Map::chunkDim(item, lane);
                 const uint32_t k   = Map::chunkK(item, lane) + first;
-                const DataT*   reg = x + item * ItemElems + first;
                 if constexpr(KContiguous)
                     copyBytes<Count * sizeof(DataT)>(data + dim * ld + k, reg);
                 else
@@ -292,7 +299,10 @@ namespace rocwmma
                     // (stores to LDS stay element-wise: 2-byte LDS writes cost less than the transpose)
                     if constexpr(Count == ItemElems && Vectors > 0u)
                     {
-                        if(!isLdsPointer(data))
+#ifndef ROCWMMA_AMD_DIM_MAJOR_LDS_VECTOR_STORES
+#define ROCWMMA_AMD_DIM_MAJOR_LDS_VECTOR_STORES 0
+#endif
+                        if(ROCWMMA_AMD_DIM_MAJOR_LDS_VECTOR_STORES || !isLdsPointer(data))
                         {
 #pragma unroll
                             for(uint32_t v = 0; v < Vectors; ++v)
@@ -321,11 +331,10 @@ namespace rocwmma
 
             template <uint32_t Count>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
-                loadPart(DataT* x, uint32_t item, uint32_t first, const DataT* data, uint32_t ld, uint32_t lane)
+                loadPart(DataT* reg, uint32_t item, uint32_t first, const DataT* data, uint32_t ld, uint32_t lane)
             {
                 const uint32_t row = Map::runRow(item, lane);
                 const uint32_t col = Map::runCol(item, lane) + first;
-                DataT*         reg = x + item * ItemElems + first;
                 if constexpr(RowMajor)
                     copyBytes<Count * sizeof(DataT)>(reg, data + row * ld + col);
                 else
@@ -338,11 +347,10 @@ namespace rocwmma
 
             template <uint32_t Count>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
-                storePart(const DataT* x, uint32_t item, uint32_t first, DataT* data, uint32_t ld, uint32_t lane)
+                storePart(const DataT* reg, uint32_t item, uint32_t first, DataT* data, uint32_t ld, uint32_t lane)
             {
                 const uint32_t row = Map::runRow(item, lane);
                 const uint32_t col = Map::runCol(item, lane) + first;
-                const DataT*   reg = x + item * ItemElems + first;
                 if constexpr(RowMajor)
                     copyBytes<Count * sizeof(DataT)>(data + row * ld + col, reg);
                 else
@@ -355,8 +363,10 @@ namespace rocwmma
         };
 
         // ---- whole-fragment and cooperative drivers --------------------------------------
-        // `move(item, first, Count)` callbacks below receive a compile-time item and piece so that
-        // register indices stay static; which of them run is decided by (waveIndex, waveCount).
+        // Register positions are compile-time constants everywhere; a wave's index only enters address
+        // arithmetic (which item, which piece), never a register index and never a branch around code that
+        // differs in nothing but its registers (the compiler merges such branches into one body with a
+        // computed register index, and the fragment then lives in scratch memory).
         template <typename IO, typename DataT>
         struct FragmentMover
         {
@@ -364,14 +374,15 @@ namespace rocwmma
             static constexpr uint32_t ItemElems = IO::ItemElems;
             static constexpr uint32_t MaxWaves  = 16u; // 1024 threads per workgroup
 
+            // `reg`: where the part's first element lives in registers
             template <bool Load, uint32_t Count, typename Ptr, typename Reg>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
-                part(Reg* x, uint32_t item, uint32_t first, Ptr* data, uint32_t ld, uint32_t lane)
+                part(Reg* reg, uint32_t item, uint32_t first, Ptr* data, uint32_t ld, uint32_t lane)
             {
                 if constexpr(Load)
-                    IO::template loadPart<Count>(x, item, first, data, ld, lane);
+                    IO::template loadPart<Count>(reg, item, first, data, ld, lane);
                 else
-                    IO::template storePart<Count>(x, item, first, data, ld, lane);
+                    IO::template storePart<Count>(reg, item, first, data, ld, lane);
             }
 
             template <bool Load, typename Ptr, typename Reg>
@@ -380,7 +391,7 @@ namespace rocwmma
                 const uint32_t lane = threadIdx.x & (kWaveSize - 1u);
 #pragma unroll
                 for(uint32_t item = 0; item < Items; ++item)
-                    part<Load, ItemElems>(x, item, 0u, data, ld, lane);
+                    part<Load, ItemElems>(x + item * ItemElems, item, 0u, data, ld, lane);
             }
 
             // Wave count known at compile time.
@@ -390,26 +401,27 @@ namespace rocwmma
                 const uint32_t lane = threadIdx.x & (kWaveSize - 1u);
                 if constexpr(WaveCount > Items && WaveCount % Items == 0u && ItemElems % (WaveCount / Items) == 0u)
                 {
+                    // one piece of one item per wave, in its first registers
                     constexpr uint32_t pieces = WaveCount / Items, count = ItemElems / pieces;
-#pragma unroll
-                    for(uint32_t item = 0; item < Items; ++item)
-#pragma unroll
-                        for(uint32_t piece = 0; piece < pieces; ++piece)
-                            if(waveIndex == item * pieces + piece)
-                                part<Load, count>(x, item, piece * count, data, ld, lane);
+                    if(waveIndex < WaveCount)
+                        part<Load, count>(x, waveIndex / pieces, (waveIndex % pieces) * count, data, ld, lane);
                 }
                 else
                 {
+                    // items [w * per, (w + 1) * per) in register slots 0 .. per - 1
                     constexpr uint32_t per = (Items + WaveCount - 1u) / WaveCount;
 #pragma unroll
-                    for(uint32_t item = 0; item < Items; ++item)
-                        if(waveIndex == item / per)
-                            part<Load, ItemElems>(x, item, 0u, data, ld, lane);
+                    for(uint32_t s = 0; s < per; ++s)
+                    {
+                        const uint32_t item = waveIndex * per + s;
+                        if(Items % WaveCount == 0u ? waveIndex < WaveCount : item < Items)
+                            part<Load, ItemElems>(x + s * ItemElems, item, 0u, data, ld, lane);
+                    }
                 }
             }
 
-            // Pieces of `Count` elements, for a wave count only known at run time: tried for every
-            // piece size an item can be cut into with at most MaxWaves waves.
+            // One piece of `Count` elements per wave, for a wave count only known at run time: tried for
+            // every piece size an item can be cut into with at most MaxWaves waves.
             template <bool Load, uint32_t Count, typename Ptr, typename Reg>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
                 pieces(Reg* x, Ptr* data, uint32_t ld, uint32_t lane, uint32_t waveIndex, uint32_t count)
@@ -419,12 +431,8 @@ namespace rocwmma
                     constexpr uint32_t perItem = ItemElems / Count;
                     if(count == Count)
                     {
-#pragma unroll
-                        for(uint32_t item = 0; item < Items; ++item)
-#pragma unroll
-                            for(uint32_t piece = 0; piece < perItem; ++piece)
-                                if(waveIndex == item * perItem + piece)
-                                    part<Load, Count>(x, item, piece * Count, data, ld, lane);
+                        if(waveIndex < Items * perItem)
+                            part<Load, Count>(x, waveIndex / perItem, (waveIndex % perItem) * Count, data, ld, lane);
                     }
                     else
                         pieces<Load, Count / 2u>(x, data, ld, lane, waveIndex, count);
@@ -440,12 +448,14 @@ namespace rocwmma
                     pieces<Load, ItemElems / 2u>(x, data, ld, lane, waveIndex, ItemElems / (waveCount / Items));
                 else
                 {
-                    const uint32_t per   = (Items + waveCount - 1u) / waveCount;
-                    const uint32_t begin = waveIndex * per;
+                    const uint32_t per = (Items + waveCount - 1u) / waveCount;
 #pragma unroll
-                    for(uint32_t item = 0; item < Items; ++item)
-                        if(item >= begin && item - begin < per)
-                            part<Load, ItemElems>(x, item, 0u, data, ld, lane);
+                    for(uint32_t s = 0; s < Items; ++s)
+                    {
+                        const uint32_t item = waveIndex * per + s;
+                        if(s < per && item < Items)
+                            part<Load, ItemElems>(x + s * ItemElems, item, 0u, data, ld, lane);
+                    }
                 }
             }
 
