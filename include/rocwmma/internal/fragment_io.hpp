@@ -8,6 +8,7 @@
 // row-major matrix_b) also move as 16-byte vectors: every lane accesses one memory row (16 bytes along
 // the contiguous dimension, one K index) and a transpose inside groups of 8 lanes (16-bit elements) or
 // 16 lanes (8-bit elements) converts between that and the register order (see LaneTranspose).
+// Column-major accumulator runs move as one vector after a 4 x 4 transpose inside quads of lanes.
 // Everything else moves element by element.
 //
 // The same walk serves the cooperative API.  Wave w of a pool of W waves owns the fragment's
@@ -135,6 +136,41 @@ namespace rocwmma
                 x[3] = upper ? x[3] : p2;
                 // element bit 0 = half of a register, lane bit 0
                 tradeWithinRegisters<QuadXor1, 1u, 0x05040100u, 0x03020706u>(x, lane);
+            }
+
+            // 4 x 4 transposes inside quads of lanes (lane q holds row q; afterwards column q), for elements
+            // of 4, 2 and 1 bytes: 4, 2 and 1 registers per lane.
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void transpose4x4(uint32_t (&x)[4], uint32_t lane)
+            {
+                bool           upper = (lane & 2u) != 0u;
+                const uint32_t p0 = quad<QuadXor2>(x[0]), p1 = quad<QuadXor2>(x[1]);
+                const uint32_t p2 = quad<QuadXor2>(x[2]), p3 = quad<QuadXor2>(x[3]);
+                x[0] = upper ? p2 : x[0];
+                x[1] = upper ? p3 : x[1];
+                x[2] = upper ? x[2] : p0;
+                x[3] = upper ? x[3] : p1;
+                upper = (lane & 1u) != 0u;
+                const uint32_t q0 = quad<QuadXor1>(x[0]), q1 = quad<QuadXor1>(x[1]);
+                const uint32_t q2 = quad<QuadXor1>(x[2]), q3 = quad<QuadXor1>(x[3]);
+                x[0] = upper ? q1 : x[0];
+                x[1] = upper ? x[1] : q0;
+                x[2] = upper ? q3 : x[2];
+                x[3] = upper ? x[3] : q2;
+            }
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void transpose4x4(uint32_t (&x)[2], uint32_t lane)
+            {
+                const bool     upper = (lane & 2u) != 0u;
+                const uint32_t p0 = quad<QuadXor2>(x[0]), p1 = quad<QuadXor2>(x[1]);
+                x[0] = upper ? p1 : x[0];
+                x[1] = upper ? x[1] : p0;
+                const uint32_t sel = (lane & 1u) ? 0x03020706u : 0x05040100u;
+                x[0] = __builtin_amdgcn_perm(quad<QuadXor1>(x[0]), x[0], sel);
+                x[1] = __builtin_amdgcn_perm(quad<QuadXor1>(x[1]), x[1], sel);
+            }
+            ROCWMMA_DEVICE static ROCWMMA_INLINE void transpose4x4(uint32_t (&x)[1], uint32_t lane)
+            {
+                x[0] = __builtin_amdgcn_perm(quad<QuadXor2>(x[0]), x[0], (lane & 2u) ? 0x03020706u : 0x05040100u);
+                x[0] = __builtin_amdgcn_perm(quad<QuadXor1>(x[0]), x[0], (lane & 1u) ? 0x03070105u : 0x06020400u);
             }
 
             ROCWMMA_DEVICE static ROCWMMA_INLINE void transpose16x16Bytes(uint32_t (&x)[4], uint32_t lane)
@@ -329,6 +365,16 @@ namespace rocwmma
             static constexpr uint32_t Items     = Map::nruns;
             static constexpr uint32_t ItemElems = Map::runLen; // 4 (1 for 64-bit accumulators)
 
+            // Column-major memory: the four lanes of a quad own the same four columns of four consecutive
+            // rows, so a 4 x 4 transpose inside the quad turns "four columns of my row" into "four rows of one
+            // column", which is contiguous: one 16 / 8 / 4-byte access instead of four element accesses.
+#ifndef ROCWMMA_AMD_COL_MAJOR_ACC_VECTORS
+#define ROCWMMA_AMD_COL_MAJOR_ACC_VECTORS 1
+#endif
+            static constexpr bool     QuadVectors = ROCWMMA_AMD_COL_MAJOR_ACC_VECTORS && !RowMajor && ItemElems == 4u
+                                                && (sizeof(DataT) == 4u || sizeof(DataT) == 2u || sizeof(DataT) == 1u);
+            static constexpr uint32_t QuadWords = QuadVectors ? sizeof(DataT) : 1u; // registers per run
+
             template <uint32_t Count>
             ROCWMMA_DEVICE static ROCWMMA_INLINE void
                 loadPart(DataT* reg, uint32_t item, uint32_t first, const DataT* data, uint32_t ld, uint32_t lane)
@@ -337,6 +383,13 @@ namespace rocwmma
                 const uint32_t col = Map::runCol(item, lane) + first;
                 if constexpr(RowMajor)
                     copyBytes<Count * sizeof(DataT)>(reg, data + row * ld + col);
+                else if constexpr(QuadVectors && Count == ItemElems)
+                {
+                    uint32_t w[QuadWords];
+                    copyBytes<4u * sizeof(DataT)>(w, data + (col + (lane & 3u)) * ld + (row - (lane & 3u)));
+                    LaneTranspose::transpose4x4(w, lane);
+                    copyBytes<4u * sizeof(DataT)>(reg, w);
+                }
                 else
                 {
 #pragma unroll
@@ -353,6 +406,13 @@ namespace rocwmma
                 const uint32_t col = Map::runCol(item, lane) + first;
                 if constexpr(RowMajor)
                     copyBytes<Count * sizeof(DataT)>(data + row * ld + col, reg);
+                else if constexpr(QuadVectors && Count == ItemElems)
+                {
+                    uint32_t w[QuadWords];
+                    copyBytes<4u * sizeof(DataT)>(w, reg);
+                    LaneTranspose::transpose4x4(w, lane);
+                    copyBytes<4u * sizeof(DataT)>(data + (col + (lane & 3u)) * ld + (row - (lane & 3u)), w);
+                }
                 else
                 {
 #pragma unroll
