@@ -29,8 +29,8 @@ namespace rocwmma_amd
             gemmTile<Cfg>(tm, tn, 0u, k / Cfg::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
         }
 
-        // Two tilings in one launch: the first `fullTiles` workgroups run Full tiles over the columns
-        // [0, nFull), the others Half tiles (same rows, half the columns) over the columns [nFull, n).
+        // Two tilings in one launch: the first `fullTiles` workgroups run Full tiles, the others the two
+        // halves (same rows, half the columns each) of the remaining Full tiles, in the same tile order.
         // Used when the Full tiles alone would leave the last round of workgroups at most half occupied.
         template <typename Full, typename Half>
         __global__ void __launch_bounds__(Full::Threads) __attribute__((amdgpu_waves_per_eu(Full::WavesPerSimd, Full::WavesPerSimd)))
@@ -47,32 +47,31 @@ namespace rocwmma_amd
                                    uint32_t                   ldd,
                                    typename Full::CompT       alpha,
                                    typename Full::CompT       beta,
-                                   uint32_t                   nFull,
                                    uint32_t                   fullTiles)
         {
             // (The half tiles go last.  Running half of them first, on half of the compute units of every
             // XCD or on XCDs 0-3, so that one half of the device writes its results while the other is in
             // its main loop, was 3-4 % slower either way.)
-            uint32_t tm, tn;
+            const uint32_t tilesM = m / Full::MacroM, tilesN = n / Full::MacroN;
+            uint32_t       tm, tn;
             if(blockIdx.x < fullTiles)
             {
-                tileOfWorkgroup(blockIdx.x, m / Full::MacroM, nFull / Full::MacroN, tm, tn);
-                gemmTile<Full>(tm, tn, 0u, k / Full::MacroK, m, nFull, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
+                tileOfWorkgroup(blockIdx.x, tilesM, tilesN, tm, tn);
+                gemmTile<Full>(tm, tn, 0u, k / Full::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
             }
             else
             {
-                const uint32_t nHalf = n - nFull;
-                tileOfWorkgroup(blockIdx.x - fullTiles, m / Half::MacroM, nHalf / Half::MacroN, tm, tn);
-                b += static_cast<size_t>(nFull) * (Half::BKMajor ? ldb : 1u);
-                gemmTile<Half>(tm, tn, 0u, k / Half::MacroK, m, nHalf, k, a, b, c == nullptr ? c : c + nFull, d + nFull, lda, ldb,
-                               ldc, ldd, alpha, beta, StreamKPart{});
+                const uint32_t j = blockIdx.x - fullTiles;
+                tileOfWorkgroup(fullTiles + j / 2u, tilesM, tilesN, tm, tn);
+                gemmTile<Half>(tm, 2u * tn + (j & 1u), 0u, k / Half::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha,
+                               beta, StreamKPart{});
             }
         }
 
-        // Launches Full tiles with the last tile columns cut into Half tiles when that fills the last
-        // round: T = q * units + r tiles with 0 < r <= units / 2 would otherwise end with a round that
-        // occupies at most half of the compute units for the time of a whole tile (4096 x 14336: 896 tiles
-        // on 256 units, 3.5 rounds).  Whole tile columns are cut, as many as fit into r.
+        // Launches Full tiles with the tiles of the last round cut into Half tiles when that round would be
+        // at most half full: T = q * units + r tiles with 0 < r <= units / 2 would otherwise end with a round
+        // that occupies at most half of the compute units for the time of a whole tile (4096 x 14336: 896
+        // tiles on 256 units, 3.5 rounds; 6144^3: 2.25 rounds).
         template <typename Full, typename Half>
         int launchSplitTail(GemmArgs const& g, hipStream_t stream)
         {
@@ -85,8 +84,7 @@ namespace rocwmma_amd
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             const uint32_t tilesM = g.m / Full::MacroM, tilesN = g.n / Full::MacroN, units = computeUnits();
             const uint32_t total = tilesM * tilesN, rest = total % units;
-            const uint32_t cutColumns = rest / tilesM;
-            if(total < units || rest == 0u || 2u * rest > units || cutColumns == 0u)
+            if(total < units || rest == 0u || 2u * rest > units)
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             {
                 const uint64_t spanA = static_cast<uint64_t>(g.lda) * sizeof(typename Full::InT)
@@ -102,13 +100,12 @@ namespace rocwmma_amd
                                    static_cast<int>(lds))
                != hipSuccess)
                 return ROCWMMA_AMD_LAUNCH_FAILED;
-            const uint32_t nFull     = (tilesN - cutColumns) * Full::MacroN;
-            const uint32_t fullTiles = tilesM * (tilesN - cutColumns);
-            hipLaunchKernelGGL(kernel, dim3(fullTiles + 2u * cutColumns * tilesM), dim3(Full::Threads), lds, stream, g.m, g.n,
-                               g.k, static_cast<typename Full::InT const*>(g.a), static_cast<typename Full::InT const*>(g.b),
+            const uint32_t fullTiles = total - rest;
+            hipLaunchKernelGGL(kernel, dim3(fullTiles + 2u * rest), dim3(Full::Threads), lds, stream, g.m, g.n, g.k,
+                               static_cast<typename Full::InT const*>(g.a), static_cast<typename Full::InT const*>(g.b),
                                static_cast<typename Full::OutT const*>(g.c), static_cast<typename Full::OutT*>(g.d), g.lda,
                                g.ldb, g.ldc, g.ldd, static_cast<typename Full::CompT>(g.alpha),
-                               static_cast<typename Full::CompT>(g.beta), nFull, fullTiles);
+                               static_cast<typename Full::CompT>(g.beta), fullTiles);
             return launchStatus();
         }
 

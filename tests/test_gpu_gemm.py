@@ -412,14 +412,14 @@ def test_blocked_kernel_more_workgroups_than_compute_units(dtype_in, m, n, k, la
 
 @pytest.mark.parametrize("la,lb,lc", [(RM, CM, RM), (CM, RM, RM), (RM, RM, CM), (CM, CM, CM)])
 @pytest.mark.parametrize("dtype_in,dtype_out,m,n,k", [
-    (orc.F16, orc.F32, 2560, 8192, 256),   # 10 x 32 tiles = 256 + 64: six tile columns cut into halves, four whole tiles left
-    (orc.I8, orc.I32, 4096, 5120, 384),    # 16 x 20 = 256 + 64: four tile columns cut
+    (orc.F16, orc.F32, 2560, 8192, 256),   # 10 x 32 tiles = 256 + 64: the last 64 tiles run as 128 half tiles
+    (orc.I8, orc.I32, 4096, 5120, 384),    # 16 x 20 = 256 + 64
     (orc.E4M3, orc.F32, 4096, 5120, 256),
     (orc.BF16, orc.BF16, 5120, 4096, 256),  # (column-major C: the transposed problem is the one that is cut)
 ])
 def test_blocked_kernel_last_round_cut_into_half_tiles(dtype_in, dtype_out, m, n, k, la, lb, lc):
-    """256 x 256 tiles whose count leaves a last round of at most half of the compute units: the last
-    tile columns run as 256 x 128 tiles in the same launch (on a 256-unit device).  alpha, beta != 0 and every
+    """256 x 256 tiles whose count leaves a last round of at most half of the compute units: the tiles of
+    that round run as 256 x 128 tiles in the same launch (on a 256-unit device).  alpha, beta != 0 and every
     37th row checked over all columns: a half tile that lands on the wrong columns shows."""
     a = uniform_bits(61, dtype_in, m * k) if dtype_in in (orc.I8, orc.F16, orc.BF16) else normal_fp8_bits(61, dtype_in, m * k)
     b = uniform_bits(62, dtype_in, k * n) if dtype_in in (orc.I8, orc.F16, orc.BF16) else normal_fp8_bits(62, dtype_in, k * n)
