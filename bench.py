@@ -362,7 +362,8 @@ def run_ceiling(rw, torch, dev, gen, dtypes=None):
     }
     shapes = [("f16_16x16x32", rw.MFMA_F16_16X16X32, "f16", 20000), ("f16_32x32x16", rw.MFMA_F16_32X32X16, "f16", 7000),
               ("bf16_16x16x32", rw.MFMA_BF16_16X16X32, "bf16", 20000), ("i8_16x16x64", rw.MFMA_I8_16X16X64, "i8", 20000),
-              ("fp8_32x32x64", rw.MFMA_F8_32X32X64, "fp8", 5000), ("fp8_16x16x128", rw.MFMA_F8_16X16X128, "fp8", 10000)]
+              ("fp8_32x32x64", rw.MFMA_F8_32X32X64, "fp8", 5000), ("fp8_16x16x128", rw.MFMA_F8_16X16X128, "fp8", 10000),
+              ("fp8_16x16x128_scaled", rw.MFMA_F8_16X16X128_SCALED, "fp8", 10000)]
     sink = torch.empty(info_lanes(rw), device=dev)
     out = {}
     for name, shape, kind, trips in shapes:
@@ -542,6 +543,28 @@ def run_extras(rw, torch, dev, gen, only=None):
                 "ms_weights_cache_resident": round(ms_res, 4),
             }
         del Bq, Bf
+
+    # config 3's fp8 shape with block scales (one E8M0 byte per 32 elements of K): the same blocked kernel
+    # on the scaled matrix instruction, plus the small kernels that re-order the scales
+    if wanted("gemm_mxfp8_m4096"):
+        m = 4096
+        Am = (torch.randn(m * k, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+        Bm = (torch.randn(k * n, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+        SAm = torch.randint(124, 131, (m * (k // 32),), device=dev, dtype=torch.uint8, generator=gen)
+        SBm = torch.randint(124, 131, (n * (k // 32),), device=dev, dtype=torch.uint8, generator=gen)
+        Dm = torch.empty(m * n, device=dev, dtype=torch.float32)
+        ws = torch.empty(rw.gemm_mx_workspace_size(m, n, k), device=dev, dtype=torch.uint8)
+
+        def fnm():
+            rw.gemm_mx(rw.E4M3, RM, CM, RM, m, n, k, Am, SAm, Bm, SBm, None, Dm, 1.0, 0.0, workspace=ws)
+
+        fnm()
+        ms = event_ms(fnm, iters, torch)
+        flops = 2.0 * m * n * k
+        out["gemm_mxfp8_m4096"] = {"ms": round(ms, 4), "tops": round(flops / ms / 1e9, 1),
+                                   "frac_mfma": round(flops / ms / 1e9 / PEAK_TFLOPS["fp8"], 4),
+                                   "note": "E4M3 operands, E8M0 scales per 32 elements of K, scale re-ordering included"}
+        del Am, Bm, SAm, SBm, Dm, ws
 
     # config 4: GEMV, buffers rotated over > 512 MB so the 256 MB Infinity Cache cannot serve A
     for (m, kk) in ((8192, 8192), (14336, 4096)):

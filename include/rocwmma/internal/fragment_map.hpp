@@ -22,8 +22,9 @@
 //      element e = (db * nk + ks) * kpack + j   holds
 //        dim = db * tile + lane % tile
 //        k   = ks * kstep + (lane / tile) * kpack + j
-//    which is exactly the operand layout of v_mfma_*_16x16x{16,32,64,128} /
-//    v_mfma_*_32x32x{8,16,32,64}: one lane = one row (column) and a contiguous run of K.
+//    which is exactly the operand layout of v_mfma_*_16x16x{16,32,64} / v_mfma_*_32x32x{8,16,32}:
+//    one lane = one row (column) and a contiguous run of K.  The fp8 wide-K instructions
+//    (16x16x128 / 32x32x64) take two consecutive K steps of 16-byte runs in one go (mmaSteps = 2).
 //
 //  * Accumulators are held TRANSPOSED with respect to the MFMA result (mma_sync swaps the
 //    two multiplicands), so that a lane owns runs of 4 consecutive columns of one row:
@@ -80,7 +81,7 @@ namespace rocwmma
             case PackClass::Bits16:
                 return 8u; // v_mfma_f32_16x16x32_f16 / 32x32x16: 8 halves per lane
             case PackClass::Fp8:
-                return 32u; // v_mfma_f32_16x16x128_f8f6f4 / 32x32x64: 32 bytes per lane
+                return 32u; // v_mfma_f32_16x16x128_f8f6f4 / 32x32x64: 32 bytes per lane (two runs of 16)
             case PackClass::Int8:
                 return 16u; // v_mfma_i32_16x16x64_i8 / 32x32x32: 16 bytes per lane
             default:
@@ -88,17 +89,24 @@ namespace rocwmma
             }
         }
 
-        // A K run of 16 bytes of fp8 has no instruction (128/64-wide use 32, 32/16-wide use 8).
-        constexpr bool kPackAllowed(PackClass c, uint32_t p)
+        // fp8: the wide-K instructions take their 32 bytes per lane as two runs of 16 bytes of K, one
+        // from each half of the instruction's K range (lane group g holds k = 16 g + 0..15 and
+        // k = 16 groups + 16 g + 0..15: the first four registers are the operand of one 16x16x64-shaped
+        // half, the last four of the other; the block scales of the scaled forms go by this order).  So
+        // the run is 16 bytes long, and it exists only where the K steps pair up into whole instructions;
+        // elsewhere fp8 uses the 8-byte runs of the 16x16x32 / 32x32x16 instructions.
+        constexpr bool kPackAllowed(PackClass c, uint32_t p, uint32_t groups, uint32_t blockK)
         {
-            return !(c == PackClass::Fp8 && p == 16u);
+            if(c != PackClass::Fp8)
+                return true;
+            return p <= 8u || (p == 16u && blockK % (32u * groups) == 0u);
         }
 
         constexpr uint32_t chooseKPack(PackClass c, uint32_t tile, uint32_t blockK)
         {
             uint32_t groups = kWaveSize / tile;
             uint32_t p      = maxKPack(c);
-            while(p > 1u && !(kPackAllowed(c, p) && blockK % (p * groups) == 0u))
+            while(p > 1u && !(kPackAllowed(c, p, groups, blockK) && blockK % (p * groups) == 0u))
                 p >>= 1u;
             return p;
         }
@@ -118,6 +126,10 @@ namespace rocwmma
             static constexpr uint32_t ndim    = BlockDim / Tile;
             static constexpr uint32_t nchunks = ndim * nk; // MFMA operands held
             static constexpr uint32_t size    = nchunks * kpack; // elements per lane
+            // consecutive K steps one instruction consumes (fp8 wide-K forms: two 16-byte runs)
+            static constexpr uint32_t mmaSteps = (Class == PackClass::Fp8 && kpack == 16u) ? 2u : 1u;
+            static constexpr uint32_t mmaKPack = kpack * mmaSteps; // elements per lane and instruction
+            static constexpr uint32_t nmma     = nk / mmaSteps; // instructions along K
 
             static_assert(BlockK % kstep == 0u && nk >= 1u,
                           "BlockK must be a multiple of 64 / tile (4 for 16-wide, 2 for 32-wide blocks)");

@@ -12,7 +12,8 @@
 //   f16    32    8      v_mfma_f32_32x32x16_f16              16
 //   f16    32    4      v_mfma_f32_32x32x8_f16               8
 //   bf16   (same four shapes, *_bf16 / *_bf16_1k)
-//   fp8    16    32     v_mfma_f32_16x16x128_f8f6f4          128   (e4m3 / e5m2 in any mix)
+//   fp8    16    32     v_mfma_f32_16x16x128_f8f6f4          128   (e4m3 / e5m2 in any mix; two 16-byte runs
+//                                                                  per lane, see fragment_map.hpp)
 //   fp8    16    8      v_mfma_f32_16x16x32_{fp8,bf8}_{fp8,bf8}   32
 //   fp8    32    32     v_mfma_f32_32x32x64_f8f6f4           64
 //   fp8    32    8      v_mfma_f32_32x32x16_{fp8,bf8}_{fp8,bf8}   16
@@ -155,6 +156,48 @@ namespace rocwmma
         ROCWMMA_MFMA_F8F6F4(BF8, BF8)
 #undef ROCWMMA_MFMA_F8F6F4
         // clang-format on
+#endif // ROCWMMA_ARCH_GFX950
+
+        // The same wide-K family with block scales (OCP microscaling, MX): every 32 elements along K
+        // of a row share an E8M0 scale (a biased power-of-two exponent: value = element *
+        // 2^(scale - 127)).  Lane l passes, for each multiplicand, the scale of row (column) l % Tile and
+        // K block l / Tile of the instruction's K range, in one byte of a 32-bit register.  SelX / SelY
+        // choose that byte (instruction immediates), so one register can carry the scales of four
+        // instructions.
+        template <MmaClass CX, MmaClass CY, uint32_t Tile>
+        struct MfmaScaled
+        {
+            static constexpr bool supported = false;
+        };
+
+#if ROCWMMA_ARCH_GFX950
+#define ROCWMMA_MFMA_SCALED(CX, CY, TILE, SHAPE)                                                                     \
+    template <>                                                                                                       \
+    struct MfmaScaled<MmaClass::CX, MmaClass::CY, TILE>                                                              \
+    {                                                                                                                 \
+        static constexpr bool supported = true;                                                                       \
+        using Acc                       = typename AccRegs<float, TILE>::type;                                        \
+        template <int SelX = 0, int SelY = 0>                                                                         \
+        ROCWMMA_DEVICE static ROCWMMA_INLINE Acc exec(const void* x, const void* y, Acc acc, uint32_t scaleX,         \
+                                                      uint32_t scaleY)                                                \
+        {                                                                                                             \
+            const i32x8_t& X = *reinterpret_cast<const i32x8_t*>(x);                                                  \
+            const i32x8_t& Y = *reinterpret_cast<const i32x8_t*>(y);                                                  \
+            return __builtin_amdgcn_mfma_scale_f32_##SHAPE##_f8f6f4(X, Y, acc, F8Format<MmaClass::CX>::value,         \
+                                                                    F8Format<MmaClass::CY>::value, SelX,              \
+                                                                    static_cast<int>(scaleX), SelY,                   \
+                                                                    static_cast<int>(scaleY));                        \
+        }                                                                                                             \
+    };
+#define ROCWMMA_MFMA_SCALED_PAIR(CX, CY)       \
+    ROCWMMA_MFMA_SCALED(CX, CY, 16, 16x16x128) \
+    ROCWMMA_MFMA_SCALED(CX, CY, 32, 32x32x64)
+        ROCWMMA_MFMA_SCALED_PAIR(F8, F8)
+        ROCWMMA_MFMA_SCALED_PAIR(F8, BF8)
+        ROCWMMA_MFMA_SCALED_PAIR(BF8, F8)
+        ROCWMMA_MFMA_SCALED_PAIR(BF8, BF8)
+#undef ROCWMMA_MFMA_SCALED_PAIR
+#undef ROCWMMA_MFMA_SCALED
 #endif // ROCWMMA_ARCH_GFX950
 
 #undef ROCWMMA_MFMA_ENTRY

@@ -365,7 +365,7 @@ namespace rocwmma
                                 detail::TypeInfo<InputTA>::cls,
                                 NativeT,
                                 MapAcc::tile,
-                                MapA::kpack>;
+                                MapA::mmaKPack>;
         static_assert(Op::supported,
                       "no gfx950 MFMA instruction for this combination of input types, "
                       "accumulator type, block size and BlockK");
@@ -390,13 +390,14 @@ namespace rocwmma
 
             // K outermost so consecutive instructions write different accumulators
 #pragma unroll
-        for(uint32_t ks = 0; ks < MapA::nk; ++ks)
+        // (an fp8 wide-K instruction takes the registers of two consecutive K steps)
+        for(uint32_t ks = 0; ks < MapA::nmma; ++ks)
 #pragma unroll
             for(uint32_t bi = 0; bi < MapAcc::nbi; ++bi)
 #pragma unroll
                 for(uint32_t bj = 0; bj < MapAcc::nbj; ++bj)
-                    acc[bi][bj] = Op::exec(&b.x[MapB::chunkIndex(bj, ks) * MapB::kpack],
-                                           &a.x[MapA::chunkIndex(bi, ks) * MapA::kpack],
+                    acc[bi][bj] = Op::exec(&b.x[MapB::chunkIndex(bj, ks * MapB::mmaSteps) * MapB::kpack],
+                                           &a.x[MapA::chunkIndex(bi, ks * MapA::mmaSteps) * MapA::kpack],
                                            acc[bi][bj]);
 
 #pragma unroll

@@ -232,6 +232,55 @@ int rocwmma_amd_gemm_streamk_static(int         dtype_in,
                                     void*       stream);
 
 /*
+ * Block-scaled ("microscaled", MX) fp8 GEMM:
+ *     D = alpha * (A . 2^(scale_a - 127)) * (B . 2^(scale_b - 127)) + beta * C.
+ *
+ * A and B hold E4M3 or E5M2 elements (dtype_in); every 32 consecutive elements along K of a row of A
+ * and of a column of B share one E8M0 scale, a biased power-of-two exponent (the MXFP8 formats of the
+ * OCP Microscaling Formats specification v1.0; scale 255 encodes NaN).  C and D are F32.  On gfx950 the
+ * scales are applied inside the matrix cores (v_mfma_scale_f32_*_f8f6f4).
+ * The reference has no counterpart: its fp8 GEMMs multiply unscaled operands
+ * (test/gemm/gemm_common_test_params.hpp:170-196).  Arguments are those of rocwmma_amd_gemm plus
+ *   scale_a : m x (k / 32) bytes, K blocks of a row contiguous, leading dimension ld_scale_a >= k / 32;
+ *   scale_b : n x (k / 32) bytes, K blocks of a column of B contiguous, ld_scale_b >= k / 32;
+ * whatever the layouts of A and B themselves.
+ * Shapes: m, n multiples of 16 and k a multiple of 128, or m, n multiples of 32 and k a multiple of 64.
+ * workspace: NULL, or device memory (256-byte aligned) of at least
+ * rocwmma_amd_gemm_mx_workspace_size(m, n, k) bytes.  With a workspace, row-major A / col-major B
+ * (for a col-major C: col-major A / row-major B), m and n multiples of 256 and k a multiple of 128
+ * run on the blocked kernel (256 x 256 tiles, v_mfma_scale_f32_16x16x128_f8f6f4): the call then
+ * enqueues a small kernel that re-orders the scales into the workspace, and the GEMM (two launches).  Everything else
+ * runs one block per wave straight from global memory.  Two calls that use the same workspace must
+ * not overlap in time.
+ */
+size_t rocwmma_amd_gemm_mx_workspace_size(uint32_t m, uint32_t n, uint32_t k);
+
+int rocwmma_amd_gemm_mx(int         dtype_in,
+                        int         layout_a,
+                        int         layout_b,
+                        int         layout_c,
+                        uint32_t    m,
+                        uint32_t    n,
+                        uint32_t    k,
+                        const void* a,
+                        uint32_t    lda,
+                        const void* scale_a,
+                        uint32_t    ld_scale_a,
+                        const void* b,
+                        uint32_t    ldb,
+                        const void* scale_b,
+                        uint32_t    ld_scale_b,
+                        const void* c,
+                        uint32_t    ldc,
+                        void*       d,
+                        uint32_t    ldd,
+                        float       alpha,
+                        float       beta,
+                        void*       workspace,
+                        size_t      workspace_bytes,
+                        void*       stream);
+
+/*
  * Skinny GEMV / GEMM:  Y = alpha * A * X + beta * Y,  in place on Y.
  *
  * Stands in for sgemv_rocwmma_d and its host (samples/simple_sgemv.cpp:103-155,207-227), whose

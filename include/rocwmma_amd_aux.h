@@ -72,7 +72,8 @@ typedef enum rocwmma_amd_mfma_shape
     ROCWMMA_AMD_MFMA_I8_16X16X64   = 4,
     ROCWMMA_AMD_MFMA_I8_32X32X32   = 5,
     ROCWMMA_AMD_MFMA_F8_16X16X128  = 6, /* v_mfma_f32_16x16x128_f8f6f4 on e4m3 operands */
-    ROCWMMA_AMD_MFMA_F8_32X32X64   = 7
+    ROCWMMA_AMD_MFMA_F8_32X32X64   = 7,
+    ROCWMMA_AMD_MFMA_F8_16X16X128_SCALED = 8 /* the same instruction with per-lane block scales */
 } rocwmma_amd_mfma_shape;
 
 /*

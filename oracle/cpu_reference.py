@@ -117,6 +117,39 @@ def gemm(dtype_in, dtype_out, layA, layB, layC, layD, m, n, k, a, b, c, alpha, b
     return d
 
 
+MX_BLOCK = 32  # elements along K that share one scale (OCP Microscaling Formats v1.0, section 5)
+
+
+def mx_scale_values(scales):
+    """E8M0 scale bytes -> float32 factors 2^(e - 127) (e = 255 encodes NaN)."""
+    e = np.ascontiguousarray(scales, dtype=np.uint8).astype(np.int32)
+    out = np.ldexp(np.float32(1.0), e - 127).astype(np.float32)
+    out[e == 255] = np.nan
+    return out
+
+
+def mx_dequantise(dtype, bits, scales, layout, rows, k):
+    """Values of a block-scaled operand: `bits` holds a rows x k matrix (`layout` says whether rows
+    or K are contiguous: ROW_MAJOR = K contiguous), `scales` a rows x k/32 byte matrix (K blocks
+    contiguous).  Returns float32 in the same layout as `bits`.  The product element * 2^(e-127) is
+    exact in float32 for every finite fp8 value and every scale whose result stays normal."""
+    vals = decode(dtype, bits).reshape((rows, k) if layout == ROW_MAJOR else (k, rows))
+    fac = np.repeat(mx_scale_values(scales).reshape(rows, k // MX_BLOCK), MX_BLOCK, axis=1)
+    return (vals * (fac if layout == ROW_MAJOR else fac.T)).astype(np.float32)
+
+
+def gemm_mx(dtype_in, layA, layB, layC, layD, m, n, k, a, scale_a, b, scale_b, c, alpha, beta, rows=None):
+    """Block-scaled GEMM.  The reference has no such path; the definition is that of the OCP
+    Microscaling Formats specification v1.0 (section 6.2: the dot product of two MX vectors is the
+    sum over blocks of scaleA * scaleB * sum of element products), restated as: dequantise both
+    operands (exact, see mx_dequantise), then gemm_CPU's loop nest in float32
+    (test/reference_impl.hpp:36-81) on the dequantised values."""
+    af = mx_dequantise(dtype_in, a, scale_a, layA, m, k)
+    # B is k x n: its "rows" in the sense of mx_dequantise are its columns
+    bf = mx_dequantise(dtype_in, b, scale_b, ROW_MAJOR if layB == COL_MAJOR else COL_MAJOR, n, k)
+    return gemm(F32, F32, layA, layB, layC, layD, m, n, k, af, bf, c, alpha, beta, rows=rows)
+
+
 def dlrm_fwd(inp, m, k, batch):
     """dlrm_fwd_CPU (test/reference_impl.hpp:83-119) on f16 bit patterns."""
     inp = np.ascontiguousarray(inp, dtype=np.uint16).reshape(-1)

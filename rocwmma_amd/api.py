@@ -19,13 +19,14 @@ EXPORTS = [
     "rocwmma_amd_version", "rocwmma_amd_status_string", "rocwmma_amd_device_info", "rocwmma_amd_gemm",
     "rocwmma_amd_gemm_ex", "rocwmma_amd_gemv", "rocwmma_amd_dlrm_fwd", "rocwmma_amd_dlrm_bwd",
     "rocwmma_amd_gemm_streamk", "rocwmma_amd_gemm_streamk_workspace_size", "rocwmma_amd_gemm_streamk_static",
+    "rocwmma_amd_gemm_mx", "rocwmma_amd_gemm_mx_workspace_size",
 ]
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
 _AUX_LIB_NAME = "librocwmma_amd_aux.so"
 AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_bench_mfma_ceiling",
                "rocwmma_amd_bench_stream"]
 (MFMA_F16_16X16X32, MFMA_F16_32X32X16, MFMA_BF16_16X16X32, MFMA_BF16_32X32X16, MFMA_I8_16X16X64, MFMA_I8_32X32X32,
- MFMA_F8_16X16X128, MFMA_F8_32X32X64) = range(8)
+ MFMA_F8_16X16X128, MFMA_F8_32X32X64, MFMA_F8_16X16X128_SCALED) = range(9)
 
 
 class RocwmmaError(RuntimeError):
@@ -65,6 +66,10 @@ def library():
         L.rocwmma_amd_gemm_streamk.restype = i
         L.rocwmma_amd_gemm_streamk_static.argtypes = gemm_args
         L.rocwmma_amd_gemm_streamk_static.restype = i
+        L.rocwmma_amd_gemm_mx.argtypes = [i, i, i, i, u, u, u, vp, u, vp, u, vp, u, vp, u, vp, u, vp, u, f, f, vp, ctypes.c_size_t, vp]
+        L.rocwmma_amd_gemm_mx_workspace_size.argtypes = [u, u, u]
+        L.rocwmma_amd_gemm_mx_workspace_size.restype = ctypes.c_size_t
+        L.rocwmma_amd_gemm_mx.restype = i
         L.rocwmma_amd_gemm_streamk_workspace_size.argtypes = []
         L.rocwmma_amd_gemm_streamk_workspace_size.restype = ctypes.c_size_t
         L.rocwmma_amd_gemv.argtypes = [u, u, u, vp, u, vp, u, vp, u, f, f, vp]
@@ -196,6 +201,31 @@ def gemm_streamk_static(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n,
     rc = library().rocwmma_amd_gemm_streamk_static(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, _ptr(a),
                                                    lda, _ptr(b), ldb, _ptr(c), ldc, _ptr(d), ldd, alpha, beta, _stream())
     _check(rc, "gemm_streamk_static")
+    return d
+
+
+def gemm_mx_workspace_size(m, n, k):
+    return int(library().rocwmma_amd_gemm_mx_workspace_size(m, n, k))
+
+
+def gemm_mx(dtype_in, layout_a, layout_b, layout_c, m, n, k, a, scale_a, b, scale_b, c, d, alpha, beta,
+            workspace=None, lda=None, ldb=None, ldc=None, ldd=None, ld_scale_a=None, ld_scale_b=None):
+    """rocwmma_amd_gemm_mx on device tensors: fp8 / bf8 operands with one E8M0 scale byte per 32
+    elements along K (scale_a: m x k/32, scale_b: n x k/32, K blocks contiguous), f32 C / D.
+    `workspace`: None (one-block-per-wave kernel) or a device tensor of at least
+    gemm_mx_workspace_size(m, n, k) bytes (blocked kernel where the shape allows)."""
+    lda = lda if lda is not None else (k if layout_a == ROW_MAJOR else m)
+    ldb = ldb if ldb is not None else (n if layout_b == ROW_MAJOR else k)
+    nat = n if layout_c == ROW_MAJOR else m
+    ldc = ldc if ldc is not None else nat
+    ldd = ldd if ldd is not None else nat
+    ld_scale_a = ld_scale_a if ld_scale_a is not None else k // 32
+    ld_scale_b = ld_scale_b if ld_scale_b is not None else k // 32
+    rc = library().rocwmma_amd_gemm_mx(dtype_in, layout_a, layout_b, layout_c, m, n, k, _ptr(a), lda, _ptr(scale_a),
+                                       ld_scale_a, _ptr(b), ldb, _ptr(scale_b), ld_scale_b, _ptr(c), ldc, _ptr(d), ldd,
+                                       alpha, beta, _ptr(workspace),
+                                       0 if workspace is None else workspace.numel() * workspace.element_size(), _stream())
+    _check(rc, "gemm_mx")
     return d
 
 

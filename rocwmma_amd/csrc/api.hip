@@ -285,6 +285,78 @@ int rocwmma_amd_gemm_streamk_static(int         dtype_in,
     return launchGemmStreamKStatic(dtype_in, dtype_out, la, lb, args, asStream(stream));
 }
 
+size_t rocwmma_amd_gemm_mx_workspace_size(uint32_t m, uint32_t n, uint32_t k)
+{
+    return mxPackedScaleBytes(m, n, k);
+}
+
+int rocwmma_amd_gemm_mx(int         dtype_in,
+                        int         layout_a,
+                        int         layout_b,
+                        int         layout_c,
+                        uint32_t    m,
+                        uint32_t    n,
+                        uint32_t    k,
+                        const void* a,
+                        uint32_t    lda,
+                        const void* scale_a,
+                        uint32_t    ld_scale_a,
+                        const void* b,
+                        uint32_t    ldb,
+                        const void* scale_b,
+                        uint32_t    ld_scale_b,
+                        const void* c,
+                        uint32_t    ldc,
+                        void*       d,
+                        uint32_t    ldd,
+                        float       alpha,
+                        float       beta,
+                        void*       workspace,
+                        size_t      workspace_bytes,
+                        void*       stream)
+{
+    if(dtype_in != ROCWMMA_AMD_E4M3 && dtype_in != ROCWMMA_AMD_E5M2)
+        return ROCWMMA_AMD_UNSUPPORTED_TYPE;
+    int rc = checkGemm(dtype_in, ROCWMMA_AMD_F32, layout_a, layout_b, layout_c, m, n, k, a, lda, b, ldb, c, ldc, d, ldd, alpha, beta);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(!scale_a || !scale_b)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(k % 64u != 0u)
+        return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+    if(ld_scale_a < k / 32u || ld_scale_b < k / 32u)
+        return ROCWMMA_AMD_BAD_LEADING_DIM;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    GemmArgs args{m, n, k, a, b, c, d, lda, ldb, c ? ldc : ldd, ldd, alpha, beta, layout_c};
+    MxScales scales{static_cast<const uint8_t*>(scale_a), static_cast<const uint8_t*>(scale_b), ld_scale_a, ld_scale_b};
+    if(workspace && workspace_bytes >= mxPackedScaleBytes(m, n, k) && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0u)
+    {
+        GemmArgs blocked = args;
+        MxScales sc      = scales;
+        int      la = layout_a, lb = layout_b;
+        if(blocked.layoutC == ROCWMMA_AMD_COL_MAJOR)
+        {
+            std::swap(sc.a, sc.b);
+            std::swap(sc.lda, sc.ldb);
+        }
+        transposeForColMajorC(blocked, la, lb);
+        if(la == ROCWMMA_AMD_ROW_MAJOR && lb == ROCWMMA_AMD_COL_MAJOR && blocked.m % 256u == 0u && blocked.n % 256u == 0u
+           && k % 128u == 0u)
+        {
+            char* packedA = static_cast<char*>(workspace);
+            char* packedB = packedA + mxPackedScaleOffsetB(blocked.m, k);
+            rc            = launchMxPackScales(sc, blocked.m, blocked.n, k, packedA, packedB, asStream(stream));
+            if(rc != ROCWMMA_AMD_OK)
+                return rc;
+            rc = launchGemmMxBlocked(dtype_in, blocked, packedA, packedB, asStream(stream));
+            if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                return rc;
+        }
+    }
+    return launchGemmMxWaveTile(dtype_in, layout_a, layout_b, args, scales, asStream(stream));
+}
+
 int rocwmma_amd_gemm(int         dtype_in,
                      int         dtype_out,
                      int         layout_a,

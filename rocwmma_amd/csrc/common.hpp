@@ -81,6 +81,15 @@ namespace rocwmma_amd
         int         layoutC;
     };
 
+    // Block scales of a microscaled GEMM: one E8M0 byte per 32 elements along K of every row of A
+    // (a: m x k/32, leading dimension lda) and every column of B (b: n x k/32, leading dimension ldb).
+    struct MxScales
+    {
+        const uint8_t* a;
+        const uint8_t* b;
+        uint32_t       lda, ldb;
+    };
+
     // Family launchers (one translation unit each).  Return a rocwmma_amd_status;
     // ROCWMMA_AMD_UNSUPPORTED_SHAPE / _TYPE mean "this family has no kernel for it".
     int launchGemmWaveTile(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
@@ -96,6 +105,31 @@ namespace rocwmma_amd
                              size_t workspaceBytes, hipStream_t stream);
     // the same on the library's own scratch (a static device array): allocates nothing
     int    launchGemmStreamKStatic(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
+
+    // Scales of the blocked block-scaled kernel, re-ordered into the order its lanes load them in:
+    // per operand, groups of 64 rows of A (columns of B) x pairs of 128-byte K stages x 64 lanes x 4
+    // blocks of 16 rows x 2 stages, one byte each -- 8 contiguous bytes per lane, group and stage pair.
+    // A's part comes first; B's starts at the next multiple of 256 bytes.
+    inline size_t mxPackedScaleBytesOf(uint32_t rows, uint32_t k)
+    {
+        return static_cast<size_t>((rows + 63u) / 64u) * ((k + 255u) / 256u) * 64u * 8u;
+    }
+    inline size_t mxPackedScaleOffsetB(uint32_t m, uint32_t k)
+    {
+        return (mxPackedScaleBytesOf(m, k) + 255u) & ~static_cast<size_t>(255u);
+    }
+    inline size_t mxPackedScaleBytes(uint32_t m, uint32_t n, uint32_t k)
+    {
+        return mxPackedScaleOffsetB(m, k) + mxPackedScaleBytesOf(n, k);
+    }
+    // Re-orders both operands' scales (one launch).
+    int launchMxPackScales(MxScales const& scales, uint32_t m, uint32_t n, uint32_t k, void* packedA, void* packedB, hipStream_t stream);
+    // The blocked kernel on packed scales: row-major A, col-major B, row-major C/D, m and n multiples
+    // of 256, k a multiple of 128.
+    int launchGemmMxBlocked(int dtypeIn, GemmArgs const& args, const void* packedA, const void* packedB, hipStream_t stream);
+
+    // Block-scaled fp8 / bf8 GEMM (f32 C/D): one block per wave, every layout pair
+    int launchGemmMxWaveTile(int dtypeIn, int layoutA, int layoutB, GemmArgs const& args, MxScales const& scales, hipStream_t stream);
 
 } // namespace rocwmma_amd
 

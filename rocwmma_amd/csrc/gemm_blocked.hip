@@ -22,11 +22,12 @@ namespace rocwmma_amd
                           uint32_t                   ldc,
                           uint32_t                   ldd,
                           typename Cfg::CompT        alpha,
-                          typename Cfg::CompT        beta)
+                          typename Cfg::CompT        beta,
+                          MxPacked                   mx) // block scales (Scaled configurations only)
         {
             uint32_t tm, tn;
             tileOfWorkgroup(blockIdx.x, ceilDiv(m, Cfg::MacroM), ceilDiv(n, Cfg::MacroN), tm, tn);
-            gemmTile<Cfg>(tm, tn, 0u, k / Cfg::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
+            gemmTile<Cfg>(tm, tn, 0u, k / Cfg::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{}, mx);
         }
 
         // Two tilings in one launch: the first `fullTiles` workgroups run Full tiles, the others the two
@@ -47,7 +48,8 @@ namespace rocwmma_amd
                                    uint32_t                   ldd,
                                    typename Full::CompT       alpha,
                                    typename Full::CompT       beta,
-                                   uint32_t                   fullTiles)
+                                   uint32_t                   fullTiles,
+                                   MxPacked                   mx)
         {
             // (The half tiles go last.  Running half of them first, on half of the compute units of every
             // XCD or on XCDs 0-3, so that one half of the device writes its results while the other is in
@@ -57,14 +59,14 @@ namespace rocwmma_amd
             if(blockIdx.x < fullTiles)
             {
                 tileOfWorkgroup(blockIdx.x, tilesM, tilesN, tm, tn);
-                gemmTile<Full>(tm, tn, 0u, k / Full::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{});
+                gemmTile<Full>(tm, tn, 0u, k / Full::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{}, mx);
             }
             else
             {
                 const uint32_t j = blockIdx.x - fullTiles;
                 tileOfWorkgroup(fullTiles + j / 2u, tilesM, tilesN, tm, tn);
                 gemmTile<Half>(tm, 2u * tn + (j & 1u), 0u, k / Half::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha,
-                               beta, StreamKPart{});
+                               beta, StreamKPart{}, mx);
             }
         }
 
@@ -73,7 +75,7 @@ namespace rocwmma_amd
         // that occupies at most half of the compute units for the time of a whole tile (4096 x 14336: 896
         // tiles on 256 units, 3.5 rounds; 6144^3: 2.25 rounds).
         template <typename Full, typename Half>
-        int launchSplitTail(GemmArgs const& g, hipStream_t stream)
+        int launchSplitTail(GemmArgs const& g, hipStream_t stream, MxPacked const& mx = MxPacked{})
         {
             static_assert(Full::MacroM == Half::MacroM && Full::MacroN == 2u * Half::MacroN && Full::MacroK == Half::MacroK
                               && Full::Threads == Half::Threads && Full::Stages == Half::Stages
@@ -105,12 +107,12 @@ namespace rocwmma_amd
                                static_cast<typename Full::InT const*>(g.a), static_cast<typename Full::InT const*>(g.b),
                                static_cast<typename Full::OutT const*>(g.c), static_cast<typename Full::OutT*>(g.d), g.lda,
                                g.ldb, g.ldc, g.ldd, static_cast<typename Full::CompT>(g.alpha),
-                               static_cast<typename Full::CompT>(g.beta), fullTiles);
+                               static_cast<typename Full::CompT>(g.beta), fullTiles, mx);
             return launchStatus();
         }
 
         template <typename Cfg>
-        int launchCfg(GemmArgs const& g, hipStream_t stream)
+        int launchCfg(GemmArgs const& g, hipStream_t stream, MxPacked const& mx = MxPacked{})
         {
             if((!Cfg::Edges && (g.m % Cfg::MacroM != 0u || g.n % Cfg::MacroN != 0u)) || g.k % Cfg::MacroK != 0u
                || g.k < (Cfg::Stages - 1u) * Cfg::MacroK)
@@ -149,7 +151,8 @@ namespace rocwmma_amd
                                g.ldc,
                                g.ldd,
                                static_cast<typename Cfg::CompT>(g.alpha),
-                               static_cast<typename Cfg::CompT>(g.beta));
+                               static_cast<typename Cfg::CompT>(g.beta),
+                               mx);
             return launchStatus();
         }
 
@@ -311,6 +314,34 @@ namespace rocwmma_amd
             return pickTile<InT, OutT, CompT, false, false>(g, stream, big);
         }
     } // namespace
+
+    namespace
+    {
+        template <typename InT>
+        int launchMx(GemmArgs const& g, MxPacked const& mx, hipStream_t stream)
+        {
+            // 256 x 256 tiles of 16x16x128 blocks with block scales; the tiles of a last round at most half
+            // full run as 256 x 128 half tiles, as in the unscaled kernel
+            using Big     = BlockedConfig<InT, float32_t, float32_t, true, true, 4, 2, 4, 8, 2, 2, 16, false, true>;
+            using BigHalf = BlockedConfig<InT, float32_t, float32_t, true, true, 4, 2, 4, 4, 2, 2, 16, false, true>;
+            const int rc  = launchSplitTail<Big, BigHalf>(g, stream, mx);
+            if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                return rc;
+            return launchCfg<Big>(g, stream, mx);
+        }
+    } // namespace
+
+    int launchGemmMxBlocked(int dtypeIn, GemmArgs const& g, const void* packedA, const void* packedB, hipStream_t stream)
+    {
+        if(g.layoutC != ROCWMMA_AMD_ROW_MAJOR || g.m % 256u != 0u || g.n % 256u != 0u || g.k % 128u != 0u)
+            return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+        const MxPacked mx{packedA, packedB, (g.k / 128u + 1u) / 2u};
+        if(dtypeIn == ROCWMMA_AMD_E4M3)
+            return launchMx<float8_t>(g, mx, stream);
+        if(dtypeIn == ROCWMMA_AMD_E5M2)
+            return launchMx<bfloat8_t>(g, mx, stream);
+        return ROCWMMA_AMD_UNSUPPORTED_TYPE;
+    }
 
     int launchGemmBlocked(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream,
                           bool forceLargeTile)

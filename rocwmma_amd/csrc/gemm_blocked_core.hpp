@@ -49,7 +49,8 @@ namespace rocwmma_amd
                   uint32_t Stages_       = 4u, // LDS ring depth
                   uint32_t WavesPerSimd_ = 1u, // waves per SIMD: sizes the register budget, and no more become resident
                   uint32_t BlockEdge_    = 32u, // MFMA block edge: 32 (32x32xK) or 16 (16x16x2K)
-                  bool     Edges_        = false> // M and N need not fill whole macro tiles (multiples of 16 do)
+                  bool     Edges_        = false, // M and N need not fill whole macro tiles (multiples of 16 do)
+                  bool     Scaled_       = false> // fp8 operands with one E8M0 scale per 32 elements of K (MX)
         struct BlockedConfig
         {
             using InT   = InT_;
@@ -62,6 +63,10 @@ namespace rocwmma_amd
             // are cut off by the buffer bounds (rows and columns beyond the problem only ever meet
             // results beyond it), C reads and D stores are masked lane by lane.
             static constexpr bool     Edges   = Edges_;
+            // Block-scaled operands: the scaled instruction's K order decides which bytes a lane holds
+            // (two runs of 16 from the two halves of the stage, see rocwmma/internal/fragment_map.hpp),
+            // so the fragments are read like two steps of a 16-bytes-per-lane operand.
+            static constexpr bool     Scaled  = Scaled_;
             static constexpr uint32_t WavesM  = WavesM_;
             static constexpr uint32_t WavesN  = WavesN_;
             static constexpr uint32_t BlocksM = BlocksM_;
@@ -94,7 +99,7 @@ namespace rocwmma_amd
             using DimTile = std::conditional_t<sizeof(InT) == 2u, lds::DimMajorTile<Dim, StageKB / 2u>,
                                                lds::DimMajorTile8<(Dim == 128u || Dim == 256u) ? Dim : 128u, StageKB>>;
             // (16-wide blocks with 32 bytes of K per lane, fp8 16x16x128: the K-major tile's pair reader)
-            static constexpr bool PairReads = Block == 16u && KPackBytes == 32u;
+            static constexpr bool PairReads = Block == 16u && KPackBytes == 32u && !Scaled;
             using TileA = std::conditional_t<AKMajor, lds::KMajorTile<MacroM, StageKB, PairReads>, DimTile<MacroM>>;
             using TileB = std::conditional_t<BKMajor, lds::KMajorTile<MacroN, StageKB, PairReads>, DimTile<MacroN>>;
 
@@ -122,7 +127,9 @@ namespace rocwmma_amd
                                             && 2u * Block * GroupBlocks * Block * sizeof(OutT) * Waves <= LdsBytes;
 
             static_assert(Block == 32u || Block == 16u, "MFMA blocks are 32 or 16 wide");
-            static_assert(Block == 32u || KPackBytes == 16u || (PairReads && AKMajor && BKMajor && Stages_ == 2u),
+            static_assert(!Scaled || (Block == 16u && KPackBytes == 32u && AKMajor && BKMajor && Stages_ == 2u && !Edges_),
+                          "block scales: fp8 16x16x128 on K-contiguous operands in the ring of two, whole tiles");
+            static_assert(Block == 32u || KPackBytes == 16u || ((PairReads || Scaled) && AKMajor && BKMajor && Stages_ == 2u),
                           "16-wide blocks: 16 bytes of K per lane (16-bit types, int8), or fp8 16x16x128 on K-contiguous "
                           "operands in the ring of two");
             static_assert(sizeof(InT) == 2u || sizeof(InT) == 1u, "16-bit and 8-bit operands");
@@ -193,6 +200,30 @@ namespace rocwmma_amd
             }
         }
 
+
+        // Compile-time loop: f(std::integral_constant<uint32_t, 0>{}), ..., f(<N - 1>) -- for bodies whose
+        // iteration index must be a constant expression (instruction immediates).
+        template <typename F, uint32_t... I>
+        ROCWMMA_DEVICE ROCWMMA_INLINE void staticForImpl(F&& f, std::integer_sequence<uint32_t, I...>)
+        {
+            (f(std::integral_constant<uint32_t, I>{}), ...);
+        }
+        template <uint32_t N, typename F>
+        ROCWMMA_DEVICE ROCWMMA_INLINE void staticFor(F&& f)
+        {
+            staticForImpl(f, std::make_integer_sequence<uint32_t, N>{});
+        }
+
+        // Block scales of a Scaled configuration, in the order the lanes load them (written by the
+        // re-ordering kernel in gemm_mx.hip): per operand, group of 64 rows of A (columns of B) and pair
+        // of K stages, 8 bytes per lane = [block of 16 rows 0..3][stage of the pair 0..1]; lane l's bytes
+        // are the scales of row l % 16 of each block and K block l / 16 of each stage.
+        struct MxPacked
+        {
+            const void* a;
+            const void* b;
+            uint32_t    pairs; // pairs of stages along K (the last one padded when the stage count is odd)
+        };
 
         // ---- stream-K support ------------------------------------------------------------------
         // Which part of a tile's K range a call of gemmTile computes.
@@ -329,7 +360,8 @@ namespace rocwmma_amd
                                                     uint32_t                   ldd,
                                                     typename Cfg::CompT        alpha,
                                                     typename Cfg::CompT        beta,
-                                                    StreamKPart const&         sk)
+                                                    StreamKPart const&         sk,
+                                                    MxPacked const&            mx = MxPacked{})
         {
             using InT   = typename Cfg::InT;
             using OutT  = typename Cfg::OutT;
@@ -412,6 +444,10 @@ namespace rocwmma_amd
             auto readFrags = [&](Frags& f, uint32_t slot, uint32_t ks) {
                 const char* ldsA = ldsRaw + slot * Cfg::StageBytes;
                 const char* ldsB = ldsA + Cfg::BytesA;
+                if constexpr(Cfg::Scaled) // (has a reader of its own in its loop)
+                    return;
+                else
+                {
 #pragma unroll
                 for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
                 {
@@ -427,6 +463,7 @@ namespace rocwmma_amd
                         TileB::template readBlock32<Cfg::KPackBytes>(f.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, ks, lane);
                     else
                         TileB::template readBlock16<Cfg::KPackBytes>(f.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, ks, lane);
+                }
                 }
             };
 
@@ -476,6 +513,33 @@ namespace rocwmma_amd
                 // needs from stage i (the last column's fragment arrived with the wait), stage i + 1 has
                 // landed, and the copies of stage i + 2 go out into stage i's slot.
                 static_assert(Cfg::AKMajor && Cfg::BKMajor, "streamed columns: K-contiguous operands");
+                static_assert(!Cfg::Scaled || Part == TilePart::Whole, "block scales: whole K ranges from stage 0");
+                // Block scales (Scaled only): per lane, pair of stages and group of four blocks, two
+                // registers: byte (block % 2) * 2 + stage parity of register (block % 4) / 2.  The next
+                // pair's are loaded while the first stage of a pair is multiplied and take over after the
+                // second.
+                typedef uint32_t   Scales __attribute__((ext_vector_type(2)));
+                constexpr uint32_t GroupsN = Cfg::BlocksN / 4u;
+                static_assert(!Cfg::Scaled || (Cfg::BlocksM == 4u && Cfg::BlocksN % 4u == 0u), "packed scales: groups of four blocks");
+                Scales        sA = {}, sAnext = {};
+                Scales        sB[GroupsN > 0u ? GroupsN : 1u] = {}, sBnext[GroupsN > 0u ? GroupsN : 1u] = {};
+                const Scales* mxA = nullptr;
+                const Scales* mxB = nullptr;
+                auto loadScales = [&](Scales& a_, Scales(&b_)[GroupsN > 0u ? GroupsN : 1u], uint32_t pair) {
+                    a_ = mxA[static_cast<size_t>(pair) * 64u];
+#pragma unroll
+                    for(uint32_t gN = 0; gN < GroupsN; ++gN)
+                        b_[gN] = mxB[(static_cast<size_t>(gN) * mx.pairs + pair) * 64u];
+                };
+                if constexpr(Cfg::Scaled)
+                {
+                    mxA = static_cast<const Scales*>(mx.a) + static_cast<size_t>(row0 / 64u + waveM) * mx.pairs * 64u + lane;
+                    mxB = static_cast<const Scales*>(mx.b) + static_cast<size_t>(col0 / 64u + waveN * GroupsN) * mx.pairs * 64u + lane;
+                    // (in front of the first copies: the wait for stage 0 below then covers these loads, and the
+                    // loop is entered with none of them in flight)
+                    loadScales(sA, sB, 0u);
+                    __builtin_amdgcn_sched_barrier(0); // (and stay in front of them)
+                }
                 issueStage(0u, 1u < stages);
                 issueStage(1u, 2u < stages);
                 lds::waitCopiesAndReads<Cfg::Copies>(); // stage 0 has landed
@@ -486,48 +550,98 @@ namespace rocwmma_amd
                     const char* ldsA = ldsRaw + slot * Cfg::StageBytes;
 #pragma unroll
                     for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
-                        TileA::template readBlock16<Cfg::KPackBytes>(dst[bi].x, ldsA, waveM * Cfg::WaveM + bi * Cfg::Block, 0u, lane);
+                    {
+                        const uint32_t r0 = waveM * Cfg::WaveM + bi * Cfg::Block;
+                        if constexpr(Cfg::Scaled)
+                        {
+                            TileA::template readBlock16<16u>(dst[bi].x, ldsA, r0, 0u, lane);
+                            TileA::template readBlock16<16u>(dst[bi].x + 16, ldsA, r0, 1u, lane);
+                        }
+                        else
+                            TileA::template readBlock16<Cfg::KPackBytes>(dst[bi].x, ldsA, r0, 0u, lane);
+                    }
                 };
                 auto readB = [&](typename Cfg::FragB& dst, uint32_t slot, uint32_t bj) {
-                    const char* ldsB = ldsRaw + slot * Cfg::StageBytes + Cfg::BytesA;
-                    TileB::template readBlock16<Cfg::KPackBytes>(dst.x, ldsB, waveN * Cfg::WaveN + bj * Cfg::Block, 0u, lane);
+                    const char*    ldsB = ldsRaw + slot * Cfg::StageBytes + Cfg::BytesA;
+                    const uint32_t c0   = waveN * Cfg::WaveN + bj * Cfg::Block;
+                    if constexpr(Cfg::Scaled)
+                    {
+                        TileB::template readBlock16<16u>(dst.x, ldsB, c0, 0u, lane);
+                        TileB::template readBlock16<16u>(dst.x + 16, ldsB, c0, 1u, lane);
+                    }
+                    else
+                        TileB::template readBlock16<Cfg::KPackBytes>(dst.x, ldsB, c0, 0u, lane);
                 };
-                auto column = [&](typename Cfg::FragA const(&a_)[Cfg::BlocksM], typename Cfg::FragB const& b_, uint32_t bj) {
+                auto column = [&](typename Cfg::FragA const(&a_)[Cfg::BlocksM], typename Cfg::FragB const& b_, auto bjC, auto stC) {
+                    constexpr uint32_t bj = decltype(bjC)::value, st = decltype(stC)::value;
+                    if constexpr(Cfg::Scaled)
+                    {
+#if ROCWMMA_ARCH_GFX950 // (the instruction table exists in the device pass only)
+                        using Op  = detail::MfmaScaled<detail::TypeInfo<InT>::cls, detail::TypeInfo<InT>::cls, 16u>;
+                        using Acc = typename Op::Acc;
+                        staticFor<Cfg::BlocksM>([&](auto biC) {
+                            constexpr uint32_t bi = decltype(biC)::value;
+                            Acc&               v  = *reinterpret_cast<Acc*>(acc[bi][bj].x);
+                            // (the accumulator is kept transposed: the instruction's first multiplicand is B)
+                            v = Op::template exec<(bj % 2u) * 2u + st, (bi % 2u) * 2u + st>(b_.x, a_[bi].x, v, sB[bj / 4u][(bj % 4u) / 2u],
+                                                                                           sA[bi / 2u]);
+                        });
+#else
+                        (void)a_, (void)b_, (void)bj, (void)st;
+#endif
+                    }
+                    else
+                    {
 #pragma unroll
-                    for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
-                        mma_sync(acc[bi][bj], a_[bi], b_, acc[bi][bj]);
+                        for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+                            mma_sync(acc[bi][bj], a_[bi], b_, acc[bi][bj]);
+                    }
                 };
                 constexpr uint32_t RB = Cfg::KPackBytes / 16u; // LDS reads per block
                 readA(fa[0], 0u);
                 readB(fb[0], 0u, 0u);
                 // (the A sets alternate with the stage parity; two stages per trip keep the indices static)
-                auto stage = [&](typename Cfg::FragA(&cur)[Cfg::BlocksM], typename Cfg::FragA(&nxt)[Cfg::BlocksM],
-                                 uint32_t slot, uint32_t ii) {
-#pragma unroll
-                        for(uint32_t bj = 0; bj + 1u < Cfg::BlocksN; ++bj)
-                        {
+                auto stage = [&](typename Cfg::FragA(&cur)[Cfg::BlocksM], typename Cfg::FragA(&nxt)[Cfg::BlocksM], auto slotC,
+                                 uint32_t ii) {
+                        constexpr uint32_t slot = decltype(slotC)::value;
+                        staticFor<Cfg::BlocksN - 1u>([&](auto bjC) {
+                            constexpr uint32_t bj = decltype(bjC)::value;
                             readB(fb[(bj + 1u) & 1u], slot, bj + 1u);
-                            column(cur, fb[bj & 1u], bj);
+                            column(cur, fb[bj & 1u], bjC, slotC);
                             scheduleInterleaved<Cfg::BlocksM, RB, 0u>();
                             __builtin_amdgcn_sched_barrier(0);
-                        }
+                        });
                         lds::waitCopiesAndReads<0u>(); // stage ii + 1 has landed, stage ii is in registers
                         lds::barrier();
                         __builtin_amdgcn_sched_barrier(0);
                         issueStage(slot, ii + 3u < stages);
+                        if constexpr(Cfg::Scaled && slot == 0u)
+                        {
+                            // scales of the next pair of stages (the last pair again past the end of K)
+                            loadScales(sAnext, sBnext, ii / 2u + 1u < mx.pairs ? ii / 2u + 1u : mx.pairs - 1u);
+                        }
                         readA(nxt, slot ^ 1u);
                         readB(fb[0], slot ^ 1u, 0u);
-                        column(cur, fb[(Cfg::BlocksN - 1u) & 1u], Cfg::BlocksN - 1u);
+                        column(cur, fb[(Cfg::BlocksN - 1u) & 1u], std::integral_constant<uint32_t, Cfg::BlocksN - 1u>{}, slotC);
                         __builtin_amdgcn_sched_barrier(0);
+                        if constexpr(Cfg::Scaled && slot == 1u)
+                        {
+                            sA = sAnext;
+#pragma unroll
+                            for(uint32_t gN = 0; gN < GroupsN; ++gN)
+                                sB[gN] = sBnext[gN];
+                        }
                 };
+                const std::integral_constant<uint32_t, 0u> even{};
+                const std::integral_constant<uint32_t, 1u> odd{};
                 uint32_t i = 0;
                 for(; i + 1u < stages; i += 2u)
                 {
-                    stage(fa[0], fa[1], 0u, i);
-                    stage(fa[1], fa[0], 1u, i + 1u);
+                    stage(fa[0], fa[1], even, i);
+                    stage(fa[1], fa[0], odd, i + 1u);
                 }
                 if(i < stages)
-                    stage(fa[0], fa[1], 0u, i);
+                    stage(fa[0], fa[1], even, i);
                 lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
                 lds::barrier();
             }

@@ -1,0 +1,177 @@
+// Block-scaled (OCP microscaling) fp8 / bf8 GEMM: D = alpha * (A . 2^(SA - 127)) * (B . 2^(SB - 127)) + beta * C,
+// one E8M0 scale per 32 elements along K of every row of A and every column of B.
+//
+// The reference has no block-scaled path (its fp8 GEMM tests multiply unscaled operands,
+// test/gemm/gemm_common_test_params.hpp:170-196); this is the CDNA4 form of the same GEMM for
+// quantised inference, where the scales are applied inside the matrix cores
+// (v_mfma_scale_f32_*_f8f6f4) at no cost in instructions.
+//
+// Kernels here: one output block per wave, operands and scales straight from global memory through the
+// fragment API (rocwmma_mx.hpp) -- every layout pair, every shape in whole blocks; and the kernel that
+// re-orders the scales for the blocked kernel (gemm_blocked.hip, Scaled configurations).
+#include "common.hpp"
+
+#include <rocwmma/rocwmma_mx.hpp>
+
+using namespace rocwmma;
+
+namespace rocwmma_amd
+{
+    namespace
+    {
+        constexpr uint32_t kWavesX = 2; // along M  (blockDim.x = 64 * kWavesX)
+        constexpr uint32_t kWavesY = 2; // along N  (blockDim.y = kWavesY)
+
+        template <typename InT, typename LA, typename LB, uint32_t B, uint32_t BK>
+        __global__ void __launch_bounds__(64 * kWavesX * kWavesY) gemmMxWaveTileKernel(GemmArgs g, MxScales s)
+        {
+            using FragA   = fragment<matrix_a, B, B, BK, InT, LA>;
+            using FragB   = fragment<matrix_b, B, B, BK, InT, LB>;
+            using FragAcc = fragment<accumulator, B, B, BK, float32_t>;
+            using MapA    = GetDataLayout_t<FragA>;
+            using MapB    = GetDataLayout_t<FragB>;
+
+            const uint32_t waveRow = (blockIdx.x * blockDim.x + threadIdx.x) / Constants::AMDGCN_WAVE_SIZE;
+            const uint32_t waveCol = blockIdx.y * blockDim.y + threadIdx.y;
+            const uint32_t cRow    = waveRow * B;
+            const uint32_t cCol    = waveCol * B;
+            if(cRow >= g.m || cCol >= g.n)
+                return;
+
+            FragAcc acc;
+            fill_fragment(acc, 0.0f);
+
+            const InT* aPtr = static_cast<const InT*>(g.a) + (std::is_same<LA, row_major>::value ? static_cast<size_t>(cRow) * g.lda : cRow);
+            const InT* bPtr = static_cast<const InT*>(g.b) + (std::is_same<LB, row_major>::value ? cCol : static_cast<size_t>(cCol) * g.ldb);
+            const mx::scale_t* saPtr = s.a + static_cast<size_t>(cRow) * s.lda;
+            const mx::scale_t* sbPtr = s.b + static_cast<size_t>(cCol) * s.ldb;
+            const uint32_t     aStep = MapA::fromMatrixCoord(make_coord2d(0u, BK), g.lda);
+            const uint32_t     bStep = MapB::fromMatrixCoord(make_coord2d(BK, 0u), g.ldb);
+
+            for(uint32_t i = 0; i < g.k; i += BK)
+            {
+                FragA                     fa;
+                FragB                     fb;
+                mx::scale_fragment<FragA> sa;
+                mx::scale_fragment<FragB> sb;
+                load_matrix_sync(fa, aPtr, g.lda);
+                load_matrix_sync(fb, bPtr, g.ldb);
+                mx::load_scale_sync(sa, saPtr, s.lda);
+                mx::load_scale_sync(sb, sbPtr, s.ldb);
+                mx::mma_sync(acc, fa, sa, fb, sb, acc);
+                aPtr += aStep;
+                bPtr += bStep;
+                saPtr += BK / mx::BLOCK_SIZE;
+                sbPtr += BK / mx::BLOCK_SIZE;
+            }
+
+            const layout_t layoutC = g.layoutC == ROCWMMA_AMD_ROW_MAJOR ? mem_row_major : mem_col_major;
+            const float*   c       = static_cast<const float*>(g.c);
+            float*         d       = static_cast<float*>(g.d);
+            const size_t   cOff = layoutC == mem_row_major ? static_cast<size_t>(cRow) * g.ldc + cCol : static_cast<size_t>(cCol) * g.ldc + cRow;
+            const size_t   dOff = layoutC == mem_row_major ? static_cast<size_t>(cRow) * g.ldd + cCol : static_cast<size_t>(cCol) * g.ldd + cRow;
+            FragAcc        fc;
+            if(g.beta != 0.0f)
+            {
+                load_matrix_sync(fc, c + cOff, g.ldc, layoutC);
+#pragma unroll
+                for(uint32_t i = 0; i < fc.num_elements; ++i)
+                    fc.x[i] = g.alpha * acc.x[i] + g.beta * fc.x[i];
+            }
+            else
+            {
+#pragma unroll
+                for(uint32_t i = 0; i < fc.num_elements; ++i)
+                    fc.x[i] = g.alpha * acc.x[i];
+            }
+            store_matrix_sync(d + dOff, fc, g.ldd, layoutC);
+        }
+
+        template <typename InT, typename LA, typename LB, uint32_t B, uint32_t BK>
+        int launchOne(GemmArgs const& g, MxScales const& s, hipStream_t stream)
+        {
+            dim3 block(64 * kWavesX, kWavesY);
+            dim3 grid((g.m + B * kWavesX - 1u) / (B * kWavesX), (g.n + B * kWavesY - 1u) / (B * kWavesY));
+            hipLaunchKernelGGL((gemmMxWaveTileKernel<InT, LA, LB, B, BK>), grid, block, 0, stream, g, s);
+            return launchStatus();
+        }
+
+        // 16-wide blocks walk K in steps of 128 (v_mfma_scale_f32_16x16x128_f8f6f4), 32-wide blocks in steps
+        // of 64 (32x32x64): K that is a multiple of 64 only needs m and n in whole 32-wide blocks.
+        template <typename InT, typename LA, typename LB>
+        int pickBlock(GemmArgs const& g, MxScales const& s, hipStream_t stream)
+        {
+            if(g.m % 16u != 0u || g.n % 16u != 0u)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            if(g.k % 128u == 0u)
+                return launchOne<InT, LA, LB, 16, 128>(g, s, stream);
+            if(g.k % 64u == 0u && g.m % 32u == 0u && g.n % 32u == 0u)
+                return launchOne<InT, LA, LB, 32, 64>(g, s, stream);
+            return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+        }
+
+        template <typename InT>
+        int pickLayout(int layoutA, int layoutB, GemmArgs const& g, MxScales const& s, hipStream_t stream)
+        {
+            const bool aRow = layoutA == ROCWMMA_AMD_ROW_MAJOR;
+            const bool bRow = layoutB == ROCWMMA_AMD_ROW_MAJOR;
+            if(aRow && !bRow)
+                return pickBlock<InT, row_major, col_major>(g, s, stream);
+            if(aRow && bRow)
+                return pickBlock<InT, row_major, row_major>(g, s, stream);
+            if(!aRow && !bRow)
+                return pickBlock<InT, col_major, col_major>(g, s, stream);
+            return pickBlock<InT, col_major, row_major>(g, s, stream);
+        }
+
+        // One thread per (operand, group of 64 rows, pair of K stages, lane): the 8 bytes that lane loads.
+        // The first blocksA workgroups re-order A's scales, the others B's.
+        __global__ void __launch_bounds__(64) mxPackScalesKernel(MxScales s, uint32_t m, uint32_t n, uint32_t kBlocks, uint32_t pairs,
+                                                                 uint32_t blocksA, uint2* packedA, uint2* packedB)
+        {
+            const bool     isA     = blockIdx.x < blocksA;
+            const uint32_t item    = isA ? blockIdx.x : blockIdx.x - blocksA;
+            const uint8_t* scales  = isA ? s.a : s.b;
+            const uint32_t ld      = isA ? s.lda : s.ldb;
+            const uint32_t rows    = isA ? m : n;
+            const uint32_t lane    = threadIdx.x;
+            const uint32_t pair    = item % pairs;
+            const uint32_t group   = item / pairs;
+            uint32_t       word[2] = {0u, 0u};
+#pragma unroll
+            for(uint32_t blk = 0; blk < 4u; ++blk)
+#pragma unroll
+                for(uint32_t st = 0; st < 2u; ++st)
+                {
+                    const uint32_t row = group * 64u + blk * 16u + lane % 16u;
+                    const uint32_t kb  = (pair * 2u + st) * 4u + lane / 16u;
+                    // (rows and K blocks beyond the operand: never multiplied with anything stored)
+                    const uint32_t e   = (row < rows && kb < kBlocks) ? scales[static_cast<size_t>(row) * ld + kb] : 127u;
+                    word[blk / 2u] |= e << (8u * ((blk % 2u) * 2u + st));
+                }
+            (isA ? packedA : packedB)[static_cast<size_t>(item) * 64u + lane] = make_uint2(word[0], word[1]);
+        }
+    } // namespace
+
+    int launchMxPackScales(MxScales const& s, uint32_t m, uint32_t n, uint32_t k, void* packedA, void* packedB, hipStream_t stream)
+    {
+        const uint32_t pairs   = (k + 255u) / 256u;
+        const uint32_t blocksA = ((m + 63u) / 64u) * pairs;
+        const uint32_t blocksB = ((n + 63u) / 64u) * pairs;
+        hipLaunchKernelGGL(mxPackScalesKernel, dim3(blocksA + blocksB), dim3(64), 0, stream, s, m, n, k / 32u, pairs, blocksA,
+                           static_cast<uint2*>(packedA), static_cast<uint2*>(packedB));
+        return launchStatus();
+    }
+
+    int launchGemmMxWaveTile(int dtypeIn, int layoutA, int layoutB, GemmArgs const& g, MxScales const& s, hipStream_t stream)
+    {
+        if(static_cast<uint64_t>(g.lda) * 256u >= (1ull << 32) || static_cast<uint64_t>(g.ldb) * 256u >= (1ull << 32))
+            return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+        if(dtypeIn == ROCWMMA_AMD_E4M3)
+            return pickLayout<float8_t>(layoutA, layoutB, g, s, stream);
+        if(dtypeIn == ROCWMMA_AMD_E5M2)
+            return pickLayout<bfloat8_t>(layoutA, layoutB, g, s, stream);
+        return ROCWMMA_AMD_UNSUPPORTED_TYPE;
+    }
+
+} // namespace rocwmma_amd

@@ -32,6 +32,7 @@ namespace rocwmma_amd
             I8_32x32x32,
             F8_16x16x128,
             F8_32x32x64,
+            F8_16x16x128_SCALED, // v_mfma_scale_f32_16x16x128_f8f6f4 with per-lane block scales
         };
 
         // flops (or integer ops) of one instruction of the shape
@@ -50,6 +51,7 @@ namespace rocwmma_amd
             case I8_32x32x32:
                 return 2.0 * 32 * 32 * 32;
             case F8_16x16x128:
+            case F8_16x16x128_SCALED:
                 return 2.0 * 16 * 16 * 128;
             default:
                 return 2.0 * 32 * 32 * 64;
@@ -70,7 +72,7 @@ namespace rocwmma_amd
         __global__ void __launch_bounds__(256) mfmaCeilingKernel(const uint32_t* operands, float* out, uint32_t trips)
         {
             // 16 bytes (four dwords) per lane and operand for the 16-bit and int8 shapes, 32 bytes for fp8
-            constexpr bool     Fp8     = S == F8_16x16x128 || S == F8_32x32x64;
+            constexpr bool     Fp8     = S == F8_16x16x128 || S == F8_32x32x64 || S == F8_16x16x128_SCALED;
             constexpr bool     Wide    = S == F16_32x32x16 || S == BF16_32x32x16 || S == I8_32x32x32 || S == F8_32x32x64;
             constexpr bool     Integer = S == I8_16x16x64 || S == I8_32x32x32;
             constexpr uint32_t Words   = Fp8 ? 8u : 4u;
@@ -126,6 +128,14 @@ namespace rocwmma_amd
                             ROCWMMA_AMD_MFMA("v_mfma_f32_16x16x32_bf16", acc[q], ra, rb);
                         else if constexpr(S == I8_16x16x64)
                             ROCWMMA_AMD_MFMA("v_mfma_i32_16x16x64_i8", acc[q], ra, rb);
+                        else if constexpr(S == F8_16x16x128_SCALED)
+                        {
+#if defined(__HIP_DEVICE_COMPILE__)
+                            // scales near one (E8M0 124..131), different per lane and operand set
+                            acc[q] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ra, rb, acc[q], 0, 0, 0, 124 + (ra[0] & 7), 0,
+                                                                                     124 + (rb[0] & 7));
+#endif
+                        }
                         else
                             ROCWMMA_AMD_MFMA("v_mfma_f32_16x16x128_f8f6f4", acc[q], ra, rb);
                     }
@@ -152,7 +162,7 @@ namespace rocwmma_amd
     int benchMfmaCeiling(int shape, uint32_t trips, uint32_t wavesPerSimd, const void* operands, float* out, double* ops,
                          hipStream_t stream)
     {
-        if(shape < F16_16x16x32 || shape > F8_32x32x64 || trips == 0u || wavesPerSimd == 0u || wavesPerSimd > 2u)
+        if(shape < F16_16x16x32 || shape > F8_16x16x128_SCALED || trips == 0u || wavesPerSimd == 0u || wavesPerSimd > 2u)
             return ROCWMMA_AMD_INVALID_ARGUMENT;
         const uint32_t workgroups = computeUnits() * wavesPerSimd;
         if(ops)
@@ -174,6 +184,8 @@ namespace rocwmma_amd
             return launchShape<I8_32x32x32>(src, out, trips, workgroups, stream);
         case F8_16x16x128:
             return launchShape<F8_16x16x128>(src, out, trips, workgroups, stream);
+        case F8_16x16x128_SCALED:
+            return launchShape<F8_16x16x128_SCALED>(src, out, trips, workgroups, stream);
         default:
             return launchShape<F8_32x32x64>(src, out, trips, workgroups, stream);
         }

@@ -111,10 +111,10 @@ int main()
     checkInput<16, 32, 16, PackClass::Int8>("i8 16x32 t16", 8); // 16x16x32
     checkInput<32, 32, 32, PackClass::Int8>("i8 32x32 t32", 16); // 32x32x32
     checkInput<32, 16, 32, PackClass::Int8>("i8 32x16 t32", 8);
-    checkInput<16, 128, 16, PackClass::Fp8>("f8 16x128 t16", 32); // 16x16x128
+    checkInput<16, 128, 16, PackClass::Fp8>("f8 16x128 t16", 16); // 16x16x128: two 16-byte runs per lane
     checkInput<16, 64, 16, PackClass::Fp8>("f8 16x64 t16", 8); // 2 x 16x16x32 (no 16-byte fp8 operand)
     checkInput<16, 32, 16, PackClass::Fp8>("f8 16x32 t16", 8);
-    checkInput<32, 64, 32, PackClass::Fp8>("f8 32x64 t32", 32); // 32x32x64
+    checkInput<32, 64, 32, PackClass::Fp8>("f8 32x64 t32", 16); // 32x32x64: two 16-byte runs per lane
     checkInput<32, 32, 32, PackClass::Fp8>("f8 32x32 t32", 8);
     checkInput<32, 16, 32, PackClass::Fp8>("f8 32x16 t32", 8);
     checkInput<16, 16, 16, PackClass::Bits32>("f32 16x16 t16", 1); // 16x16x4

@@ -1,0 +1,152 @@
+"""Block-scaled (MX) fp8 GEMM on the GPU against the CPU oracle's restatement of the OCP definition,
+on the same seeded bits.  Bar: fp8 <= 1e-2 in the reference's compareEqual metric; patterns whose
+partial sums are exact (small integers times powers of two) must match bit for bit."""
+import numpy as np
+import pytest
+
+import oracle as orc
+import rocwmma_amd as rw
+from util import CM, RM, exact_int_bits, to_device, to_host, uniform_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def run_mx(dtype, la, lb, lc, m, n, k, a, sa, b, sb, c, alpha, beta, workspace):
+    import torch
+
+    d = to_device(np.full(m * n, np.nan, dtype=np.float32))
+    ws = None
+    if workspace:
+        ws = torch.empty(rw.gemm_mx_workspace_size(m, n, k), dtype=torch.uint8, device="cuda")
+    rw.gemm_mx(dtype, la, lb, lc, m, n, k, to_device(a), to_device(sa), to_device(b), to_device(sb),
+               None if c is None else to_device(c), d, alpha, beta, workspace=ws)
+    torch.cuda.synchronize()
+    return to_host(d, np.float32)
+
+
+def scales(seed, rows, k, lo, hi):
+    return np.random.default_rng(seed).integers(lo, hi + 1, size=(rows, k // 32), dtype=np.uint8)
+
+
+def check(got, want, tol):
+    if tol == 0.0:
+        assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} elements differ"
+        return
+    err, inf, nan = orc.compare_equal(orc.F32, got, orc.F32, want)
+    assert not inf and not nan, (inf, nan)
+    assert err <= tol, f"max relative error {err} > {tol}"
+
+
+@pytest.mark.parametrize("workspace", [False, True])
+@pytest.mark.parametrize("la,lb", [(RM, CM), (CM, RM), (RM, RM), (CM, CM)])
+@pytest.mark.parametrize("dtype", [orc.E4M3, orc.E5M2])
+@pytest.mark.parametrize("m,n,k", [(48, 80, 384), (64, 96, 192), (256, 512, 512)])
+def test_exact_pattern_with_power_of_two_scales_is_bit_exact(dtype, la, lb, m, n, k, workspace):
+    """Elements 0, -1, -2 (the reference's device fill, test/device/common.hpp:204-219) and scales
+    1/2, 1, 2: every partial sum is an integer multiple of 1/4 below 2^24 of them, so any order of
+    accumulation gives the same bits.  A scale applied to the wrong block, row or operand does not."""
+    a = exact_int_bits(dtype, m, k, la)
+    b = exact_int_bits(dtype, k, n, lb)
+    sa, sb = scales(11, m, k, 126, 128), scales(12, n, k, 126, 128)
+    c = exact_int_bits(orc.F32, m, n, RM)
+    got = run_mx(dtype, la, lb, RM, m, n, k, a, sa, b, sb, c, 2.0, 3.0, workspace)
+    want = orc.gemm_mx(dtype, la, lb, RM, RM, m, n, k, a, sa, b, sb, c, 2.0, 3.0)
+    check(got, want, 0.0)
+
+
+@pytest.mark.parametrize("workspace", [False, True])
+@pytest.mark.parametrize("la,lb,lc", [(RM, CM, RM), (RM, CM, CM), (CM, RM, CM), (CM, CM, RM), (RM, RM, CM)])
+@pytest.mark.parametrize("dtype", [orc.E4M3, orc.E5M2])
+def test_random_operands_and_scales(dtype, la, lb, lc, workspace):
+    m, n, k = 256, 512, 640
+    a = uniform_bits(21, dtype, m * k)
+    b = uniform_bits(22, dtype, k * n)
+    sa, sb = scales(23, m, k, 124, 130), scales(24, n, k, 124, 130)
+    c = uniform_bits(25, orc.F32, m * n)
+    for beta in (0.0, -0.5):
+        got = run_mx(dtype, la, lb, lc, m, n, k, a, sa, b, sb, c if beta else None, 1.5, beta, workspace)
+        want = orc.gemm_mx(dtype, la, lb, lc, lc, m, n, k, a, sa, b, sb, c if beta else None, 1.5, beta)
+        check(got, want, 1e-2)
+
+
+@pytest.mark.parametrize("workspace", [False, True])
+def test_wide_range_of_scales_against_the_size_of_the_terms(workspace):
+    """Scales from 2^-7 to 2^7 per operand: a result is then a small difference of terms up to 2^14
+    times larger, and two float32 summations in different orders agree to a few ulp of the LARGEST
+    partial sums, not of the result.  So the error is measured against the sum of the terms'
+    magnitudes (float64).  Measured: 2^-16.2 of that sum, the same for both kernels (the matrix core
+    adds the 128 products of an instruction aligned to the largest of them and drops what falls
+    below its adder width); the bound of 2^-14 still catches any scale applied to the wrong block (a
+    factor of two on one block moves a result by about 1/20 of that sum)."""
+    m, n, k = 256, 256, 640
+    dtype = orc.E4M3
+    a = uniform_bits(61, dtype, m * k)
+    b = uniform_bits(62, dtype, k * n)
+    sa, sb = scales(63, m, k, 120, 134), scales(64, n, k, 120, 134)
+    got = run_mx(dtype, RM, CM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0, workspace).reshape(m, n).astype(np.float64)
+    af = orc.mx_dequantise(dtype, a, sa, RM, m, k).astype(np.float64)
+    bf = orc.mx_dequantise(dtype, b, sb, RM, n, k).astype(np.float64)
+    want = af @ bf.T
+    size = np.abs(af) @ np.abs(bf).T
+    assert np.max(np.abs(got - want) / size) < 2.0 ** -14
+
+
+def test_unit_scales_give_the_unscaled_gemm():
+    import torch
+
+    m, n, k = 256, 256, 1024
+    dtype = orc.E4M3
+    a = uniform_bits(31, dtype, m * k)
+    b = uniform_bits(32, dtype, k * n)
+    one_a = np.full((m, k // 32), 127, dtype=np.uint8)
+    one_b = np.full((n, k // 32), 127, dtype=np.uint8)
+    for workspace in (False, True):
+        got = run_mx(dtype, RM, CM, RM, m, n, k, a, one_a, b, one_b, None, 1.0, 0.0, workspace)
+        d = to_device(np.zeros(m * n, dtype=np.float32))
+        rw.gemm(dtype, orc.F32, RM, CM, RM, m, n, k, to_device(a), to_device(b), None, d, 1.0, 0.0)
+        torch.cuda.synchronize()
+        check(got, to_host(d, np.float32), 1e-5)
+
+
+def test_padded_leading_dimensions_of_the_scale_matrices():
+    import torch
+
+    m, n, k = 256, 256, 512
+    dtype = orc.E5M2
+    a = uniform_bits(41, dtype, m * k)
+    b = uniform_bits(42, dtype, k * n)
+    sa, sb = scales(43, m, k, 124, 130), scales(44, n, k, 124, 130)
+    want = orc.gemm_mx(dtype, RM, CM, RM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0)
+    pad_a = np.full((m, k // 32 + 5), 255, dtype=np.uint8)  # (NaN scales in the padding: never read)
+    pad_b = np.full((n, k // 32 + 3), 255, dtype=np.uint8)
+    pad_a[:, :k // 32] = sa
+    pad_b[:, :k // 32] = sb
+    for workspace in (False, True):
+        d = to_device(np.full(m * n, np.nan, dtype=np.float32))
+        ws = torch.empty(rw.gemm_mx_workspace_size(m, n, k), dtype=torch.uint8, device="cuda") if workspace else None
+        rw.gemm_mx(dtype, RM, CM, RM, m, n, k, to_device(a), to_device(pad_a), to_device(b), to_device(pad_b), None, d,
+                   1.0, 0.0, workspace=ws, ld_scale_a=k // 32 + 5, ld_scale_b=k // 32 + 3)
+        torch.cuda.synchronize()
+        check(to_host(d, np.float32), want, 1e-2)
+
+
+def test_full_size_quantised_inference_shape_sampled_rows():
+    """4096 x 14336 x 4096 (the fp8 shape of the quantised-inference configuration) with block scales:
+    64 oracle rows and the row sums of every row against float64 sums of the dequantised operands."""
+    import torch
+
+    m, n, k = 4096, 14336, 4096
+    dtype = orc.E4M3
+    a = uniform_bits(51, dtype, m * k)
+    b = uniform_bits(52, dtype, k * n)
+    sa, sb = scales(53, m, k, 124, 130), scales(54, n, k, 124, 130)
+    got = run_mx(dtype, RM, CM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0, True).reshape(m, n)
+    rows = np.random.default_rng(55).choice(m, size=64, replace=False).astype(np.uint32)
+    want = orc.gemm_mx(dtype, RM, CM, RM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0, rows=np.sort(rows)).reshape(m, n)
+    check(np.ascontiguousarray(got[np.sort(rows)]), np.ascontiguousarray(want[np.sort(rows)]), 1e-2)
+    # every row and column takes part: D summed over columns = A_deq * (B_deq summed over columns)
+    af = orc.mx_dequantise(dtype, a, sa, RM, m, k).astype(np.float64)
+    bsum = orc.mx_dequantise(dtype, b, sb, RM, n, k).astype(np.float64).sum(axis=0)
+    ref = af @ bsum
+    size = np.abs(af) @ np.abs(orc.mx_dequantise(dtype, b, sb, RM, n, k).astype(np.float64)).sum(axis=0)
+    assert np.max(np.abs(got.astype(np.float64).sum(axis=1) - ref) / size) < 1e-5

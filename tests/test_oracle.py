@@ -248,6 +248,79 @@ def test_gemm_accumulation_order_is_sequential_f32():
 
 
 # ---------------------------------------------------------------- compare metric
+# ---- block-scaled GEMM (the reference has none: pinned on the OCP definition) ------------------
+def _mx_case(seed, m, n, k, dtype, lo=120, hi=134):
+    rng = np.random.default_rng(seed)
+    a = orc.encode(dtype, rng.uniform(-1, 1, m * k).astype(np.float32))
+    b = orc.encode(dtype, rng.uniform(-1, 1, k * n).astype(np.float32))
+    sa = rng.integers(lo, hi + 1, size=(m, k // 32), dtype=np.uint8)
+    sb = rng.integers(lo, hi + 1, size=(n, k // 32), dtype=np.uint8)
+    return a, sa, b, sb
+
+
+def test_mx_scale_decoding():
+    """E8M0: 2^(e - 127); 127 is one, 0 the smallest (a float32 subnormal), 255 NaN."""
+    v = orc.mx_scale_values(np.array([0, 1, 126, 127, 128, 254, 255], dtype=np.uint8))
+    assert v[3] == 1.0 and v[2] == 0.5 and v[4] == 2.0
+    assert v[0] == np.float32(2.0) ** -127 and v[1] == np.float32(2.0) ** -126
+    assert v[5] == np.float32(2.0) ** 127 and np.isnan(v[6])
+
+
+@pytest.mark.parametrize("dtype", [orc.E4M3, orc.E5M2])
+def test_mx_gemm_with_unit_scales_is_the_unscaled_gemm(dtype):
+    m, n, k = 48, 32, 128
+    a, _, b, _ = _mx_case(1, m, n, k, dtype)
+    one = np.full((max(m, n), k // 32), 127, dtype=np.uint8)
+    for la, lb in [(orc.ROW_MAJOR, orc.COL_MAJOR), (orc.COL_MAJOR, orc.ROW_MAJOR)]:
+        got = orc.gemm_mx(dtype, la, lb, 0, 0, m, n, k, a, one[:m], b, one[:n], None, 1.0, 0.0)
+        want = orc.gemm(dtype, orc.F32, la, lb, 0, 0, m, n, k, a, b, None, 1.0, 0.0)
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (0, 0), (1, 1)])
+def test_mx_gemm_against_float64_block_formula(la, lb):
+    """Independent statement of the definition: per K block, scaleA * scaleB * (sum of element
+    products), summed over blocks, in float64.  A swapped scale matrix, a scale applied to the wrong
+    block or operand, or a wrong bias all fail this."""
+    m, n, k = 32, 48, 256
+    dtype = orc.E4M3
+    a, sa, b, sb = _mx_case(2, m, n, k, dtype)
+    c = np.random.default_rng(3).uniform(-1, 1, m * n).astype(np.float32)
+    got = orc.gemm_mx(dtype, la, lb, 0, 0, m, n, k, a, sa, b, sb, c, 2.0, -0.5).reshape(m, n).astype(np.float64)
+    A = orc.decode(dtype, a).astype(np.float64).reshape((m, k) if la == 0 else (k, m))
+    A = A if la == 0 else A.T
+    B = orc.decode(dtype, b).astype(np.float64).reshape((k, n) if lb == 0 else (n, k))
+    B = B if lb == 0 else B.T  # k x n
+    want = np.zeros((m, n))
+    size = np.zeros((m, n))  # sum of the terms' magnitudes: what float32 rounding errors scale with
+    for kb in range(k // 32):
+        part = A[:, kb * 32:(kb + 1) * 32] @ B[kb * 32:(kb + 1) * 32, :]
+        mag = np.abs(A[:, kb * 32:(kb + 1) * 32]) @ np.abs(B[kb * 32:(kb + 1) * 32, :])
+        fa = 2.0 ** (sa[:, kb].astype(np.float64) - 127)
+        fb = 2.0 ** (sb[:, kb].astype(np.float64) - 127)
+        want += part * fa[:, None] * fb[None, :]
+        size += mag * fa[:, None] * fb[None, :]
+    want = 2.0 * want - 0.5 * c.reshape(m, n)
+    # (float32 summation of k terms: a few ulp of the running sum per term, far below k * 2^-24 * size)
+    assert np.max(np.abs(got - want) / (2.0 * size + 1.0)) < 2e-6
+
+
+def test_mx_gemm_scales_are_exact_powers_of_two():
+    """Raising every scale of A by one doubles the product exactly; raising one K block's scale of
+    one row changes that row only."""
+    m, n, k = 16, 16, 128
+    dtype = orc.E5M2
+    a, sa, b, sb = _mx_case(4, m, n, k, dtype)
+    base = orc.gemm_mx(dtype, 0, 1, 0, 0, m, n, k, a, sa, b, sb, None, 1.0, 0.0)
+    twice = orc.gemm_mx(dtype, 0, 1, 0, 0, m, n, k, a, sa + 1, b, sb, None, 1.0, 0.0)
+    assert np.array_equal(twice, 2.0 * base)
+    sa2 = sa.copy()
+    sa2[5, 2] += 3
+    one = orc.gemm_mx(dtype, 0, 1, 0, 0, m, n, k, a, sa2, b, sb, None, 1.0, 0.0).reshape(m, n)
+    differs = np.any(one != base.reshape(m, n), axis=1)
+    assert differs[5] and differs.sum() == 1
+
+
 def test_compare_equal_metric():
     a = np.array([1.0, 2.0, -3.0, 0.0], dtype=np.float32)
     b = np.array([1.0, 2.5, -3.0, 0.0], dtype=np.float32)
