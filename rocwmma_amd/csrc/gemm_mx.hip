@@ -125,16 +125,20 @@ namespace rocwmma_amd
         }
 
         // One thread per (operand, group of 64 rows, pair of K stages, lane): the 8 bytes that lane loads.
-        // The first blocksA workgroups re-order A's scales, the others B's.
-        __global__ void __launch_bounds__(64) mxPackScalesKernel(MxScales s, uint32_t m, uint32_t n, uint32_t kBlocks, uint32_t pairs,
-                                                                 uint32_t blocksA, uint2* packedA, uint2* packedB)
+        // Items 0 .. blocksA - 1 re-order A's scales, the others B's; a workgroup of four waves takes four
+        // consecutive items.
+        __global__ void __launch_bounds__(256) mxPackScalesKernel(MxScales s, uint32_t m, uint32_t n, uint32_t kBlocks, uint32_t pairs,
+                                                                  uint32_t blocksA, uint32_t blocksB, uint2* packedA, uint2* packedB)
         {
-            const bool     isA     = blockIdx.x < blocksA;
-            const uint32_t item    = isA ? blockIdx.x : blockIdx.x - blocksA;
+            const uint32_t id = blockIdx.x * 4u + threadIdx.x / 64u;
+            if(id >= blocksA + blocksB)
+                return;
+            const bool     isA     = id < blocksA;
+            const uint32_t item    = isA ? id : id - blocksA;
             const uint8_t* scales  = isA ? s.a : s.b;
             const uint32_t ld      = isA ? s.lda : s.ldb;
             const uint32_t rows    = isA ? m : n;
-            const uint32_t lane    = threadIdx.x;
+            const uint32_t lane    = threadIdx.x % 64u;
             const uint32_t pair    = item % pairs;
             const uint32_t group   = item / pairs;
             uint32_t       word[2] = {0u, 0u};
@@ -158,8 +162,8 @@ namespace rocwmma_amd
         const uint32_t pairs   = (k + 255u) / 256u;
         const uint32_t blocksA = ((m + 63u) / 64u) * pairs;
         const uint32_t blocksB = ((n + 63u) / 64u) * pairs;
-        hipLaunchKernelGGL(mxPackScalesKernel, dim3(blocksA + blocksB), dim3(64), 0, stream, s, m, n, k / 32u, pairs, blocksA,
-                           static_cast<uint2*>(packedA), static_cast<uint2*>(packedB));
+        hipLaunchKernelGGL(mxPackScalesKernel, dim3((blocksA + blocksB + 3u) / 4u), dim3(256), 0, stream, s, m, n, k / 32u, pairs,
+                           blocksA, blocksB, static_cast<uint2*>(packedA), static_cast<uint2*>(packedB));
         return launchStatus();
     }
 
