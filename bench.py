@@ -500,6 +500,31 @@ def run_extras(rw, torch, dev, gen, only=None):
                             "32x32x16 blocks, 128 x 128 macro tile, single LDS buffer"}
         del Ap, Bp, Cp, Dp
 
+    # the headline f16 A-row / B-col GEMM with the fused epilogue (bias per column, GELU) against the same
+    # GEMM without it: what the epilogue costs when it rides on the accumulators
+    if wanted("gemm_f16_rc_8192_bias_gelu"):
+        sz = 8192
+        Af = (torch.rand(sz * sz, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        Bf_ = (torch.rand(sz * sz, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        Cf = torch.rand(sz * sz, device=dev, generator=gen) * 2 - 1
+        Df = torch.empty(sz * sz, device=dev)
+        bias = torch.rand(sz, device=dev, generator=gen) * 2 - 1
+
+        def fn_fused():
+            rw.gemm_bias_act(rw.F16, rw.F32, RM, CM, RM, sz, sz, sz, Af, Bf_, Cf, Df, 1.0, 1.0, bias, rw.ACT_GELU)
+
+        def fn_plain():
+            rw.gemm(rw.F16, rw.F32, RM, CM, RM, sz, sz, sz, Af, Bf_, Cf, Df, 1.0, 1.0)
+
+        fn_fused()
+        ms = event_ms(fn_fused, 20, torch)
+        fn_plain()
+        ms_plain = event_ms(fn_plain, 20, torch)
+        out["gemm_f16_rc_8192_bias_gelu"] = {"ms": round(ms, 4), "tflops": round(2.0 * sz ** 3 / ms / 1e9, 1),
+                                             "ms_without_epilogue": round(ms_plain, 4),
+                                             "note": "D = gelu(A*B + C + bias[column]), f32 C/D"}
+        del Af, Bf_, Cf, Df, bias
+
     # config 3: N = 14336, K = 4096, M in {16, 128, 4096}; int8 and e4m3, A row / B col.  The weight
     # matrix (56 MiB) would stay in the 256 MiB Infinity Cache between launches, so the timed loop
     # rotates over 5 weight buffers (280 MiB); the cache-resident time is reported beside it.

@@ -70,6 +70,14 @@ typedef enum rocwmma_amd_gemm_algo
                                         fall back to 128 x 128 tiles below half occupancy)  */
 } rocwmma_amd_gemm_algo;
 
+/* Activation applied by rocwmma_amd_gemm_bias_act. */
+typedef enum rocwmma_amd_activation
+{
+    ROCWMMA_AMD_ACT_NONE = 0,
+    ROCWMMA_AMD_ACT_RELU = 1, /* max(x, 0)                          */
+    ROCWMMA_AMD_ACT_GELU = 2  /* x * (1 + erf(x / sqrt(2))) / 2     */
+} rocwmma_amd_activation;
+
 /* Library identification: returns 10000*major + 100*minor + patch. */
 int rocwmma_amd_version(void);
 
@@ -230,6 +238,42 @@ int rocwmma_amd_gemm_streamk_static(int         dtype_in,
                                     float       alpha,
                                     float       beta,
                                     void*       stream);
+
+/*
+ * GEMM with a fused epilogue:  D = act(alpha * A * B + beta * C + bias[j])  for column j of D.
+ *
+ * The reference's GEMM kernels end with D = alpha * acc + beta * C on fragments
+ * (samples/perf_hgemm.cpp:683-713) and leave bias and activation to further kernels, i.e. to two more
+ * passes over D; here they are applied to the accumulators on their way out.  Arguments and limits are
+ * those of rocwmma_amd_gemm with
+ *   dtype_in / dtype_out : the float triples only (F16, BF16, E4M3, E5M2 inputs; F32, or F16 / BF16 with
+ *                          inputs of the same type); the sum and the activation are computed in f32;
+ *   bias       : n floats (device memory, 16-byte aligned), or NULL for none;
+ *   activation : a rocwmma_amd_activation.
+ * Row-major C/D with k in whole 64-byte stages (at least three) runs on the blocked kernel, everything
+ * else one block per wave.
+ */
+int rocwmma_amd_gemm_bias_act(int          dtype_in,
+                              int          dtype_out,
+                              int          layout_a,
+                              int          layout_b,
+                              int          layout_c,
+                              uint32_t     m,
+                              uint32_t     n,
+                              uint32_t     k,
+                              const void*  a,
+                              uint32_t     lda,
+                              const void*  b,
+                              uint32_t     ldb,
+                              const void*  c,
+                              uint32_t     ldc,
+                              void*        d,
+                              uint32_t     ldd,
+                              float        alpha,
+                              float        beta,
+                              const float* bias,
+                              int          activation,
+                              void*        stream);
 
 /*
  * Block-scaled ("microscaled", MX) fp8 GEMM:

@@ -150,6 +150,35 @@ def gemm_mx(dtype_in, layA, layB, layC, layD, m, n, k, a, scale_a, b, scale_b, c
     return gemm(F32, F32, layA, layB, layC, layD, m, n, k, af, bf, c, alpha, beta, rows=rows)
 
 
+ACT_NONE, ACT_RELU, ACT_GELU = range(3)
+
+
+def gemm_bias_act(dtype_in, dtype_out, layA, layB, layC, m, n, k, a, b, c, alpha, beta, bias, activation, rows=None):
+    """D = act(alpha*A*B + beta*C + bias[column]).  The reference has no fused epilogue: this is
+    gemm_CPU (test/reference_impl.hpp:36-81) with a float32 result, followed by the bias and the
+    activation in float64 (ReLU: max(x, 0); GELU: x (1 + erf(x / sqrt 2)) / 2), rounded once to
+    `dtype_out`.  C and D share layC."""
+    from scipy.special import erf
+
+    cf = None if c is None else decode(dtype_out, c)
+    acc = gemm(dtype_in, F32, layA, layB, layC, layC, m, n, k, a, b, cf, alpha, beta, rows=rows).astype(np.float64)
+    acc = acc.reshape((m, n) if layC == ROW_MAJOR else (n, m))
+    if bias is not None:
+        bv = np.asarray(bias, dtype=np.float32).astype(np.float64)
+        acc = acc + (bv[None, :] if layC == ROW_MAJOR else bv[:, None])
+    if activation == ACT_RELU:
+        acc = np.maximum(acc, 0.0)
+    elif activation == ACT_GELU:
+        acc = 0.5 * acc * (1.0 + erf(acc / np.sqrt(2.0)))
+    out = encode(dtype_out, acc.astype(np.float32).reshape(-1))
+    if rows is not None:  # rows that were not computed stay zero, as in gemm()
+        keep = np.zeros(m, dtype=bool)
+        keep[np.asarray(rows)] = True
+        mask = np.broadcast_to(keep[:, None] if layC == ROW_MAJOR else keep[None, :], acc.shape).reshape(-1)
+        out = np.where(mask, out, np.zeros_like(out))
+    return out
+
+
 def dlrm_fwd(inp, m, k, batch):
     """dlrm_fwd_CPU (test/reference_impl.hpp:83-119) on f16 bit patterns."""
     inp = np.ascontiguousarray(inp, dtype=np.uint16).reshape(-1)

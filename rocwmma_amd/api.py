@@ -19,8 +19,9 @@ EXPORTS = [
     "rocwmma_amd_version", "rocwmma_amd_status_string", "rocwmma_amd_device_info", "rocwmma_amd_gemm",
     "rocwmma_amd_gemm_ex", "rocwmma_amd_gemv", "rocwmma_amd_dlrm_fwd", "rocwmma_amd_dlrm_bwd",
     "rocwmma_amd_gemm_streamk", "rocwmma_amd_gemm_streamk_workspace_size", "rocwmma_amd_gemm_streamk_static",
-    "rocwmma_amd_gemm_mx", "rocwmma_amd_gemm_mx_workspace_size",
+    "rocwmma_amd_gemm_mx", "rocwmma_amd_gemm_mx_workspace_size", "rocwmma_amd_gemm_bias_act",
 ]
+ACT_NONE, ACT_RELU, ACT_GELU = range(3)
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
 _AUX_LIB_NAME = "librocwmma_amd_aux.so"
 AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_bench_mfma_ceiling",
@@ -66,6 +67,8 @@ def library():
         L.rocwmma_amd_gemm_streamk.restype = i
         L.rocwmma_amd_gemm_streamk_static.argtypes = gemm_args
         L.rocwmma_amd_gemm_streamk_static.restype = i
+        L.rocwmma_amd_gemm_bias_act.argtypes = gemm_args[:-1] + [vp, i, vp]
+        L.rocwmma_amd_gemm_bias_act.restype = i
         L.rocwmma_amd_gemm_mx.argtypes = [i, i, i, i, u, u, u, vp, u, vp, u, vp, u, vp, u, vp, u, vp, u, f, f, vp, ctypes.c_size_t, vp]
         L.rocwmma_amd_gemm_mx_workspace_size.argtypes = [u, u, u]
         L.rocwmma_amd_gemm_mx_workspace_size.restype = ctypes.c_size_t
@@ -201,6 +204,22 @@ def gemm_streamk_static(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n,
     rc = library().rocwmma_amd_gemm_streamk_static(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, _ptr(a),
                                                    lda, _ptr(b), ldb, _ptr(c), ldc, _ptr(d), ldd, alpha, beta, _stream())
     _check(rc, "gemm_streamk_static")
+    return d
+
+
+def gemm_bias_act(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, b, c, d, alpha, beta, bias, activation,
+                  lda=None, ldb=None, ldc=None, ldd=None):
+    """rocwmma_amd_gemm_bias_act on device tensors: D = act(alpha*A*B + beta*C + bias[column]);
+    `bias` is a float32 device tensor of n values or None."""
+    lda = lda if lda is not None else (k if layout_a == ROW_MAJOR else m)
+    ldb = ldb if ldb is not None else (n if layout_b == ROW_MAJOR else k)
+    nat = n if layout_c == ROW_MAJOR else m
+    ldc = ldc if ldc is not None else nat
+    ldd = ldd if ldd is not None else nat
+    rc = library().rocwmma_amd_gemm_bias_act(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, _ptr(a), lda,
+                                             _ptr(b), ldb, _ptr(c), ldc, _ptr(d), ldd, alpha, beta, _ptr(bias), activation,
+                                             _stream())
+    _check(rc, "gemm_bias_act")
     return d
 
 

@@ -285,6 +285,46 @@ int rocwmma_amd_gemm_streamk_static(int         dtype_in,
     return launchGemmStreamKStatic(dtype_in, dtype_out, la, lb, args, asStream(stream));
 }
 
+int rocwmma_amd_gemm_bias_act(int          dtype_in,
+                              int          dtype_out,
+                              int          layout_a,
+                              int          layout_b,
+                              int          layout_c,
+                              uint32_t     m,
+                              uint32_t     n,
+                              uint32_t     k,
+                              const void*  a,
+                              uint32_t     lda,
+                              const void*  b,
+                              uint32_t     ldb,
+                              const void*  c,
+                              uint32_t     ldc,
+                              void*        d,
+                              uint32_t     ldd,
+                              float        alpha,
+                              float        beta,
+                              const float* bias,
+                              int          activation,
+                              void*        stream)
+{
+    int rc = checkGemm(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, lda, b, ldb, c, ldc, d, ldd, alpha, beta);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(dtype_in == ROCWMMA_AMD_I8 || dtype_in == ROCWMMA_AMD_F32)
+        return ROCWMMA_AMD_UNSUPPORTED_TYPE;
+    if(activation != ROCWMMA_AMD_ACT_NONE && activation != ROCWMMA_AMD_ACT_RELU && activation != ROCWMMA_AMD_ACT_GELU)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(bias && !aligned16(bias))
+        return ROCWMMA_AMD_BAD_ALIGNMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    GemmArgs args{m, n, k, a, b, c, d, lda, ldb, c ? ldc : ldd, ldd, alpha, beta, layout_c, bias, activation};
+    rc = launchGemmBlockedFused(dtype_in, dtype_out, layout_a, layout_b, args, asStream(stream));
+    if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE && rc != ROCWMMA_AMD_UNSUPPORTED_TYPE)
+        return rc;
+    return launchGemmWaveTile(dtype_in, dtype_out, layout_a, layout_b, args, asStream(stream));
+}
+
 size_t rocwmma_amd_gemm_mx_workspace_size(uint32_t m, uint32_t n, uint32_t k)
 {
     return mxPackedScaleBytes(m, n, k);

@@ -79,7 +79,28 @@ namespace rocwmma_amd
         uint32_t    lda, ldb, ldc, ldd;
         float       alpha, beta;
         int         layoutC;
+        // fused epilogue (rocwmma_amd_gemm_bias_act): D = act(alpha * A * B + beta * C + bias[column])
+        const float* bias       = nullptr; // one value per column of D, or nullptr
+        int          activation = ROCWMMA_AMD_ACT_NONE;
     };
+
+    ROCWMMA_DEVICE ROCWMMA_INLINE float applyActivation(float v, int activation)
+    {
+        if(activation == ROCWMMA_AMD_ACT_RELU)
+            return v > 0.0f ? v : 0.0f;
+        if(activation == ROCWMMA_AMD_ACT_GELU)
+        {
+            // x * Phi(x) with Phi(x) = erfc(-x / sqrt 2) / 2 and, for z >= 0, erfc(z) = (a1 t + ... + a5 t^5)
+            // exp(-z^2), t = 1 / (1 + p z) (Abramowitz & Stegun 7.1.26, absolute error below 1.5e-7): one
+            // reciprocal, one exponential and a dozen multiply-adds, a third of the library erff.
+            const float z    = fabsf(v) * 0.70710678118654752f;
+            const float t    = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
+            const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+            const float half = 0.5f * poly * __builtin_amdgcn_exp2f(-1.4426950408889634f * z * z);
+            return v * (v >= 0.0f ? 1.0f - half : half);
+        }
+        return v;
+    }
 
     // Block scales of a microscaled GEMM: one E8M0 byte per 32 elements along K of every row of A
     // (a: m x k/32, leading dimension lda) and every column of B (b: n x k/32, leading dimension ldb).
@@ -127,6 +148,9 @@ namespace rocwmma_amd
     // The blocked kernel on packed scales: row-major A, col-major B, row-major C/D, m and n multiples
     // of 256, k a multiple of 128.
     int launchGemmMxBlocked(int dtypeIn, GemmArgs const& args, const void* packedA, const void* packedB, hipStream_t stream);
+
+    // The blocked kernel with the fused epilogue (float types, row-major C/D; args.bias / args.activation)
+    int launchGemmBlockedFused(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
 
     // Block-scaled fp8 / bf8 GEMM (f32 C/D): one block per wave, every layout pair
     int launchGemmMxWaveTile(int dtypeIn, int layoutA, int layoutB, GemmArgs const& args, MxScales const& scales, hipStream_t stream);

@@ -1,6 +1,7 @@
-// Blocked GEMM for gfx950, one macro tile per workgroup: kernel, tile ladder and dispatch.  The device
-// side (configuration, LDS pipeline, epilogue) is in gemm_blocked_core.hpp.
-#include "gemm_blocked_core.hpp"
+// Blocked GEMM for gfx950, one macro tile per workgroup: tile ladder and dispatch.  The device side
+// (configuration, LDS pipeline, epilogue) is in gemm_blocked_core.hpp, the kernels and launch helpers in
+// gemm_blocked_launch.hpp.
+#include "gemm_blocked_launch.hpp"
 
 using namespace rocwmma;
 
@@ -8,174 +9,6 @@ namespace rocwmma_amd
 {
     namespace
     {
-        template <typename Cfg>
-        __global__ void __launch_bounds__(Cfg::Threads) __attribute__((amdgpu_waves_per_eu(Cfg::WavesPerSimd, Cfg::WavesPerSimd)))
-        gemmBlockedKernel(uint32_t                   m,
-                          uint32_t                   n,
-                          uint32_t                   k,
-                          typename Cfg::InT const*   a,
-                          typename Cfg::InT const*   b,
-                          typename Cfg::OutT const*  c,
-                          typename Cfg::OutT*        d,
-                          uint32_t                   lda,
-                          uint32_t                   ldb,
-                          uint32_t                   ldc,
-                          uint32_t                   ldd,
-                          typename Cfg::CompT        alpha,
-                          typename Cfg::CompT        beta,
-                          MxPacked                   mx) // block scales (Scaled configurations only)
-        {
-            uint32_t tm, tn;
-            tileOfWorkgroup(blockIdx.x, ceilDiv(m, Cfg::MacroM), ceilDiv(n, Cfg::MacroN), tm, tn);
-            gemmTile<Cfg>(tm, tn, 0u, k / Cfg::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{}, mx);
-        }
-
-        // Two tilings in one launch: the first `fullTiles` workgroups run Full tiles, the others the two
-        // halves (same rows, half the columns each) of the remaining Full tiles, in the same tile order.
-        // Used when the Full tiles alone would leave the last round of workgroups at most half occupied.
-        template <typename Full, typename Half>
-        __global__ void __launch_bounds__(Full::Threads) __attribute__((amdgpu_waves_per_eu(Full::WavesPerSimd, Full::WavesPerSimd)))
-        gemmBlockedSplitTailKernel(uint32_t                   m,
-                                   uint32_t                   n,
-                                   uint32_t                   k,
-                                   typename Full::InT const*  a,
-                                   typename Full::InT const*  b,
-                                   typename Full::OutT const* c,
-                                   typename Full::OutT*       d,
-                                   uint32_t                   lda,
-                                   uint32_t                   ldb,
-                                   uint32_t                   ldc,
-                                   uint32_t                   ldd,
-                                   typename Full::CompT       alpha,
-                                   typename Full::CompT       beta,
-                                   uint32_t                   fullTiles,
-                                   MxPacked                   mx)
-        {
-            // (The half tiles go last.  Running half of them first, on half of the compute units of every
-            // XCD or on XCDs 0-3, so that one half of the device writes its results while the other is in
-            // its main loop, was 3-4 % slower either way.)
-            const uint32_t tilesM = m / Full::MacroM, tilesN = n / Full::MacroN;
-            uint32_t       tm, tn;
-            if(blockIdx.x < fullTiles)
-            {
-                tileOfWorkgroup(blockIdx.x, tilesM, tilesN, tm, tn);
-                gemmTile<Full>(tm, tn, 0u, k / Full::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha, beta, StreamKPart{}, mx);
-            }
-            else
-            {
-                const uint32_t j = blockIdx.x - fullTiles;
-                tileOfWorkgroup(fullTiles + j / 2u, tilesM, tilesN, tm, tn);
-                gemmTile<Half>(tm, 2u * tn + (j & 1u), 0u, k / Half::MacroK, m, n, k, a, b, c, d, lda, ldb, ldc, ldd, alpha,
-                               beta, StreamKPart{}, mx);
-            }
-        }
-
-        // Launches Full tiles with the tiles of the last round cut into Half tiles when that round would be
-        // at most half full: T = q * units + r tiles with 0 < r <= units / 2 would otherwise end with a round
-        // that occupies at most half of the compute units for the time of a whole tile (4096 x 14336: 896
-        // tiles on 256 units, 3.5 rounds; 6144^3: 2.25 rounds).
-        template <typename Full, typename Half>
-        int launchSplitTail(GemmArgs const& g, hipStream_t stream, MxPacked const& mx = MxPacked{})
-        {
-            static_assert(Full::MacroM == Half::MacroM && Full::MacroN == 2u * Half::MacroN && Full::MacroK == Half::MacroK
-                              && Full::Threads == Half::Threads && Full::Stages == Half::Stages
-                              && Full::WavesPerSimd == Half::WavesPerSimd && !Full::Edges && !Half::Edges,
-                          "half tiles: same rows, half the columns, same pipeline");
-            if(g.m % Full::MacroM != 0u || g.n % Full::MacroN != 0u || g.k % Full::MacroK != 0u
-               || g.k < (Full::Stages - 1u) * Full::MacroK)
-                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-            const uint32_t tilesM = g.m / Full::MacroM, tilesN = g.n / Full::MacroN, units = computeUnits();
-            const uint32_t total = tilesM * tilesN, rest = total % units;
-            if(total < units || rest == 0u || 2u * rest > units)
-                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-            {
-                const uint64_t spanA = static_cast<uint64_t>(g.lda) * sizeof(typename Full::InT)
-                                       * (Full::AKMajor ? Full::MacroM : Full::MacroK);
-                const uint64_t spanB = static_cast<uint64_t>(g.ldb) * sizeof(typename Full::InT)
-                                       * (Full::BKMajor ? Full::MacroN : Full::MacroK);
-                if(spanA >= 0x7FFF0000ull || spanB >= 0x7FFF0000ull)
-                    return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-            }
-            auto               kernel = gemmBlockedSplitTailKernel<Full, Half>;
-            constexpr uint32_t lds    = Full::LdsBytes > Half::LdsBytes ? Full::LdsBytes : Half::LdsBytes;
-            if(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   static_cast<int>(lds))
-               != hipSuccess)
-                return ROCWMMA_AMD_LAUNCH_FAILED;
-            const uint32_t fullTiles = total - rest;
-            hipLaunchKernelGGL(kernel, dim3(fullTiles + 2u * rest), dim3(Full::Threads), lds, stream, g.m, g.n, g.k,
-                               static_cast<typename Full::InT const*>(g.a), static_cast<typename Full::InT const*>(g.b),
-                               static_cast<typename Full::OutT const*>(g.c), static_cast<typename Full::OutT*>(g.d), g.lda,
-                               g.ldb, g.ldc, g.ldd, static_cast<typename Full::CompT>(g.alpha),
-                               static_cast<typename Full::CompT>(g.beta), fullTiles, mx);
-            return launchStatus();
-        }
-
-        template <typename Cfg>
-        int launchCfg(GemmArgs const& g, hipStream_t stream, MxPacked const& mx = MxPacked{})
-        {
-            if((!Cfg::Edges && (g.m % Cfg::MacroM != 0u || g.n % Cfg::MacroN != 0u)) || g.k % Cfg::MacroK != 0u
-               || g.k < (Cfg::Stages - 1u) * Cfg::MacroK)
-                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-            // a stage's copies address their source inside a 2 GiB window from the stage origin
-            {
-                const uint64_t spanA = static_cast<uint64_t>(g.lda) * sizeof(typename Cfg::InT)
-                                       * (Cfg::AKMajor ? Cfg::MacroM : Cfg::MacroK);
-                const uint64_t spanB = static_cast<uint64_t>(g.ldb) * sizeof(typename Cfg::InT)
-                                       * (Cfg::BKMajor ? Cfg::MacroN : Cfg::MacroK);
-                if(spanA >= 0x7FFF0000ull || spanB >= 0x7FFF0000ull)
-                    return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-            }
-            auto kernel = gemmBlockedKernel<Cfg>;
-            // more than 64 KiB of dynamic LDS needs an explicit opt-in (idempotent, no allocation)
-            if(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   static_cast<int>(Cfg::LdsBytes))
-               != hipSuccess)
-                return ROCWMMA_AMD_LAUNCH_FAILED;
-            const uint32_t tiles = ceilDiv(g.m, Cfg::MacroM) * ceilDiv(g.n, Cfg::MacroN);
-            hipLaunchKernelGGL(kernel,
-                               dim3(tiles),
-                               dim3(Cfg::Threads),
-                               Cfg::LdsBytes,
-                               stream,
-                               g.m,
-                               g.n,
-                               g.k,
-                               static_cast<typename Cfg::InT const*>(g.a),
-                               static_cast<typename Cfg::InT const*>(g.b),
-                               static_cast<typename Cfg::OutT const*>(g.c),
-                               static_cast<typename Cfg::OutT*>(g.d),
-                               g.lda,
-                               g.ldb,
-                               g.ldc,
-                               g.ldd,
-                               static_cast<typename Cfg::CompT>(g.alpha),
-                               static_cast<typename Cfg::CompT>(g.beta),
-                               mx);
-            return launchStatus();
-        }
-
-        // The 4-wave configurations come with either LDS pipeline.  With at most one workgroup per
-        // compute unit a launch is one round of latency-bound workgroups, and the ring of four 64-byte
-        // stages (copies three stages ahead) hides more of it: 128 x 14336 x 4096 int8 25.8 against 29.7 us,
-        // 2048^3 f16 24 against 27 us.  With more workgroups than compute units the units stream operands
-        // all the time, the L2 request rate limits them, and the ring of two 128-byte stages (whole-line
-        // requests) wins: 512 x 14336 x 4096 int8 51 -> 44 us, f16 with a row-major B 101 -> 85 us,
-        // 192 x 14336 x 4096 f16 (64 x 64 tiles) 74 -> 56 us.  Results are identical bit for bit.
-        template <typename Ring4, typename Ring2>
-        int launchByRounds(GemmArgs const& g, hipStream_t stream)
-        {
-            static_assert(Ring4::MacroM == Ring2::MacroM && Ring4::MacroN == Ring2::MacroN, "same tiling");
-            if(ceilDiv(g.m, Ring4::MacroM) * ceilDiv(g.n, Ring4::MacroN) > computeUnits())
-            {
-                const int rc = launchCfg<Ring2>(g, stream);
-                if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE) // (K not in whole 128-byte stages)
-                    return rc;
-            }
-            return launchCfg<Ring4>(g, stream);
-        }
-
         // Tile ladder: the 256 x 256 macro tile when the problem divides into enough of them to occupy
         // at least half of the compute units, else 128 x 128; when that gives at most one tile per two
         // compute units (few token rows against a wide weight matrix), 128 x 64 tiles double the
@@ -318,16 +151,16 @@ namespace rocwmma_amd
     namespace
     {
         template <typename InT>
-        int launchMx(GemmArgs const& g, MxPacked const& mx, hipStream_t stream)
+        int launchMx(GemmArgs const& g, TileExtras const& ex, hipStream_t stream)
         {
             // 256 x 256 tiles of 16x16x128 blocks with block scales; the tiles of a last round at most half
             // full run as 256 x 128 half tiles, as in the unscaled kernel
             using Big     = BlockedConfig<InT, float32_t, float32_t, true, true, 4, 2, 4, 8, 2, 2, 16, false, true>;
             using BigHalf = BlockedConfig<InT, float32_t, float32_t, true, true, 4, 2, 4, 4, 2, 2, 16, false, true>;
-            const int rc  = launchSplitTail<Big, BigHalf>(g, stream, mx);
+            const int rc  = launchSplitTail<Big, BigHalf>(g, stream, ex);
             if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
                 return rc;
-            return launchCfg<Big>(g, stream, mx);
+            return launchCfg<Big>(g, stream, ex);
         }
     } // namespace
 
@@ -335,11 +168,12 @@ namespace rocwmma_amd
     {
         if(g.layoutC != ROCWMMA_AMD_ROW_MAJOR || g.m % 256u != 0u || g.n % 256u != 0u || g.k % 128u != 0u)
             return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-        const MxPacked mx{packedA, packedB, (g.k / 128u + 1u) / 2u};
+        TileExtras ex{};
+        ex.mx = MxPacked{packedA, packedB, (g.k / 128u + 1u) / 2u};
         if(dtypeIn == ROCWMMA_AMD_E4M3)
-            return launchMx<float8_t>(g, mx, stream);
+            return launchMx<float8_t>(g, ex, stream);
         if(dtypeIn == ROCWMMA_AMD_E5M2)
-            return launchMx<bfloat8_t>(g, mx, stream);
+            return launchMx<bfloat8_t>(g, ex, stream);
         return ROCWMMA_AMD_UNSUPPORTED_TYPE;
     }
 

@@ -50,7 +50,8 @@ namespace rocwmma_amd
                   uint32_t WavesPerSimd_ = 1u, // waves per SIMD: sizes the register budget, and no more become resident
                   uint32_t BlockEdge_    = 32u, // MFMA block edge: 32 (32x32xK) or 16 (16x16x2K)
                   bool     Edges_        = false, // M and N need not fill whole macro tiles (multiples of 16 do)
-                  bool     Scaled_       = false> // fp8 operands with one E8M0 scale per 32 elements of K (MX)
+                  bool     Scaled_       = false, // fp8 operands with one E8M0 scale per 32 elements of K (MX)
+                  bool     Fused_        = false> // epilogue adds a per-column bias and applies an activation
         struct BlockedConfig
         {
             using InT   = InT_;
@@ -67,6 +68,8 @@ namespace rocwmma_amd
             // (two runs of 16 from the two halves of the stage, see rocwmma/internal/fragment_map.hpp),
             // so the fragments are read like two steps of a 16-bytes-per-lane operand.
             static constexpr bool     Scaled  = Scaled_;
+            // D = act(alpha * A * B + beta * C + bias[column]): see FusedEpilogue
+            static constexpr bool     Fused   = Fused_;
             static constexpr uint32_t WavesM  = WavesM_;
             static constexpr uint32_t WavesN  = WavesN_;
             static constexpr uint32_t BlocksM = BlocksM_;
@@ -225,6 +228,20 @@ namespace rocwmma_amd
             uint32_t    pairs; // pairs of stages along K (the last one padded when the stage count is odd)
         };
 
+        // What a Fused configuration's epilogue does beyond alpha * acc + beta * C.
+        struct FusedEpilogue
+        {
+            const float* bias; // one value per column of D (n floats), or nullptr
+            int          activation; // rocwmma_amd_activation
+        };
+
+        // Per-launch arguments beyond the GEMM's own, for the configurations that use them.
+        struct TileExtras
+        {
+            MxPacked      mx;
+            FusedEpilogue fused;
+        };
+
         // ---- stream-K support ------------------------------------------------------------------
         // Which part of a tile's K range a call of gemmTile computes.
         enum class TilePart
@@ -361,8 +378,9 @@ namespace rocwmma_amd
                                                     typename Cfg::CompT        alpha,
                                                     typename Cfg::CompT        beta,
                                                     StreamKPart const&         sk,
-                                                    MxPacked const&            mx = MxPacked{})
+                                                    TileExtras const&          ex = TileExtras{})
         {
+            const MxPacked& mx = ex.mx;
             using InT   = typename Cfg::InT;
             using OutT  = typename Cfg::OutT;
             using CompT = typename Cfg::CompT;
@@ -934,6 +952,40 @@ namespace rocwmma_amd
             auto           blockOffset = [&](uint32_t bi, uint32_t bj, uint32_t ld) {
                 return static_cast<size_t>(wRow + bi * Cfg::Block) * ld + wCol + bj * Cfg::Block;
             };
+            // Fused configurations: the bias values of a lane's columns of one block are fetched (four
+            // consecutive floats per run, cache hits after the first row of blocks) just before the
+            // block's results go out; finish() is what every result passes through.
+            static_assert(!Cfg::Fused || std::is_same<CompT, float>::value, "fused epilogue: f32 compute");
+            struct BiasOfBlock
+            {
+                float v[Cfg::Fused ? 4u * Runs : 1u];
+            };
+            auto loadBias = [&](uint32_t bj) {
+                BiasOfBlock bv = {};
+                if constexpr(Cfg::Fused)
+                {
+                    if(ex.fused.bias)
+                    {
+#pragma unroll
+                        for(uint32_t r = 0; r < Runs; ++r)
+                        {
+                            const uint32_t col = wCol + bj * Cfg::Block + 8u * r + 4u * accGroup;
+                            if(!Cfg::Edges || col < n)
+                                __builtin_memcpy(&bv.v[4u * r], ex.fused.bias + col, 16);
+                        }
+                    }
+                }
+                return bv;
+            };
+            auto finish = [&](BiasOfBlock const& bv, uint32_t e, CompT v) -> CompT {
+                if constexpr(Cfg::Fused)
+                    return applyActivation(v + bv.v[e], ex.fused.activation);
+                else
+                {
+                    (void)bv, (void)e;
+                    return v;
+                }
+            };
             if(beta != static_cast<CompT>(0))
             {
                 if constexpr(Cfg::StagedC)
@@ -1012,9 +1064,11 @@ namespace rocwmma_amd
 #pragma unroll
                         for(uint32_t bj = 0; bj < GB; ++bj)
                         {
+                            const BiasOfBlock bv = loadBias(bj0 + bj);
 #pragma unroll
                             for(uint32_t e = 0; e < io[bj].num_elements; ++e)
-                                acc[bi][bj0 + bj].x[e] = alpha * acc[bi][bj0 + bj].x[e] + beta * static_cast<CompT>(io[bj].x[e]);
+                                acc[bi][bj0 + bj].x[e]
+                                    = finish(bv, e, alpha * acc[bi][bj0 + bj].x[e] + beta * static_cast<CompT>(io[bj].x[e]));
                         }
                         // (results replace the accumulators: every store has registers of its own)
 #pragma unroll
@@ -1050,9 +1104,10 @@ namespace rocwmma_amd
                     for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
                     {
                         auto& io = fc[bi % 2u][bj];
+                        const BiasOfBlock bv = loadBias(bj);
 #pragma unroll
                         for(uint32_t e = 0; e < io.num_elements; ++e)
-                            io.x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e] + beta * static_cast<CompT>(io.x[e]));
+                            io.x[e] = static_cast<OutT>(finish(bv, e, alpha * acc[bi][bj].x[e] + beta * static_cast<CompT>(io.x[e])));
                     }
                     if constexpr(PairIO)
                     {
@@ -1083,9 +1138,10 @@ namespace rocwmma_amd
 #pragma unroll
                         for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
                         {
+                            const BiasOfBlock bv = loadBias(bj);
 #pragma unroll
                             for(uint32_t e = 0; e < acc[bi][bj].num_elements; ++e)
-                                acc[bi][bj].x[e] = alpha * acc[bi][bj].x[e];
+                                acc[bi][bj].x[e] = finish(bv, e, alpha * acc[bi][bj].x[e]);
                         }
 #pragma unroll
                         for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
@@ -1097,9 +1153,10 @@ namespace rocwmma_amd
 #pragma unroll
                         for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
                         {
+                            const BiasOfBlock bv = loadBias(bj);
 #pragma unroll
                             for(uint32_t e = 0; e < fd[bj].num_elements; ++e)
-                                fd[bj].x[e] = static_cast<OutT>(alpha * acc[bi][bj].x[e]);
+                                fd[bj].x[e] = static_cast<OutT>(finish(bv, e, alpha * acc[bi][bj].x[e]));
                         }
                         if constexpr(PairIO)
                         {

@@ -32,7 +32,9 @@ namespace rocwmma_amd
                                                                                       uint32_t     ldd,
                                                                                       CompT        alpha,
                                                                                       CompT        beta,
-                                                                                      layout_t     layoutC)
+                                                                                      layout_t     layoutC,
+                                                                                      const float* bias, // fused epilogue (float
+                                                                                      int          activation) // compute types only)
         {
             using FragA   = fragment<matrix_a, BM, BN, BK, InT, LA>;
             using FragB   = fragment<matrix_b, BM, BN, BK, InT, LB>;
@@ -69,6 +71,23 @@ namespace rocwmma_amd
                 bPtr += bStep;
             }
 
+            // fused epilogue: the bias of each element's column is added and the activation applied
+            // before the result is narrowed
+            using MapAcc = typename detail::FragConfig<accumulator, BM, BN, BK, CompT>::Map;
+            auto finish  = [&](uint32_t e, CompT v) -> CompT {
+                if constexpr(std::is_same<CompT, float32_t>::value)
+                {
+                    if(bias)
+                        v += bias[cCol + MapAcc::colOf(e, threadIdx.x % Constants::AMDGCN_WAVE_SIZE)];
+                    return applyActivation(v, activation);
+                }
+                else
+                {
+                    (void)e;
+                    return v;
+                }
+            };
+
             FragC          fc;
             const size_t   cOff = layoutC == mem_row_major ? static_cast<size_t>(cRow) * ldc + cCol
                                                            : static_cast<size_t>(cCol) * ldc + cRow;
@@ -79,13 +98,13 @@ namespace rocwmma_amd
                 load_matrix_sync(fc, c + cOff, ldc, layoutC);
 #pragma unroll
                 for(uint32_t i = 0; i < fc.num_elements; ++i)
-                    fc.x[i] = static_cast<OutT>(alpha * acc.x[i] + beta * static_cast<CompT>(fc.x[i]));
+                    fc.x[i] = static_cast<OutT>(finish(i, alpha * acc.x[i] + beta * static_cast<CompT>(fc.x[i])));
             }
             else
             {
 #pragma unroll
                 for(uint32_t i = 0; i < fc.num_elements; ++i)
-                    fc.x[i] = static_cast<OutT>(alpha * acc.x[i]);
+                    fc.x[i] = static_cast<OutT>(finish(i, alpha * acc.x[i]));
             }
             store_matrix_sync(d + dOff, fc, ldd, layoutC);
         }
@@ -113,7 +132,9 @@ namespace rocwmma_amd
                                g.ldd,
                                static_cast<CompT>(g.alpha),
                                static_cast<CompT>(g.beta),
-                               g.layoutC == ROCWMMA_AMD_ROW_MAJOR ? mem_row_major : mem_col_major);
+                               g.layoutC == ROCWMMA_AMD_ROW_MAJOR ? mem_row_major : mem_col_major,
+                               g.bias,
+                               g.activation);
             return launchStatus();
         }
 

@@ -321,6 +321,33 @@ def test_mx_gemm_scales_are_exact_powers_of_two():
     assert differs[5] and differs.sum() == 1
 
 
+def test_fused_epilogue_restatement():
+    """gemm_bias_act = gemm, then bias per column and activation: without either it is gemm bit for
+    bit; ReLU output is the positive part; GELU against math.erf element by element; the bias follows
+    the columns of D whatever D's layout."""
+    import math
+
+    m, n, k = 32, 48, 64
+    rng = np.random.default_rng(7)
+    a = orc.encode(orc.F16, rng.uniform(-1, 1, m * k).astype(np.float32))
+    b = orc.encode(orc.F16, rng.uniform(-1, 1, k * n).astype(np.float32))
+    c = rng.uniform(-1, 1, m * n).astype(np.float32)
+    bias = rng.uniform(-2, 2, n).astype(np.float32)
+    plain = orc.gemm(orc.F16, orc.F32, 0, 1, 0, 0, m, n, k, a, b, c, 2.0, 0.5)
+    assert np.array_equal(orc.gemm_bias_act(orc.F16, orc.F32, 0, 1, 0, m, n, k, a, b, c, 2.0, 0.5, None, orc.ACT_NONE), plain)
+    with_bias = orc.gemm_bias_act(orc.F16, orc.F32, 0, 1, 0, m, n, k, a, b, c, 2.0, 0.5, bias, orc.ACT_NONE).reshape(m, n)
+    assert np.allclose(with_bias - plain.reshape(m, n), np.broadcast_to(bias, (m, n)), atol=1e-5)
+    relu = orc.gemm_bias_act(orc.F16, orc.F32, 0, 1, 0, m, n, k, a, b, c, 2.0, 0.5, bias, orc.ACT_RELU).reshape(m, n)
+    assert np.array_equal(relu, np.maximum(with_bias, 0.0))
+    gelu = orc.gemm_bias_act(orc.F16, orc.F32, 0, 1, 0, m, n, k, a, b, c, 2.0, 0.5, bias, orc.ACT_GELU).reshape(m, n)
+    ref = np.array([[0.5 * x * (1.0 + math.erf(x / math.sqrt(2.0))) for x in row] for row in with_bias.astype(np.float64)])
+    assert np.max(np.abs(gelu - ref)) < 1e-5
+    # column-major D: same values, transposed storage (c given in D's layout)
+    c_cm = np.ascontiguousarray(c.reshape(m, n).T).reshape(-1)
+    gelu_cm = orc.gemm_bias_act(orc.F16, orc.F32, 0, 1, 1, m, n, k, a, b, c_cm, 2.0, 0.5, bias, orc.ACT_GELU).reshape(n, m)
+    assert np.array_equal(gelu_cm.T, gelu)
+
+
 def test_compare_equal_metric():
     a = np.array([1.0, 2.0, -3.0, 0.0], dtype=np.float32)
     b = np.array([1.0, 2.5, -3.0, 0.0], dtype=np.float32)
