@@ -43,8 +43,8 @@ FP8_BLOCKED_SHAPE = "fp8_16x16x128"  # the matrix instruction of the blocked ker
 # no longer matches is reported as null.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 KERNEL_SOURCES = {
-    "gemm_blocked": ["rocwmma_amd/csrc/gemm_blocked.hip", "rocwmma_amd/csrc/gemm_blocked_core.hpp",
-                     "include/rocwmma/rocwmma_lds.hpp"],
+    "gemm_blocked": ["rocwmma_amd/csrc/gemm_blocked.hip", "rocwmma_amd/csrc/gemm_blocked_launch.hpp",
+                     "rocwmma_amd/csrc/gemm_blocked_core.hpp", "include/rocwmma/rocwmma_lds.hpp"],
 }
 
 
