@@ -662,8 +662,13 @@ def run_extras(rw, torch, dev, gen, only=None):
         dst = torch.empty(2048 * MiB // 4, device=dev, dtype=torch.int32)
         ceil = {}
         for tag, mode, nbytes in (("read_56MiB", rw.STREAM_READ, 56 * MiB), ("read_128MiB", rw.STREAM_READ, 128 * MiB),
-                                  ("read_1792MiB", rw.STREAM_READ, 1792 * MiB), ("copy_1792MiB", rw.STREAM_COPY, 1792 * MiB)):
-            windows = max(1, (2048 * MiB) // nbytes)
+                                  ("read_1792MiB", rw.STREAM_READ, 1792 * MiB), ("copy_1792MiB", rw.STREAM_COPY, 1792 * MiB),
+                                  # what a GEMM's result write can reach: the 256 MiB of an 8192^3 f32 result, to one
+                                  # buffer over and over as the benchmark's GEMMs do (it fits the Infinity Cache) and
+                                  # through 2 GiB (what the HBM itself takes)
+                                  ("write_256MiB_same_buffer", rw.STREAM_WRITE, 256 * MiB),
+                                  ("write_1792MiB", rw.STREAM_WRITE, 1792 * MiB)):
+            windows = 1 if tag.endswith("same_buffer") else max(1, (2048 * MiB) // nbytes)
             state = {"i": 0}
             # (raw addresses and the stream handle prepared up front: a launch of 10 us must not wait for Python)
             srcs = [ctypes.c_void_p(src.data_ptr() + w * nbytes) for w in range(windows)]
