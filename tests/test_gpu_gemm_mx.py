@@ -40,7 +40,7 @@ def check(got, want, tol):
 @pytest.mark.parametrize("workspace", [False, True])
 @pytest.mark.parametrize("la,lb", [(RM, CM), (CM, RM), (RM, RM), (CM, CM)])
 @pytest.mark.parametrize("dtype", [orc.E4M3, orc.E5M2])
-@pytest.mark.parametrize("m,n,k", [(48, 80, 384), (64, 96, 192), (256, 512, 512)])
+@pytest.mark.parametrize("m,n,k", [(48, 80, 384), (64, 96, 192), (256, 512, 512), (256, 256, 128), (512, 256, 896)])
 def test_exact_pattern_with_power_of_two_scales_is_bit_exact(dtype, la, lb, m, n, k, workspace):
     """Elements 0, -1, -2 (the reference's device fill, test/device/common.hpp:204-219) and scales
     1/2, 1, 2: every partial sum is an integer multiple of 1/4 below 2^24 of them, so any order of
