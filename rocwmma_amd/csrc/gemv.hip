@@ -39,6 +39,27 @@ namespace rocwmma_amd
             return acc;
         }
 
+        // Sum over the 16 lanes that share lane % 4 (the 16 blocks of v_mfma_f32_4x4x4_16B), left in every
+        // lane: two rotations inside the rows of 16 lanes (DPP), then the rows of a half and the two halves
+        // exchanged with v_permlane16_swap / v_permlane32_swap.  All on the vector ALU: the same sum with
+        // four ds_bpermute steps per value kept the LDS pipe busy for microseconds per workgroup.
+        ROCWMMA_DEVICE inline float sumOverBlocks(float v)
+        {
+#if defined(__HIP_DEVICE_COMPILE__)
+            const auto bits = [](float f) { return __builtin_bit_cast(uint32_t, f); };
+            const auto flt  = [](uint32_t u) { return __builtin_bit_cast(float, u); };
+            v += flt(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(bits(v)), 0x124 /* row_ror:4 */, 0xF, 0xF, true)));
+            v += flt(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(bits(v)), 0x128 /* row_ror:8 */, 0xF, 0xF, true)));
+            // (x, x) -> (rows 0 0 2 2, rows 1 1 3 3) of x
+            const auto rows = __builtin_amdgcn_permlane16_swap(bits(v), bits(v), false, false);
+            v               = flt(rows[0]) + flt(rows[1]);
+            // (x, x) -> (lower half twice, upper half twice)
+            const auto halves = __builtin_amdgcn_permlane32_swap(bits(v), bits(v), false, false);
+            v                 = flt(halves[0]) + flt(halves[1]);
+#endif
+            return v;
+        }
+
         ROCWMMA_DEVICE inline float waveSum(float v)
         {
 #pragma unroll
@@ -220,8 +241,8 @@ namespace rocwmma_amd
         //     of a quarter-wave, 4 chunks x 4 columns, read 16 distinct bank groups);
         //   * a wave walks its K slice of its 4 rows, `Unroll` 1 KiB loads in flight;
         //   * block b accumulates the products of its own K chunks; at the end of a row quad the
-        //     16 blocks are summed with 4 cross-lane steps, the K-slice partial sums meet in LDS
-        //     and are added in slice order (deterministic).
+        //     16 blocks are summed on the vector ALU (sumOverBlocks), the K-slice partial sums meet in
+        //     LDS and are added in slice order (deterministic).
         constexpr uint32_t kQuadWaves = 16, kQuadSlices = 4;
 
         template <uint32_t NCols, uint32_t Unroll>
@@ -312,12 +333,7 @@ namespace rocwmma_amd
 #pragma unroll
                     for(uint32_t i = 0; i < 4u; ++i)
                     {
-                        float v = acc[g][i];
-                        v += __shfl_xor(v, 4, 64);
-                        v += __shfl_xor(v, 8, 64);
-                        v += __shfl_xor(v, 16, 64);
-                        v += __shfl_xor(v, 32, 64);
-                        acc[g][i] = v;
+                        acc[g][i] = sumOverBlocks(acc[g][i]);
                     }
                 if(blk == 0u)
                 {
