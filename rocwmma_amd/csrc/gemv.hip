@@ -60,12 +60,17 @@ namespace rocwmma_amd
             return v;
         }
 
+        // Sum over the 64 lanes, left in every lane: inside the quads with two DPP quad permutes, then
+        // over the 16 quads as above.
         ROCWMMA_DEVICE inline float waveSum(float v)
         {
-#pragma unroll
-            for(int off = 32; off >= 1; off >>= 1)
-                v += __shfl_xor(v, off, 64);
-            return v;
+#if defined(__HIP_DEVICE_COMPILE__)
+            const auto bits = [](float f) { return static_cast<int>(__builtin_bit_cast(uint32_t, f)); };
+            const auto flt  = [](int u) { return __builtin_bit_cast(float, static_cast<uint32_t>(u)); };
+            v += flt(__builtin_amdgcn_update_dpp(0, bits(v), 0xB1 /* quad_perm:[1,0,3,2] */, 0xF, 0xF, true));
+            v += flt(__builtin_amdgcn_update_dpp(0, bits(v), 0x4E /* quad_perm:[2,3,0,1] */, 0xF, 0xF, true));
+#endif
+            return sumOverBlocks(v);
         }
 
         // Split kernel: workgroup = 4 waves = (4 / KSplit) row groups x KSplit slices of K.
