@@ -86,6 +86,39 @@ def test_gemm_argument_validation(lib):
         assert _gemm(lib) == 6
 
 
+def test_fused_and_block_scaled_gemm_argument_validation(lib):
+    f = lib.rocwmma_amd_gemm_bias_act
+    ok = dict(m=32, n=32, k=32, a=4096, lda=32, b=8192, ldb=32, c=12288, ldc=32, d=16384, ldd=32)
+
+    def fused(dtype_in=rw.F16, dtype_out=rw.F32, bias=20480, act=rw.ACT_GELU, **kw):
+        v = dict(ok, **kw)
+        return f(dtype_in, dtype_out, 0, 1, 0, v["m"], v["n"], v["k"], v["a"], v["lda"], v["b"], v["ldb"], v["c"], v["ldc"],
+                 v["d"], v["ldd"], 1.0, 1.0, bias, act, None)
+
+    assert fused(dtype_in=rw.I8, dtype_out=rw.I32) == 2      # float types only
+    assert fused(dtype_in=rw.F32) == 2
+    assert fused(act=7) == 1
+    assert fused(bias=20484) == 4                              # bias must be 16-byte aligned
+    assert fused(a=None) == 1
+    assert fused(m=24) == 3
+
+    g = lib.rocwmma_amd_gemm_mx
+
+    def mx(dtype_in=rw.E4M3, m=32, n=32, k=128, sa=20480, lsa=4, sb=24576, lsb=4, ws=None, wsb=0):
+        return g(dtype_in, 0, 1, 0, m, n, k, 4096, k, sa, lsa, 8192, k, sb, lsb, 12288, n, 16384, n, 1.0, 1.0, ws, wsb, None)
+
+    assert mx(dtype_in=rw.F16) == 2                            # fp8 / bf8 only
+    assert mx(dtype_in=rw.I8) == 2
+    assert mx(sa=None) == 1
+    assert mx(k=96) == 3                                       # K in whole instructions (64 at least)
+    assert mx(lsa=3) == 5                                      # scale leading dimension below k / 32
+    assert lib.rocwmma_amd_gemm_mx_workspace_size(256, 512, 512) == (4 + 8) * 2 * 64 * 8
+    import torch
+
+    if not torch.cuda.is_available():
+        assert fused() == 6 and mx() == 6
+
+
 def test_gemv_and_dlrm_argument_validation(lib):
     f = lib.rocwmma_amd_gemv
     assert f(64, 64, 3, 4096, 64, 8192, 64, 12288, 64, 1.0, 0.0, None) == 3
