@@ -591,6 +591,29 @@ def run_extras(rw, torch, dev, gen, only=None):
                                    "note": "E4M3 operands, E8M0 scales per 32 elements of K, scale re-ordering included"}
         del Am, Bm, SAm, SBm, Dm, ws
 
+    # ... and its 16-token shape (weight streaming): weights and their scales rotated over 5 buffers
+    if wanted("gemm_mxfp8_m16"):
+        m = 16
+        Am = (torch.randn(m * k, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+        Bms = [(torch.randn(k * n, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn) for _ in range(wcopies)]
+        SAm = torch.randint(124, 131, (m * (k // 32),), device=dev, dtype=torch.uint8, generator=gen)
+        SBms = [torch.randint(124, 131, (n * (k // 32),), device=dev, dtype=torch.uint8, generator=gen) for _ in range(wcopies)]
+        Dm = torch.empty(m * n, device=dev, dtype=torch.float32)
+        state = {"i": 0}
+
+        def fnm16():
+            j = state["i"] % wcopies
+            rw.gemm_mx(rw.E4M3, RM, CM, RM, m, n, k, Am, SAm, Bms[j], SBms[j], None, Dm, 1.0, 0.0)
+            state["i"] += 1
+
+        fnm16()
+        ms = event_ms(fnm16, iters, torch)
+        byts = m * k + n * k + (m + n) * (k // 32) + 4.0 * m * n
+        out["gemm_mxfp8_m16"] = {"ms": round(ms, 4), "gbs": round(byts / ms / 1e6, 1),
+                                 "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4),
+                                 "note": "E4M3 operands, E8M0 scales per 32 elements of K (scale bytes counted)"}
+        del Am, Bms, SAm, SBms, Dm
+
     # config 4: GEMV, buffers rotated over > 512 MB so the 256 MB Infinity Cache cannot serve A
     for (m, kk) in ((8192, 8192), (14336, 4096)):
         cols = [nc for nc in (1, 4, 8) if wanted(f"gemv_{m}x{kk}_n{nc}")]

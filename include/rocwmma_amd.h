@@ -294,8 +294,11 @@ int rocwmma_amd_gemm_bias_act(int          dtype_in,
  * (for a col-major C: col-major A / row-major B), m and n multiples of 256 and k a multiple of 128
  * run on the blocked kernel (256 x 256 tiles, v_mfma_scale_f32_16x16x128_f8f6f4): the call then
  * enqueues a small kernel that re-orders the scales into the workspace, and the GEMM (two launches).  Everything else
- * runs one block per wave straight from global memory.  Two calls that use the same workspace must
- * not overlap in time.
+ * runs one block per wave straight from global memory, except up to 32 rows of a row-major A against a
+ * col-major B with k a multiple of 1024 (few tokens against a wide weight matrix), which run on the
+ * weight-streaming kernel with or without a workspace (m * k <= 128 KiB; scale_a 4-byte aligned with
+ * ld_scale_a a multiple of 4, scale_b 16-byte aligned with ld_scale_b a multiple of 16).  Two calls
+ * that use the same workspace must not overlap in time.
  */
 size_t rocwmma_amd_gemm_mx_workspace_size(uint32_t m, uint32_t n, uint32_t k);
 

@@ -370,6 +370,13 @@ int rocwmma_amd_gemm_mx(int         dtype_in,
         return ROCWMMA_AMD_NO_DEVICE;
     GemmArgs args{m, n, k, a, b, c, d, lda, ldb, c ? ldc : ldd, ldd, alpha, beta, layout_c};
     MxScales scales{static_cast<const uint8_t*>(scale_a), static_cast<const uint8_t*>(scale_b), ld_scale_a, ld_scale_b};
+    if(m <= 32u)
+    {
+        // few token rows against a wide weight matrix: the weight-streaming kernel
+        rc = launchGemmMxSkinny(dtype_in, layout_a, layout_b, args, scales, asStream(stream));
+        if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE && rc != ROCWMMA_AMD_UNSUPPORTED_TYPE)
+            return rc;
+    }
     if(workspace && workspace_bytes >= mxPackedScaleBytes(m, n, k) && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0u)
     {
         GemmArgs blocked = args;

@@ -152,6 +152,8 @@ namespace rocwmma_amd
     // The blocked kernel with the fused epilogue (float types, row-major C/D; args.bias / args.activation)
     int launchGemmBlockedFused(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
 
+    // Block-scaled weight streaming: up to 32 token rows, row-major A, col-major B, row-major C/D
+    int launchGemmMxSkinny(int dtypeIn, int layoutA, int layoutB, GemmArgs const& args, MxScales const& scales, hipStream_t stream);
     // Block-scaled fp8 / bf8 GEMM (f32 C/D): one block per wave, every layout pair
     int launchGemmMxWaveTile(int dtypeIn, int layoutA, int layoutB, GemmArgs const& args, MxScales const& scales, hipStream_t stream);
 

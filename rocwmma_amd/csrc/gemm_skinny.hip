@@ -30,7 +30,12 @@ namespace rocwmma_amd
         constexpr uint32_t kSkinnyKBytes = 128; // bytes of K per fragment step (128 8-bit or 64 16-bit elements)
         constexpr uint32_t kSkinnyMaxA   = 131072; // bytes of LDS the token matrix may take
 
-        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t Ahead>
+        // Scaled: fp8 operands with one E8M0 scale per 32 elements of K (block-scaled / MX); a fragment step
+        // is then one v_mfma_scale_f32_16x16x128_f8f6f4, whose scale operand of lane l belongs to row
+        // l % 16 and K block l / 16 of the step.  The scales of the weights are fetched with the weight
+        // fragments (one dword per lane and step: the four K blocks of the step, shifted down by the lane's
+        // own), the scales of the tokens wait in LDS next to A.
+        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t Ahead, bool Scaled = false>
         __global__ void __launch_bounds__(64 * kSkinnyWaves) gemmSkinnyKernel(uint32_t    m,
                                                                               uint32_t    n,
                                                                               uint32_t    k,
@@ -44,9 +49,11 @@ namespace rocwmma_amd
                                                                               uint32_t    ldd,
                                                                               CompT       alpha,
                                                                               CompT       beta,
-                                                                              uint32_t    rowsPerWg)
+                                                                              uint32_t    rowsPerWg,
+                                                                              MxScales    scales)
         {
             constexpr uint32_t E       = sizeof(InT); // bytes per element
+            static_assert(!Scaled || (sizeof(InT) == 1u && std::is_same<CompT, float>::value), "block scales: fp8 operands");
             constexpr uint32_t kSkinnyK = kSkinnyKBytes / E; // K elements per fragment step
             using FragA   = fragment<matrix_a, 16, 16, kSkinnyK, InT, row_major>;
             using FragB   = fragment<matrix_b, 16, 16, kSkinnyK, InT, col_major>;
@@ -60,6 +67,9 @@ namespace rocwmma_amd
             // partial[wave][mblock][lane] : the 4 accumulator registers of a lane as one 16-byte unit
             using Quad    = CompT __attribute__((ext_vector_type(4)));
             Quad* partial = reinterpret_cast<Quad*>(ldsRaw + m * k * E);
+            // (Scaled) the tokens' scales, [k / 128][m] dwords (the four K blocks of a step), in the space of the
+            // partial sums until those are due
+            uint8_t* aScales = reinterpret_cast<uint8_t*>(partial);
 
             const uint32_t lane   = threadIdx.x & 63u;
             const uint32_t wave   = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -92,6 +102,20 @@ namespace rocwmma_amd
                 }
             }
 
+            // (Scaled) the tokens' scales: at most 32 x 128 bytes, one dword per thread (k / 32 is a multiple of 4
+            // and the scale rows are 4-byte aligned: checked by the host).  Fetched here, stored to LDS only
+            // after the first weight loads have gone out: the store has to wait for the fetch, and a wait in
+            // front of the weight loads would hold them back until A has landed.
+            uint32_t       myScalesA  = 0u;
+            const uint32_t scaleWords = Scaled ? m * (k / 128u) : 0u; // <= 1024 = threads of the workgroup
+            if constexpr(Scaled)
+            {
+                const uint32_t perRow = k / 128u;
+                if(threadIdx.x < scaleWords)
+                    myScalesA = *reinterpret_cast<const uint32_t*>(scales.a + static_cast<size_t>(threadIdx.x / perRow) * scales.lda
+                                                                   + (threadIdx.x % perRow) * 4u);
+            }
+
             FragAcc acc[MBlocks];
 #pragma unroll
             for(uint32_t i = 0; i < MBlocks; ++i)
@@ -101,9 +125,31 @@ namespace rocwmma_amd
             const uint32_t aRow = lane & 15u;
             const InT*     bPtr = b + static_cast<size_t>(n0) * ldb + kBeg;
 
+            // (Scaled) this lane's weight row of scales, at the first K block of the wave's K slice
+            const uint8_t* sbPtr = nullptr;
+            uint32_t       sb[Scaled ? Ahead : 1u] = {};
+            if constexpr(Scaled)
+                sbPtr = scales.b + static_cast<size_t>(n0 + (lane & 15u)) * scales.ldb + kBeg / 32u;
+            const uint32_t myShift = 8u * (lane >> 4); // the lane's K block of a step inside the step's dword
             auto loadB = [&](FragB(&fb)[Ahead], uint32_t kk) {
                 if(rowLive) // (lanes of rows beyond a half-filled block keep their zeros)
                 {
+                    if constexpr(Scaled)
+                    {
+                        // The dwords of up to four consecutive steps in one load (16-byte aligned: checked by the
+                        // host), in front of the fragments: loads return in order, and behind them the first
+                        // MFMA of a batch would wait for the whole batch.
+                        constexpr uint32_t Vec = Ahead < 4u ? Ahead : 4u;
+                        typedef uint32_t   Dwords __attribute__((ext_vector_type(Vec)));
+#pragma unroll
+                        for(uint32_t u = 0; u < Ahead; u += Vec)
+                        {
+                            const Dwords q = *reinterpret_cast<const Dwords*>(sbPtr + (kk + u * kSkinnyK) / 32u);
+#pragma unroll
+                            for(uint32_t j = 0; j < Vec; ++j)
+                                sb[u + j] = q[j];
+                        }
+                    }
 #pragma unroll
                     for(uint32_t u = 0; u < Ahead; ++u)
                         load_matrix_sync(fb[u], bPtr + kk + u * kSkinnyK, ldb);
@@ -127,7 +173,21 @@ namespace rocwmma_amd
                                 detail::copyBytes<16u>(fa.x + ch * MapA::kpack + piece * (16u / E),
                                                        aTile + row * k * E + (((kByte >> 4) ^ (row & 15u)) << 4));
                             }
-                        mma_sync(acc[i], fa, fb[u], acc[i]);
+                        if constexpr(Scaled)
+                        {
+#if ROCWMMA_ARCH_GFX950 // (the instruction table exists in the device pass only)
+                            using Op  = detail::MfmaScaled<detail::TypeInfo<InT>::cls, detail::TypeInfo<InT>::cls, 16u>;
+                            using Acc = typename Op::Acc;
+                            // (dword of step s of row r at [s][r]: the 16 rows a quarter-wave reads are 16 consecutive
+                            // dwords; row-major, 128 bytes apart, they all fell into one bank)
+                            const uint32_t sa = reinterpret_cast<const uint32_t*>(aScales)[((kBeg + kk + u * kSkinnyK) / kSkinnyK) * m + row];
+                            Acc&           v  = *reinterpret_cast<Acc*>(acc[i].x);
+                            // (the accumulator is kept transposed: the instruction's first multiplicand is B)
+                            v = Op::template exec<0, 0>(fb[u].x, fa.x, v, sb[u] >> myShift, sa >> myShift);
+#endif
+                        }
+                        else
+                            mma_sync(acc[i], fa, fb[u], acc[i]);
                     }
             };
 
@@ -137,6 +197,11 @@ namespace rocwmma_amd
             for(uint32_t u = 0; u < Ahead; ++u)
                 fill_fragment(fb[u], static_cast<InT>(0));
             loadB(fb, 0u);
+            if constexpr(Scaled)
+            {
+                if(threadIdx.x < scaleWords)
+                    reinterpret_cast<uint32_t*>(aScales)[(threadIdx.x % (k / 128u)) * m + threadIdx.x / (k / 128u)] = myScalesA;
+            }
             lds::waitCopiesAndReads<0>();
             __syncthreads();
             multiply(fb, 0u);
@@ -147,6 +212,8 @@ namespace rocwmma_amd
             }
 
             // meet in LDS
+            if constexpr(Scaled)
+                __syncthreads(); // (everybody is done with the scales that sit where the partial sums go)
 #pragma unroll
             for(uint32_t i = 0; i < MBlocks; ++i)
                 partial[(wave * MBlocks + i) * 64u + lane] = *reinterpret_cast<Quad*>(acc[i].x);
@@ -187,11 +254,11 @@ namespace rocwmma_amd
             }
         }
 
-        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t Ahead>
-        int launchOne(GemmArgs const& g, hipStream_t stream)
+        template <typename InT, typename OutT, typename CompT, uint32_t MBlocks, uint32_t Ahead, bool Scaled = false>
+        int launchOne(GemmArgs const& g, hipStream_t stream, MxScales const& scales = MxScales{})
         {
             const uint32_t lds    = g.m * g.k * static_cast<uint32_t>(sizeof(InT)) + kSkinnyWaves * MBlocks * 1024u;
-            auto           kernel = gemmSkinnyKernel<InT, OutT, CompT, MBlocks, Ahead>;
+            auto           kernel = gemmSkinnyKernel<InT, OutT, CompT, MBlocks, Ahead, Scaled>;
             if(lds > 65536u
                && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(lds))
@@ -212,7 +279,7 @@ namespace rocwmma_amd
             hipLaunchKernelGGL(kernel, dim3((g.n + rows - 1u) / rows), dim3(64u * kSkinnyWaves), lds,
                                stream, g.m, g.n, g.k, static_cast<InT const*>(g.a), static_cast<InT const*>(g.b),
                                static_cast<OutT const*>(g.c), static_cast<OutT*>(g.d), g.lda, g.ldb, g.ldc, g.ldd,
-                               static_cast<CompT>(g.alpha), static_cast<CompT>(g.beta), rows);
+                               static_cast<CompT>(g.alpha), static_cast<CompT>(g.beta), rows, scales);
             return launchStatus();
         }
 
@@ -492,6 +559,47 @@ namespace rocwmma_amd
             return launchOne<InT, OutT, CompT, 2, 2>(g, stream);
         }
     } // namespace
+
+    namespace
+    {
+        template <typename InT>
+        int pickShapeMx(GemmArgs const& g, MxScales const& s, hipStream_t stream)
+        {
+            // as pickShape, for up to 32 token rows whose A fits the LDS; scale rows of A readable as dwords, of B
+            // as 16-byte vectors
+            if(g.m > 32u || g.m * g.k > kSkinnyMaxA)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            if(g.m % 16u != 0u || g.n % 16u != 0u || g.k % 1024u != 0u)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            if((reinterpret_cast<uintptr_t>(s.a) & 3u) || (reinterpret_cast<uintptr_t>(s.b) & 15u) || s.lda % 4u != 0u || s.ldb % 16u != 0u)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            const uint32_t steps = g.k / (kSkinnySlices * kSkinnyKBytes);
+            if(g.m == 16u)
+            {
+                if(steps % 8u == 0u)
+                    return launchOne<InT, float32_t, float32_t, 1, 8, true>(g, stream, s);
+                if(steps % 4u == 0u)
+                    return launchOne<InT, float32_t, float32_t, 1, 4, true>(g, stream, s);
+                return launchOne<InT, float32_t, float32_t, 1, 2, true>(g, stream, s);
+            }
+            if(steps % 8u == 0u)
+                return launchOne<InT, float32_t, float32_t, 2, 8, true>(g, stream, s);
+            if(steps % 4u == 0u)
+                return launchOne<InT, float32_t, float32_t, 2, 4, true>(g, stream, s);
+            return launchOne<InT, float32_t, float32_t, 2, 2, true>(g, stream, s);
+        }
+    } // namespace
+
+    int launchGemmMxSkinny(int dtypeIn, int layoutA, int layoutB, GemmArgs const& g, MxScales const& s, hipStream_t stream)
+    {
+        if(layoutA != ROCWMMA_AMD_ROW_MAJOR || layoutB != ROCWMMA_AMD_COL_MAJOR || g.layoutC != ROCWMMA_AMD_ROW_MAJOR)
+            return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+        if(dtypeIn == ROCWMMA_AMD_E4M3)
+            return pickShapeMx<float8_t>(g, s, stream);
+        if(dtypeIn == ROCWMMA_AMD_E5M2)
+            return pickShapeMx<bfloat8_t>(g, s, stream);
+        return ROCWMMA_AMD_UNSUPPORTED_TYPE;
+    }
 
     int launchGemmSkinny(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& g, hipStream_t stream)
     {

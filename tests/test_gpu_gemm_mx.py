@@ -91,6 +91,27 @@ def test_wide_range_of_scales_against_the_size_of_the_terms(workspace):
     assert np.max(np.abs(got - want) / size) < 2.0 ** -14
 
 
+@pytest.mark.parametrize("dtype", [orc.E4M3, orc.E5M2])
+@pytest.mark.parametrize("m,n,k", [(16, 14336, 4096), (32, 1024, 4096), (16, 200 * 16, 1024), (32, 80, 2048)])
+def test_few_token_rows_on_the_weight_streaming_kernel(dtype, m, n, k):
+    """Up to 32 token rows against a wide block-scaled weight matrix (row-major A, col-major B): the
+    weight-streaming kernel with the scaled instruction.  Exact pattern bit for bit, random operands
+    within the fp8 tolerance, with and without C."""
+    a = exact_int_bits(dtype, m, k, RM)
+    b = exact_int_bits(dtype, k, n, CM)
+    sa, sb = scales(71, m, k, 126, 128), scales(72, n, k, 126, 128)
+    c = exact_int_bits(orc.F32, m, n, RM)
+    got = run_mx(dtype, RM, CM, RM, m, n, k, a, sa, b, sb, c, 2.0, 3.0, False)
+    want = orc.gemm_mx(dtype, RM, CM, RM, RM, m, n, k, a, sa, b, sb, c, 2.0, 3.0)
+    check(got, want, 0.0)
+    a = uniform_bits(73, dtype, m * k)
+    b = uniform_bits(74, dtype, k * n)
+    sa, sb = scales(75, m, k, 124, 130), scales(76, n, k, 124, 130)
+    got = run_mx(dtype, RM, CM, RM, m, n, k, a, sa, b, sb, None, 0.5, 0.0, False)
+    want = orc.gemm_mx(dtype, RM, CM, RM, RM, m, n, k, a, sa, b, sb, None, 0.5, 0.0)
+    check(got, want, 1e-2)
+
+
 def test_unit_scales_give_the_unscaled_gemm():
     import torch
 
