@@ -291,8 +291,10 @@ int rocwmma_amd_gemm_bias_act(int          dtype_in,
  * Shapes: m, n multiples of 16 and k a multiple of 128, or m, n multiples of 32 and k a multiple of 64.
  * workspace: NULL, or device memory (256-byte aligned) of at least
  * rocwmma_amd_gemm_mx_workspace_size(m, n, k) bytes.  With a workspace, row-major A / col-major B
- * (for a col-major C: col-major A / row-major B), m and n multiples of 256 and k a multiple of 128
- * run on the blocked kernel (256 x 256 tiles, v_mfma_scale_f32_16x16x128_f8f6f4): the call then
+ * (for a col-major C: col-major A / row-major B) with k a multiple of 128 run on the blocked kernels
+ * (256 x 256 tiles of v_mfma_scale_f32_16x16x128_f8f6f4 blocks when m and n are multiples of 256 and the
+ * tiles occupy at least half of the compute units, else 128 x 128 or 128 x 64 tiles of 32x32x64 blocks with
+ * partly filled edge tiles): the call then
  * enqueues a small kernel that re-orders the scales into the workspace, and the GEMM (two launches).  Everything else
  * runs one block per wave straight from global memory, except up to 32 rows of a row-major A against a
  * col-major B with k a multiple of 1024 (few tokens against a wide weight matrix), which run on the

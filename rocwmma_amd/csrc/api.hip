@@ -388,12 +388,13 @@ int rocwmma_amd_gemm_mx(int         dtype_in,
             std::swap(sc.lda, sc.ldb);
         }
         transposeForColMajorC(blocked, la, lb);
-        if(la == ROCWMMA_AMD_ROW_MAJOR && lb == ROCWMMA_AMD_COL_MAJOR && blocked.m % 256u == 0u && blocked.n % 256u == 0u
-           && k % 128u == 0u)
+        if(la == ROCWMMA_AMD_ROW_MAJOR && lb == ROCWMMA_AMD_COL_MAJOR && k % 128u == 0u
+           && static_cast<uint64_t>(lda) * 128u < 0x7FFF0000ull && static_cast<uint64_t>(ldb) * 128u < 0x7FFF0000ull)
         {
             char* packedA = static_cast<char*>(workspace);
             char* packedB = packedA + mxPackedScaleOffsetB(blocked.m, k);
-            rc            = launchMxPackScales(sc, blocked.m, blocked.n, k, packedA, packedB, asStream(stream));
+            rc            = launchMxPackScales(sc, blocked.m, blocked.n, k, packedA, packedB, !gemmMxBlockedUsesLargeTile(blocked),
+                                               asStream(stream));
             if(rc != ROCWMMA_AMD_OK)
                 return rc;
             rc = launchGemmMxBlocked(dtype_in, blocked, packedA, packedB, asStream(stream));

@@ -143,11 +143,16 @@ namespace rocwmma_amd
     {
         return mxPackedScaleOffsetB(m, k) + mxPackedScaleBytesOf(n, k);
     }
-    // Re-orders both operands' scales (one launch).
-    int launchMxPackScales(MxScales const& scales, uint32_t m, uint32_t n, uint32_t k, void* packedA, void* packedB, hipStream_t stream);
-    // The blocked kernel on packed scales: row-major A, col-major B, row-major C/D, m and n multiples
-    // of 256, k a multiple of 128.
-    int launchGemmMxBlocked(int dtypeIn, GemmArgs const& args, const void* packedA, const void* packedB, hipStream_t stream);
+    // Re-orders both operands' scales (one launch).  wide32: for the tiles of 32-wide blocks (lane l = row
+    // l % 32 of a block and K block l / 32 of a 64-byte step; 8 bytes per lane = [block 0..1][step 0..3])
+    // instead of 16-wide ones (lane l = row l % 16, K block l / 16 of a 128-byte stage; [block 0..3][stage 0..1]).
+    int launchMxPackScales(MxScales const& scales, uint32_t m, uint32_t n, uint32_t k, void* packedA, void* packedB, bool wide32,
+                           hipStream_t stream);
+    // The blocked kernel on packed scales: row-major A, col-major B, row-major C/D, m and n multiples of 16,
+    // k a multiple of 128.  256 x 256 tiles of 16-wide blocks when gemmMxBlockedUsesLargeTile(), else 128 x 128
+    // tiles of 32-wide blocks: the scales must have been packed for that.
+    bool gemmMxBlockedUsesLargeTile(GemmArgs const& args);
+    int  launchGemmMxBlocked(int dtypeIn, GemmArgs const& args, const void* packedA, const void* packedB, hipStream_t stream);
 
     // The blocked kernel with the fused epilogue (float types, row-major C/D; args.bias / args.activation)
     int launchGemmBlockedFused(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);

@@ -164,16 +164,39 @@ namespace rocwmma_amd
         }
     } // namespace
 
+    namespace
+    {
+        template <typename InT>
+        int launchMxMid(GemmArgs const& g, TileExtras const& ex, hipStream_t stream)
+        {
+            // 128 x 128 tiles of 32x32x64 blocks with block scales, the last row and column of tiles partly
+            // filled: any m, n in multiples of 16
+            using Mid = BlockedConfig<InT, float32_t, float32_t, true, true, 2, 2, 2, 2, 2, 2, 32, true, true>;
+            // at most one 128 x 128 tile per two compute units (few token rows against a wide weight matrix):
+            // 128 x 64 tiles put twice as many workgroups to work
+            using Narrow = BlockedConfig<InT, float32_t, float32_t, true, true, 2, 2, 2, 1, 2, 3, 32, true, true>;
+            if(2u * ceilDiv(g.m, 128u) * ceilDiv(g.n, 128u) <= computeUnits())
+                return launchCfg<Narrow>(g, stream, ex);
+            return launchCfg<Mid>(g, stream, ex);
+        }
+    } // namespace
+
+    bool gemmMxBlockedUsesLargeTile(GemmArgs const& g)
+    {
+        return g.m % 256u == 0u && g.n % 256u == 0u && 2u * (g.m / 256u) * (g.n / 256u) >= computeUnits();
+    }
+
     int launchGemmMxBlocked(int dtypeIn, GemmArgs const& g, const void* packedA, const void* packedB, hipStream_t stream)
     {
-        if(g.layoutC != ROCWMMA_AMD_ROW_MAJOR || g.m % 256u != 0u || g.n % 256u != 0u || g.k % 128u != 0u)
+        if(g.layoutC != ROCWMMA_AMD_ROW_MAJOR || g.m % 16u != 0u || g.n % 16u != 0u || g.k % 128u != 0u)
             return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
         TileExtras ex{};
         ex.mx = MxPacked{packedA, packedB, (g.k / 128u + 1u) / 2u};
+        const bool large = gemmMxBlockedUsesLargeTile(g);
         if(dtypeIn == ROCWMMA_AMD_E4M3)
-            return launchMx<float8_t>(g, ex, stream);
+            return large ? launchMx<float8_t>(g, ex, stream) : launchMxMid<float8_t>(g, ex, stream);
         if(dtypeIn == ROCWMMA_AMD_E5M2)
-            return launchMx<bfloat8_t>(g, ex, stream);
+            return large ? launchMx<bfloat8_t>(g, ex, stream) : launchMxMid<bfloat8_t>(g, ex, stream);
         return ROCWMMA_AMD_UNSUPPORTED_TYPE;
     }
 

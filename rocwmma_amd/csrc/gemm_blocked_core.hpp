@@ -130,8 +130,8 @@ namespace rocwmma_amd
                                             && 2u * Block * GroupBlocks * Block * sizeof(OutT) * Waves <= LdsBytes;
 
             static_assert(Block == 32u || Block == 16u, "MFMA blocks are 32 or 16 wide");
-            static_assert(!Scaled || (Block == 16u && KPackBytes == 32u && AKMajor && BKMajor && Stages_ == 2u && !Edges_),
-                          "block scales: fp8 16x16x128 on K-contiguous operands in the ring of two, whole tiles");
+            static_assert(!Scaled || (KPackBytes == 32u && AKMajor && BKMajor && Stages_ == 2u && (Block == 32u || !Edges_)),
+                          "block scales: fp8 on K-contiguous operands in the ring of two (16x16x128 on whole tiles, or 32x32x64)");
             static_assert(Block == 32u || KPackBytes == 16u || ((PairReads || Scaled) && AKMajor && BKMajor && Stages_ == 2u),
                           "16-wide blocks: 16 bytes of K per lane (16-bit types, int8), or fp8 16x16x128 on K-contiguous "
                           "operands in the ring of two");
@@ -462,8 +462,25 @@ namespace rocwmma_amd
             auto readFrags = [&](Frags& f, uint32_t slot, uint32_t ks) {
                 const char* ldsA = ldsRaw + slot * Cfg::StageBytes;
                 const char* ldsB = ldsA + Cfg::BytesA;
-                if constexpr(Cfg::Scaled) // (has a reader of its own in its loop)
+                if constexpr(Cfg::Scaled && Cfg::Block == 16u) // (has a reader of its own in its loop)
                     return;
+                else if constexpr(Cfg::Scaled)
+                {
+                    // 32x32x64 with block scales: the instruction's own K order, two runs of 16 bytes per lane from
+                    // the two halves of the 64-byte step (chunks h and 2 + h of the step's four)
+#pragma unroll
+                    for(uint32_t i = 0; i < Cfg::BlocksM; ++i)
+                    {
+                        TileA::template readBlock32<16u>(f.a[i].x, ldsA, waveM * Cfg::WaveM + i * Cfg::Block, 2u * ks, lane);
+                        TileA::template readBlock32<16u>(f.a[i].x + 16, ldsA, waveM * Cfg::WaveM + i * Cfg::Block, 2u * ks + 1u, lane);
+                    }
+#pragma unroll
+                    for(uint32_t j = 0; j < Cfg::BlocksN; ++j)
+                    {
+                        TileB::template readBlock32<16u>(f.b[j].x, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, 2u * ks, lane);
+                        TileB::template readBlock32<16u>(f.b[j].x + 16, ldsB, waveN * Cfg::WaveN + j * Cfg::Block, 2u * ks + 1u, lane);
+                    }
+                }
                 else
                 {
 #pragma unroll
@@ -671,12 +688,70 @@ namespace rocwmma_amd
                 // the copies of stage i+2 go out right behind it, into stage i's slot, and have the
                 // phases up to the next barrier to land.  Past the end of K the loop copies the
                 // last stage again and reads fragments nobody multiplies, so its body is uniform.
+                // Block scales (Scaled, 32-wide blocks): per lane and pair of stages (256 bytes of K = four
+                // instruction steps), one dword per block of 32 rows, byte = step; the step's byte is shifted
+                // down at run time.  The next pair's are loaded behind the barrier of a pair's first stage.
+                static_assert(!Cfg::Scaled || Cfg::KSteps == 2u, "packed scales: two instruction steps per stage");
+                uint32_t        sA[Cfg::BlocksM] = {}, sB[Cfg::BlocksN] = {}, sAnext[Cfg::BlocksM] = {}, sBnext[Cfg::BlocksN] = {};
+                const uint32_t* mxA = nullptr; // dword of (this wave's first block, pair of stages 0, this lane)
+                const uint32_t* mxB = nullptr;
+                // (dword of block b of an operand, pair p, lane l: (((b / 2) * pairs + p) * 64 + l) * 2 + b % 2)
+                auto scalePtr = [&](const void* base, uint32_t firstBlock) {
+                    return static_cast<const uint32_t*>(base) + (static_cast<size_t>(firstBlock / 2u) * mx.pairs * 64u + lane) * 2u + firstBlock % 2u;
+                };
+                auto loadScales32 = [&](uint32_t(&a_)[Cfg::BlocksM], uint32_t(&b_)[Cfg::BlocksN], uint32_t pair) {
+                    // (a wave's blocks start at an even block or are a single one: block i sits i % 2 dwords and
+                    // i / 2 groups on)
+#pragma unroll
+                    for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+                        a_[bi] = mxA[(static_cast<size_t>(bi / 2u) * mx.pairs + pair) * 128u + bi % 2u];
+#pragma unroll
+                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                        b_[bj] = mxB[(static_cast<size_t>(bj / 2u) * mx.pairs + pair) * 128u + bj % 2u];
+                };
+                if constexpr(Cfg::Scaled)
+                {
+                    static_assert(Cfg::BlocksM == 1u || Cfg::BlocksM % 2u == 0u, "a wave's row blocks: one, or whole groups of two");
+                    static_assert(Cfg::BlocksN == 1u || Cfg::BlocksN % 2u == 0u, "a wave's column blocks: one, or whole groups of two");
+                    mxA = scalePtr(mx.a, (row0 + waveM * Cfg::WaveM) / 32u);
+                    mxB = scalePtr(mx.b, (col0 + waveN * Cfg::WaveN) / 32u);
+                    // (in front of the first copies and kept there: the wait for stage 0 then covers these loads,
+                    // and the loop is entered with none of them in flight)
+                    loadScales32(sA, sB, 0u);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 issueStage(0u, 1u < stages);
                 issueStage(1u, 2u < stages);
                 lds::waitCopiesAndReads<Cfg::Copies>(); // stage 0 has landed
                 lds::barrier();
                 constexpr uint32_t N = Cfg::KSteps; // MFMA steps per stage: 2 or 4 (even: the fragment sets alternate)
                 Frags              f[2];
+                auto multiplyStep = [&](Frags const& fr, uint32_t i, uint32_t ks) {
+                    if constexpr(Cfg::Scaled)
+                    {
+#if ROCWMMA_ARCH_GFX950 // (the instruction table exists in the device pass only)
+                        using Op  = detail::MfmaScaled<detail::TypeInfo<InT>::cls, detail::TypeInfo<InT>::cls, 32u>;
+                        using Acc = typename Op::Acc;
+                        const uint32_t shift = 8u * ((i % 2u) * N + ks); // the step's byte within the pair of stages
+#pragma unroll
+                        for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+#pragma unroll
+                            for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                            {
+                                Acc& v = *reinterpret_cast<Acc*>(acc[bi][bj].x);
+                                // (the accumulator is kept transposed: the instruction's first multiplicand is B)
+                                v = Op::template exec<0, 0>(fr.b[bj].x, fr.a[bi].x, v, sB[bj] >> shift, sA[bi] >> shift);
+                            }
+#else
+                        (void)fr, (void)i, (void)ks;
+#endif
+                    }
+                    else
+                    {
+                        (void)i, (void)ks;
+                        multiply(fr);
+                    }
+                };
                 readFrags(f[0], 0u, 0u);
                 for(uint32_t i = 0; i < stages; ++i)
                 {
@@ -690,7 +765,7 @@ namespace rocwmma_amd
                             __builtin_amdgcn_sched_barrier(0);
                         }
                         readFrags(f[(ks + 1u) & 1u], i % 2u, ks + 1u);
-                        multiply(f[ks & 1u]);
+                        multiplyStep(f[ks & 1u], i, ks);
                         scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                         __builtin_amdgcn_sched_barrier(0);
                     }
@@ -699,8 +774,25 @@ namespace rocwmma_amd
                     lds::barrier();
                     __builtin_amdgcn_sched_barrier(0);
                     issueStage(i % 2u, i + 3u < stages);
+                    if constexpr(Cfg::Scaled)
+                    {
+                        if(i % 2u == 0u)
+                            loadScales32(sAnext, sBnext, i / 2u + 1u < mx.pairs ? i / 2u + 1u : mx.pairs - 1u);
+                    }
                     readFrags(f[0], (i + 1u) % 2u, 0u);
-                    multiply(f[(N - 1u) & 1u]);
+                    multiplyStep(f[(N - 1u) & 1u], i, N - 1u);
+                    if constexpr(Cfg::Scaled)
+                    {
+                        if(i % 2u == 1u)
+                        {
+#pragma unroll
+                            for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+                                sA[bi] = sAnext[bi];
+#pragma unroll
+                            for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                                sB[bj] = sBnext[bj];
+                        }
+                    }
                     scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                     scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::Copies>();
                     __builtin_amdgcn_sched_barrier(0);

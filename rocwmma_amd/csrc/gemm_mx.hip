@@ -124,46 +124,104 @@ namespace rocwmma_amd
             return pickBlock<InT, col_major, row_major>(g, s, stream);
         }
 
-        // One thread per (operand, group of 64 rows, pair of K stages, lane): the 8 bytes that lane loads.
-        // Items 0 .. blocksA - 1 re-order A's scales, the others B's; a workgroup of four waves takes four
-        // consecutive items.
+        // Re-orders the scales of both operands for the blocked kernels.  One workgroup per (operand, group
+        // of 64 rows): it reads the group's scale rows in pieces of 128 bytes (4096 elements of K) with
+        // coalesced accesses, each line once, into LDS, and writes from there the 8 bytes every lane of the
+        // GEMM loads per pair of K stages (256 bytes of K):
+        //   16-wide blocks: lane l = row l % 16 of a block, K block l / 16 of a stage; bytes [block 0..3][stage 0..1]
+        //   32-wide blocks: lane l = row l % 32 of a block, K block l / 32 of a step;  bytes [block 0..1][step 0..3]
+        // Rows and K blocks beyond the operand get the scale 1 (they only ever meet zero operands).
+        // (A first version gathered 8 bytes from 8 different scale rows per thread straight from global
+        // memory, one workgroup per group and pair: every 128-byte line was fetched by 16 workgroups on
+        // different XCDs, 7 us for the 1.9 MB of scales of a 4096 x 14336 x 4096 problem.)
+        constexpr uint32_t kPackRowBytes = 128u; // scale bytes of a row per piece
+        constexpr uint32_t kPackRowPitch = 132u; // LDS pitch of a row (byte reads down a column spread over the banks)
+
+        template <bool Wide32>
         __global__ void __launch_bounds__(256) mxPackScalesKernel(MxScales s, uint32_t m, uint32_t n, uint32_t kBlocks, uint32_t pairs,
-                                                                  uint32_t blocksA, uint32_t blocksB, uint2* packedA, uint2* packedB)
+                                                                  uint32_t groupsA, uint2* packedA, uint2* packedB)
         {
-            const uint32_t id = blockIdx.x * 4u + threadIdx.x / 64u;
-            if(id >= blocksA + blocksB)
-                return;
-            const bool     isA     = id < blocksA;
-            const uint32_t item    = isA ? id : id - blocksA;
-            const uint8_t* scales  = isA ? s.a : s.b;
-            const uint32_t ld      = isA ? s.lda : s.ldb;
-            const uint32_t rows    = isA ? m : n;
-            const uint32_t lane    = threadIdx.x % 64u;
-            const uint32_t pair    = item % pairs;
-            const uint32_t group   = item / pairs;
-            uint32_t       word[2] = {0u, 0u};
-#pragma unroll
-            for(uint32_t blk = 0; blk < 4u; ++blk)
-#pragma unroll
-                for(uint32_t st = 0; st < 2u; ++st)
+            __shared__ uint8_t tile[64u * kPackRowPitch];
+            const bool     isA    = blockIdx.x < groupsA;
+            const uint32_t group  = isA ? blockIdx.x : blockIdx.x - groupsA;
+            const uint8_t* scales = isA ? s.a : s.b;
+            const uint32_t ld     = isA ? s.lda : s.ldb;
+            const uint32_t rows   = isA ? m : n;
+            uint2*         packed = isA ? packedA : packedB;
+            const bool     dwords = (reinterpret_cast<uintptr_t>(scales) & 3u) == 0u && ld % 4u == 0u;
+
+            for(uint32_t kb0 = 0; kb0 < pairs * 8u; kb0 += kPackRowBytes)
+            {
+                // 64 rows x 128 bytes -> LDS, consecutive threads along a row
+                for(uint32_t idx = threadIdx.x; idx < 64u * (kPackRowBytes / 4u); idx += 256u)
                 {
-                    const uint32_t row = group * 64u + blk * 16u + lane % 16u;
-                    const uint32_t kb  = (pair * 2u + st) * 4u + lane / 16u;
-                    // (rows and K blocks beyond the operand: never multiplied with anything stored)
-                    const uint32_t e   = (row < rows && kb < kBlocks) ? scales[static_cast<size_t>(row) * ld + kb] : 127u;
-                    word[blk / 2u] |= e << (8u * ((blk % 2u) * 2u + st));
+                    const uint32_t r   = idx / (kPackRowBytes / 4u);
+                    const uint32_t kb  = kb0 + (idx % (kPackRowBytes / 4u)) * 4u;
+                    const uint32_t row = group * 64u + r;
+                    uint32_t       v   = 0x7f7f7f7fu;
+                    if(row < rows && kb < kBlocks)
+                    {
+                        const uint8_t* src = scales + static_cast<size_t>(row) * ld + kb;
+                        if(dwords && kb + 4u <= kBlocks)
+                            v = *reinterpret_cast<const uint32_t*>(src);
+                        else
+                        {
+                            v = 0u;
+#pragma unroll
+                            for(uint32_t j = 0; j < 4u; ++j)
+                                v |= static_cast<uint32_t>(kb + j < kBlocks ? src[j] : 127u) << (8u * j);
+                        }
+                    }
+                    // (pitch 132: 4-byte aligned)
+                    *reinterpret_cast<uint32_t*>(tile + r * kPackRowPitch + (kb - kb0)) = v;
                 }
-            (isA ? packedA : packedB)[static_cast<size_t>(item) * 64u + lane] = make_uint2(word[0], word[1]);
+                __syncthreads();
+                // 16 pairs of stages x 64 lanes x 8 bytes
+                for(uint32_t o = threadIdx.x; o < (kPackRowBytes / 8u) * 64u; o += 256u)
+                {
+                    const uint32_t pairHere = o / 64u, lane = o % 64u;
+                    const uint32_t pair     = kb0 / 8u + pairHere;
+                    if(pair >= pairs)
+                        continue;
+                    uint32_t word[2] = {0u, 0u};
+                    if constexpr(Wide32)
+                    {
+#pragma unroll
+                        for(uint32_t blk = 0; blk < 2u; ++blk)
+#pragma unroll
+                            for(uint32_t step = 0; step < 4u; ++step)
+                                word[blk] |= static_cast<uint32_t>(tile[(blk * 32u + lane % 32u) * kPackRowPitch + pairHere * 8u + step * 2u + lane / 32u])
+                                             << (8u * step);
+                    }
+                    else
+                    {
+#pragma unroll
+                        for(uint32_t blk = 0; blk < 4u; ++blk)
+#pragma unroll
+                            for(uint32_t st = 0; st < 2u; ++st)
+                                word[blk / 2u] |= static_cast<uint32_t>(tile[(blk * 16u + lane % 16u) * kPackRowPitch + pairHere * 8u + st * 4u + lane / 16u])
+                                                  << (8u * ((blk % 2u) * 2u + st));
+                    }
+                    packed[(static_cast<size_t>(group) * pairs + pair) * 64u + lane] = make_uint2(word[0], word[1]);
+                }
+                __syncthreads();
+            }
         }
     } // namespace
 
-    int launchMxPackScales(MxScales const& s, uint32_t m, uint32_t n, uint32_t k, void* packedA, void* packedB, hipStream_t stream)
+    int launchMxPackScales(MxScales const& s, uint32_t m, uint32_t n, uint32_t k, void* packedA, void* packedB, bool wide32,
+                           hipStream_t stream)
     {
         const uint32_t pairs   = (k + 255u) / 256u;
-        const uint32_t blocksA = ((m + 63u) / 64u) * pairs;
-        const uint32_t blocksB = ((n + 63u) / 64u) * pairs;
-        hipLaunchKernelGGL(mxPackScalesKernel, dim3((blocksA + blocksB + 3u) / 4u), dim3(256), 0, stream, s, m, n, k / 32u, pairs,
-                           blocksA, blocksB, static_cast<uint2*>(packedA), static_cast<uint2*>(packedB));
+        const uint32_t groupsA = (m + 63u) / 64u;
+        const uint32_t groupsB = (n + 63u) / 64u;
+        const dim3     grid(groupsA + groupsB);
+        if(wide32)
+            hipLaunchKernelGGL(mxPackScalesKernel<true>, grid, dim3(256), 0, stream, s, m, n, k / 32u, pairs, groupsA,
+                               static_cast<uint2*>(packedA), static_cast<uint2*>(packedB));
+        else
+            hipLaunchKernelGGL(mxPackScalesKernel<false>, grid, dim3(256), 0, stream, s, m, n, k / 32u, pairs, groupsA,
+                               static_cast<uint2*>(packedA), static_cast<uint2*>(packedB));
         return launchStatus();
     }
 

@@ -54,6 +54,40 @@ def test_exact_pattern_with_power_of_two_scales_is_bit_exact(dtype, la, lb, m, n
     check(got, want, 0.0)
 
 
+@pytest.mark.parametrize("dtype", [orc.E4M3, orc.E5M2])
+@pytest.mark.parametrize("m,n,k", [(2048, 4352, 256), (4352, 2048, 384)])
+def test_large_tile_with_half_tiles_for_the_last_round(dtype, m, n, k):
+    """136 tiles of 256 x 256: on a 256-unit device the 256 x 256 / 16x16x128 configuration with every
+    tile of the (only, partly filled) round cut into half tiles.  Exact pattern, bit for bit."""
+    a = exact_int_bits(dtype, m, k, RM)
+    b = exact_int_bits(dtype, k, n, CM)
+    sa, sb = scales(81, m, k, 126, 128), scales(82, n, k, 126, 128)
+    got = run_mx(dtype, RM, CM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0, True)
+    want = orc.gemm_mx(dtype, RM, CM, RM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0)
+    check(got, want, 0.0)
+
+
+@pytest.mark.parametrize("dtype", [orc.E4M3, orc.E5M2])
+@pytest.mark.parametrize("m,n,k", [(48, 14336, 512), (128, 1040, 640), (208, 304, 128), (1024, 768, 1152)])
+def test_mid_size_shapes_on_edge_tiles(dtype, m, n, k):
+    """More than 32 rows, not enough 256 x 256 tiles for half of the device: 128 x 128 tiles of 32x32x64
+    blocks, the last row and column of tiles partly filled.  Exact pattern bit for bit; random operands
+    within the fp8 tolerance."""
+    a = exact_int_bits(dtype, m, k, RM)
+    b = exact_int_bits(dtype, k, n, CM)
+    sa, sb = scales(91, m, k, 126, 128), scales(92, n, k, 126, 128)
+    c = exact_int_bits(orc.F32, m, n, RM)
+    got = run_mx(dtype, RM, CM, RM, m, n, k, a, sa, b, sb, c, 2.0, 3.0, True)
+    want = orc.gemm_mx(dtype, RM, CM, RM, RM, m, n, k, a, sa, b, sb, c, 2.0, 3.0)
+    check(got, want, 0.0)
+    a = uniform_bits(93, dtype, m * k)
+    b = uniform_bits(94, dtype, k * n)
+    sa, sb = scales(95, m, k, 124, 130), scales(96, n, k, 124, 130)
+    got = run_mx(dtype, RM, CM, RM, m, n, k, a, sa, b, sb, None, 0.5, 0.0, True)
+    want = orc.gemm_mx(dtype, RM, CM, RM, RM, m, n, k, a, sa, b, sb, None, 0.5, 0.0)
+    check(got, want, 1e-2)
+
+
 @pytest.mark.parametrize("workspace", [False, True])
 @pytest.mark.parametrize("la,lb,lc", [(RM, CM, RM), (RM, CM, CM), (CM, RM, CM), (CM, CM, RM), (RM, RM, CM)])
 @pytest.mark.parametrize("dtype", [orc.E4M3, orc.E5M2])
