@@ -1227,13 +1227,18 @@ namespace rocwmma_amd
                     if constexpr(std::is_same<OutT, CompT>::value)
                     {
                         // results replace the accumulators, so no two stores share data registers
-#pragma unroll
-                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                        // (integer results with alpha = 1 go out as they are: a 32-bit integer multiply runs at a
+                        // quarter of the rate of the other vector instructions, 128 of them per lane and tile)
+                        if(!(std::is_integral<CompT>::value && !Cfg::Fused && alpha == static_cast<CompT>(1)))
                         {
-                            const BiasOfBlock bv = loadBias(bj);
 #pragma unroll
-                            for(uint32_t e = 0; e < acc[bi][bj].num_elements; ++e)
-                                acc[bi][bj].x[e] = finish(bv, e, alpha * acc[bi][bj].x[e]);
+                            for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                            {
+                                const BiasOfBlock bv = loadBias(bj);
+#pragma unroll
+                                for(uint32_t e = 0; e < acc[bi][bj].num_elements; ++e)
+                                    acc[bi][bj].x[e] = finish(bv, e, alpha * acc[bi][bj].x[e]);
+                            }
                         }
 #pragma unroll
                         for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
