@@ -1227,9 +1227,9 @@ namespace rocwmma_amd
                     if constexpr(std::is_same<OutT, CompT>::value)
                     {
                         // results replace the accumulators, so no two stores share data registers
-                        // (integer results with alpha = 1 go out as they are: a 32-bit integer multiply runs at a
-                        // quarter of the rate of the other vector instructions, 128 of them per lane and tile)
-                        if(!(std::is_integral<CompT>::value && !Cfg::Fused && alpha == static_cast<CompT>(1)))
+                        // (with alpha = 1 they go out as they are: a 32-bit integer multiply runs at a quarter of the
+                        // rate of the other vector instructions, 128 of them per lane and tile)
+                        if(Cfg::Fused || alpha != static_cast<CompT>(1))
                         {
 #pragma unroll
                             for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
