@@ -115,6 +115,17 @@ namespace rocwmma_amd
             static constexpr uint32_t CopiesA    = BytesA / 1024u / Waves; // direct copies per wave per stage
             static constexpr uint32_t CopiesB    = BytesB / 1024u / Waves;
             static constexpr uint32_t Copies     = CopiesA + CopiesB;
+            // With two waves per SIMD only the first wave of each SIMD issues the copies of the main loop, for
+            // itself and for its partner (wave + CopyWaves).  A copy holds its wave's instruction issue for a
+            // dozen cycles; when both waves of a SIMD issue theirs at the same point of the same phase
+            // nothing feeds the matrix pipe meanwhile, with one issuer the partner's MFMAs fill that time
+            // (8192^3, A row-major / B col-major: f16 0.845 -> 0.798 ms, bf16 0.821 -> 0.765; both row-major
+            // 0.906 -> 0.884, both col-major 0.883 -> 0.853; with the second wave of each SIMD as the issuer
+            // 1-5 % slower than that).  A col-major / B row-major (neither K-contiguous: every fragment comes
+            // from transposing reads) is left as it was: 5 % slower with one issuer.
+            static constexpr uint32_t CopyWaves
+                = (Waves == 8u && WavesPerSimd_ == 2u && Stages_ == 2u && (AKMajor || BKMajor)) ? 4u : Waves;
+            static constexpr uint32_t CopyShares = Waves / CopyWaves; // waves whose copies one issuer carries
             // LDS read instructions per MFMA step: b128 reads per block (K-major) or two transposing b64 reads
             static constexpr uint32_t TrReads      = KPackBytes / 8u; // transposing 8-byte reads per operand
             static constexpr uint32_t ReadsA       = BlocksM * (AKMajor ? KPackBytes / 16u : TrReads);
@@ -419,8 +430,15 @@ namespace rocwmma_amd
             const size_t   bStep    = TileB::stageStep(ldbB);
             aSrc += aStep * stage0; // (the whole K range starts at stage 0)
             bSrc += bStep * stage0;
-            const uint32_t aLaneOff = TileA::laneSourceOffset(lane, wave, ldaB);
-            const uint32_t bLaneOff = TileB::laneSourceOffset(lane, wave, ldbB);
+            // (the lane offset of a copy depends on the wave it is issued for through the tile's swizzle: the
+            // K-major tile's is the same for a wave and its partner, the dim-major tiles' are not)
+            uint32_t aLaneOff[Cfg::CopyShares], bLaneOff[Cfg::CopyShares];
+#pragma unroll
+            for(uint32_t j = 0; j < Cfg::CopyShares; ++j)
+            {
+                aLaneOff[j] = TileA::laneSourceOffset(lane, wave % Cfg::CopyWaves + (Cfg::AKMajor ? 0u : j * Cfg::CopyWaves), ldaB);
+                bLaneOff[j] = TileB::laneSourceOffset(lane, wave % Cfg::CopyWaves + (Cfg::BKMajor ? 0u : j * Cfg::CopyWaves), ldbB);
+            }
 
             // A stage is copied in two halves (the A operand, then the B operand) so that each
             // MFMA phase of an iteration carries half of the copy instructions.
@@ -429,22 +447,54 @@ namespace rocwmma_amd
             auto issueA = [&](uint32_t slot, bool advance = true) {
                 char*                 ldsA = ldsRaw + slot * Cfg::StageBytes;
                 const lds::BufferRsrc src  = Cfg::Edges ? lds::makeSource(aSrc, aEnd) : lds::makeSource(aSrc);
-#pragma unroll
-                for(uint32_t i = 0; i < Cfg::CopiesA; ++i)
+                if constexpr(Cfg::CopyWaves < Cfg::Waves)
                 {
-                    const uint32_t copy = i * Cfg::Waves + wave;
-                    lds::asyncCopy16(ldsA + copy * 1024u, src, aLaneOff, TileA::copySourceOffset(copy, ldaB));
+                    if(wave < Cfg::CopyWaves)
+                    {
+#pragma unroll
+                        for(uint32_t i = 0; i < Cfg::CopiesA * Cfg::CopyShares; ++i)
+                        {
+                            // (copy i * CopyWaves + wave = copy i / CopyShares of wave + (i % CopyShares) * CopyWaves)
+                            const uint32_t copy = i * Cfg::CopyWaves + wave;
+                            lds::asyncCopy16(ldsA + copy * 1024u, src, aLaneOff[i % Cfg::CopyShares], TileA::copySourceOffset(copy, ldaB));
+                        }
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for(uint32_t i = 0; i < Cfg::CopiesA; ++i)
+                    {
+                        const uint32_t copy = i * Cfg::Waves + wave;
+                        lds::asyncCopy16(ldsA + copy * 1024u, src, aLaneOff[0], TileA::copySourceOffset(copy, ldaB));
+                    }
                 }
                 aSrc += advance ? aStep : size_t{0};
             };
             auto issueB = [&](uint32_t slot, bool advance = true) {
                 char*                 ldsB = ldsRaw + slot * Cfg::StageBytes + Cfg::BytesA;
                 const lds::BufferRsrc src  = Cfg::Edges ? lds::makeSource(bSrc, bEnd) : lds::makeSource(bSrc);
-#pragma unroll
-                for(uint32_t i = 0; i < Cfg::CopiesB; ++i)
+                if constexpr(Cfg::CopyWaves < Cfg::Waves)
                 {
-                    const uint32_t copy = i * Cfg::Waves + wave;
-                    lds::asyncCopy16(ldsB + copy * 1024u, src, bLaneOff, TileB::copySourceOffset(copy, ldbB));
+                    if(wave < Cfg::CopyWaves)
+                    {
+#pragma unroll
+                        for(uint32_t i = 0; i < Cfg::CopiesB * Cfg::CopyShares; ++i)
+                        {
+                            // (copy i * CopyWaves + wave = copy i / CopyShares of wave + (i % CopyShares) * CopyWaves)
+                            const uint32_t copy = i * Cfg::CopyWaves + wave;
+                            lds::asyncCopy16(ldsB + copy * 1024u, src, bLaneOff[i % Cfg::CopyShares], TileB::copySourceOffset(copy, ldbB));
+                        }
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for(uint32_t i = 0; i < Cfg::CopiesB; ++i)
+                    {
+                        const uint32_t copy = i * Cfg::Waves + wave;
+                        lds::asyncCopy16(ldsB + copy * 1024u, src, bLaneOff[0], TileB::copySourceOffset(copy, ldbB));
+                    }
                 }
                 bSrc += advance ? bStep : size_t{0};
             };
@@ -577,7 +627,7 @@ namespace rocwmma_amd
                 }
                 issueStage(0u, 1u < stages);
                 issueStage(1u, 2u < stages);
-                lds::waitCopiesAndReads<Cfg::Copies>(); // stage 0 has landed
+                lds::waitCopiesAndReads<(Cfg::CopyWaves == Cfg::Waves ? Cfg::Copies : 0u)>(); // stage 0 has landed
                 lds::barrier();
                 typename Cfg::FragA fa[2][Cfg::BlocksM];
                 typename Cfg::FragB fb[2];
@@ -722,7 +772,7 @@ namespace rocwmma_amd
                 }
                 issueStage(0u, 1u < stages);
                 issueStage(1u, 2u < stages);
-                lds::waitCopiesAndReads<Cfg::Copies>(); // stage 0 has landed
+                lds::waitCopiesAndReads<(Cfg::CopyWaves == Cfg::Waves ? Cfg::Copies : 0u)>(); // stage 0 has landed
                 lds::barrier();
                 constexpr uint32_t N = Cfg::KSteps; // MFMA steps per stage: 2 or 4 (even: the fragment sets alternate)
                 Frags              f[2];
