@@ -122,10 +122,11 @@ namespace rocwmma_amd
             // (8192^3, A row-major / B col-major: f16 0.845 -> 0.798 ms, bf16 0.821 -> 0.765; both row-major
             // 0.906 -> 0.884, both col-major 0.883 -> 0.853; with the second wave of each SIMD as the issuer
             // 1-5 % slower than that).  A col-major / B row-major (neither K-contiguous: every fragment comes
-            // from transposing reads) is left as it was: 5 % slower with one issuer.
+            // from transposing reads) is left as it was: 5 % slower with one issuer.  So are the kernels with
+            // block scales: their main loop loads scales into registers, and behind a branch that only some
+            // waves take the compiler waits for every copy in flight before it uses them (five times slower).
             static constexpr uint32_t CopyWaves
-                = (Waves == 8u && WavesPerSimd_ == 2u && Stages_ == 2u && (AKMajor || BKMajor)) ? 4u : Waves;
-            static constexpr uint32_t CopyShares = Waves / CopyWaves; // waves whose copies one issuer carries
+                = (Waves == 8u && WavesPerSimd_ == 2u && Stages_ == 2u && (AKMajor || BKMajor) && !Scaled_) ? 4u : Waves;
             // LDS read instructions per MFMA step: b128 reads per block (K-major) or two transposing b64 reads
             static constexpr uint32_t TrReads      = KPackBytes / 8u; // transposing 8-byte reads per operand
             static constexpr uint32_t ReadsA       = BlocksM * (AKMajor ? KPackBytes / 16u : TrReads);
@@ -432,12 +433,17 @@ namespace rocwmma_amd
             bSrc += bStep * stage0;
             // (the lane offset of a copy depends on the wave it is issued for through the tile's swizzle: the
             // K-major tile's is the same for a wave and its partner, the dim-major tiles' are not)
-            uint32_t aLaneOff[Cfg::CopyShares], bLaneOff[Cfg::CopyShares];
+            // Issuers of the main loop's copies (Cfg::CopyWaves).  The partial tiles of the stream-K kernel keep
+            // every wave issuing its own: with the issuer branch their instances, which already spill, ran
+            // two to five times slower.
+            constexpr uint32_t CopyWaves  = Part == TilePart::Whole ? Cfg::CopyWaves : Cfg::Waves;
+            constexpr uint32_t CopyShares = Cfg::Waves / CopyWaves; // waves whose copies one issuer carries
+            uint32_t aLaneOff[CopyShares], bLaneOff[CopyShares];
 #pragma unroll
-            for(uint32_t j = 0; j < Cfg::CopyShares; ++j)
+            for(uint32_t j = 0; j < CopyShares; ++j)
             {
-                aLaneOff[j] = TileA::laneSourceOffset(lane, wave % Cfg::CopyWaves + (Cfg::AKMajor ? 0u : j * Cfg::CopyWaves), ldaB);
-                bLaneOff[j] = TileB::laneSourceOffset(lane, wave % Cfg::CopyWaves + (Cfg::BKMajor ? 0u : j * Cfg::CopyWaves), ldbB);
+                aLaneOff[j] = TileA::laneSourceOffset(lane, wave % CopyWaves + (Cfg::AKMajor ? 0u : j * CopyWaves), ldaB);
+                bLaneOff[j] = TileB::laneSourceOffset(lane, wave % CopyWaves + (Cfg::BKMajor ? 0u : j * CopyWaves), ldbB);
             }
 
             // A stage is copied in two halves (the A operand, then the B operand) so that each
@@ -447,16 +453,16 @@ namespace rocwmma_amd
             auto issueA = [&](uint32_t slot, bool advance = true) {
                 char*                 ldsA = ldsRaw + slot * Cfg::StageBytes;
                 const lds::BufferRsrc src  = Cfg::Edges ? lds::makeSource(aSrc, aEnd) : lds::makeSource(aSrc);
-                if constexpr(Cfg::CopyWaves < Cfg::Waves)
+                if constexpr(CopyWaves < Cfg::Waves)
                 {
-                    if(wave < Cfg::CopyWaves)
+                    if(wave < CopyWaves)
                     {
 #pragma unroll
-                        for(uint32_t i = 0; i < Cfg::CopiesA * Cfg::CopyShares; ++i)
+                        for(uint32_t i = 0; i < Cfg::CopiesA * CopyShares; ++i)
                         {
                             // (copy i * CopyWaves + wave = copy i / CopyShares of wave + (i % CopyShares) * CopyWaves)
-                            const uint32_t copy = i * Cfg::CopyWaves + wave;
-                            lds::asyncCopy16(ldsA + copy * 1024u, src, aLaneOff[i % Cfg::CopyShares], TileA::copySourceOffset(copy, ldaB));
+                            const uint32_t copy = i * CopyWaves + wave;
+                            lds::asyncCopy16(ldsA + copy * 1024u, src, aLaneOff[i % CopyShares], TileA::copySourceOffset(copy, ldaB));
                         }
                     }
                 }
@@ -474,16 +480,16 @@ namespace rocwmma_amd
             auto issueB = [&](uint32_t slot, bool advance = true) {
                 char*                 ldsB = ldsRaw + slot * Cfg::StageBytes + Cfg::BytesA;
                 const lds::BufferRsrc src  = Cfg::Edges ? lds::makeSource(bSrc, bEnd) : lds::makeSource(bSrc);
-                if constexpr(Cfg::CopyWaves < Cfg::Waves)
+                if constexpr(CopyWaves < Cfg::Waves)
                 {
-                    if(wave < Cfg::CopyWaves)
+                    if(wave < CopyWaves)
                     {
 #pragma unroll
-                        for(uint32_t i = 0; i < Cfg::CopiesB * Cfg::CopyShares; ++i)
+                        for(uint32_t i = 0; i < Cfg::CopiesB * CopyShares; ++i)
                         {
                             // (copy i * CopyWaves + wave = copy i / CopyShares of wave + (i % CopyShares) * CopyWaves)
-                            const uint32_t copy = i * Cfg::CopyWaves + wave;
-                            lds::asyncCopy16(ldsB + copy * 1024u, src, bLaneOff[i % Cfg::CopyShares], TileB::copySourceOffset(copy, ldbB));
+                            const uint32_t copy = i * CopyWaves + wave;
+                            lds::asyncCopy16(ldsB + copy * 1024u, src, bLaneOff[i % CopyShares], TileB::copySourceOffset(copy, ldbB));
                         }
                     }
                 }
@@ -627,7 +633,7 @@ namespace rocwmma_amd
                 }
                 issueStage(0u, 1u < stages);
                 issueStage(1u, 2u < stages);
-                lds::waitCopiesAndReads<(Cfg::CopyWaves == Cfg::Waves ? Cfg::Copies : 0u)>(); // stage 0 has landed
+                lds::waitCopiesAndReads<(CopyWaves == Cfg::Waves ? Cfg::Copies : 0u)>(); // stage 0 has landed
                 lds::barrier();
                 typename Cfg::FragA fa[2][Cfg::BlocksM];
                 typename Cfg::FragB fb[2];
@@ -772,7 +778,7 @@ namespace rocwmma_amd
                 }
                 issueStage(0u, 1u < stages);
                 issueStage(1u, 2u < stages);
-                lds::waitCopiesAndReads<(Cfg::CopyWaves == Cfg::Waves ? Cfg::Copies : 0u)>(); // stage 0 has landed
+                lds::waitCopiesAndReads<(CopyWaves == Cfg::Waves ? Cfg::Copies : 0u)>(); // stage 0 has landed
                 lds::barrier();
                 constexpr uint32_t N = Cfg::KSteps; // MFMA steps per stage: 2 or 4 (even: the fragment sets alternate)
                 Frags              f[2];
