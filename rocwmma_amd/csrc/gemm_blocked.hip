@@ -72,13 +72,29 @@ namespace rocwmma_amd
                         return rc;
                 }
                 using Narrow = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 3>;
+                // The same 128 x 64 tile on a ring of four stages of 128 bytes of K (96 KiB of LDS, one
+                // workgroup per compute unit): a copy requests whole lines, and three stages of 24 KiB are in
+                // flight.  These launches are one round of workgroups that stream their operands from HBM:
+                // 128 x 14336 x 4096 int8 25.1 -> 19.2 us, fp8 27.3 -> 19.5, 256 x 8192 x 8192 int8 41.5 -> 30.9,
+                // f16 74 -> 56; f16 / bf16 128 x 14336 x 4096 within 3 %.  With little K the deeper prologue
+                // costs more than it gains (128 x 14336 x 384 f16 7.0 -> 8.8 us), so from 2 KiB of K per row on.
+                // 16-wide blocks (two MFMA steps per stage) except for fp8, whose 16 x 16 x 128 needs the ring of
+                // two.  (A ring of five: the same.  128 x 128 tiles on this ring, one workgroup per compute
+                // unit, lose to the two-workgroup configurations below: 2048^3 f16 +6 %, 128 x 28672 x 4096 +12 %.)
+                constexpr bool Fp8 = sizeof(InT) == 1u && !std::is_same<InT, int8_t>::value;
+                using NarrowLines = std::conditional_t<!Fp8,
+                                                       BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 4, 2, 4, 1, 16, false, false, false, 128>,
+                                                       BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 1, 32, false, false, false, 128>>;
                 // (up to one 128 x 128 tile per two compute units; with two resident workgroups per
                 // compute unit the 128 x 128 tiling wins from 144 tiles on, fewer bytes per compute
                 // unit: 256 x 14336 x 4096 int8 30 -> 24 us, f16 73 -> 52 us)
                 if(g.m % Small::MacroM == 0u && g.n % Small::MacroN == 0u
                    && 2u * (g.m / Small::MacroM) * (g.n / Small::MacroN) <= computeUnits())
                 {
-                    int rc = launchCfg<Narrow>(g, stream);
+                    int rc = static_cast<size_t>(g.k) * sizeof(InT) >= 2048u ? launchCfg<NarrowLines>(g, stream) : ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+                    if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                        return rc;
+                    rc = launchCfg<Narrow>(g, stream);
                     if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
                         return rc;
                 }

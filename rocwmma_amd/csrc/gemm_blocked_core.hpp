@@ -51,7 +51,8 @@ namespace rocwmma_amd
                   uint32_t BlockEdge_    = 32u, // MFMA block edge: 32 (32x32xK) or 16 (16x16x2K)
                   bool     Edges_        = false, // M and N need not fill whole macro tiles (multiples of 16 do)
                   bool     Scaled_       = false, // fp8 operands with one E8M0 scale per 32 elements of K (MX)
-                  bool     Fused_        = false> // epilogue adds a per-column bias and applies an activation
+                  bool     Fused_        = false, // epilogue adds a per-column bias and applies an activation
+                  uint32_t StageKB_      = 0u> // bytes of K per stage (0: 128 in the ring of two, else 64)
         struct BlockedConfig
         {
             using InT   = InT_;
@@ -83,7 +84,7 @@ namespace rocwmma_amd
             static constexpr uint32_t MacroN  = WavesN * WaveN;
             // bytes of K per pipeline stage: 64 in the ring of four, 128 (whole lines of a K-contiguous
             // operand) in the ring of two
-            static constexpr uint32_t StageKB = Stages_ == 2u ? 128u : 64u;
+            static constexpr uint32_t StageKB = StageKB_ != 0u ? StageKB_ : (Stages_ == 2u ? 128u : 64u);
             static constexpr uint32_t MacroK  = StageKB / sizeof(InT); // K elements per stage
 
             // Fragments of one MFMA step.  BlockK = K of the widest single instruction.

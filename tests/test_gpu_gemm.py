@@ -556,6 +556,29 @@ def test_config3_quantised_inference_shapes(dtype_in, m):
               tol_for(dtype_in))
 
 
+@pytest.mark.parametrize("dtype_in,dtype_out,m,n,k,beta", [
+    (orc.I8, orc.I32, 128, 8448, 2048, 0.0), (orc.I8, orc.I32, 256, 4224, 2112, 2.0),
+    (orc.E4M3, orc.F32, 128, 8448, 2048, 0.0), (orc.E5M2, orc.F32, 128, 8320, 2176, -0.5),
+    (orc.F16, orc.F32, 128, 8448, 1024, 1.0), (orc.F16, orc.F16, 256, 4224, 1088, 0.0),
+    (orc.BF16, orc.F32, 128, 8320, 1152, 0.0),
+])
+def test_blocked_kernel_128x64_tiles_on_whole_line_stages(dtype_in, dtype_out, m, n, k, beta):
+    """One round of 128 x 64 tiles (more than a quarter, at most the number of compute units) with at least
+    2 KiB of K per row, both operands K-contiguous: the ring of four 128-byte stages.  K in whole stages and
+    with half a stage left over (the latter falls back to the 64-byte ring), with and without C."""
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(0x5EED0301, orc.I8, m * k), uniform_bits(0x5EED0302, orc.I8, k * n)
+    elif dtype_in in (orc.E4M3, orc.E5M2):
+        a, b = normal_fp8_bits(0x5EED0301, dtype_in, m * k), normal_fp8_bits(0x5EED0302, dtype_in, k * n)
+    else:
+        a, b = uniform_bits(0x5EED0301, dtype_in, m * k), uniform_bits(0x5EED0302, dtype_in, k * n)
+    c = uniform_bits(0x5EED0303, dtype_out, m * n) if beta else None
+    alpha = 1.0 if dtype_in == orc.I8 else 0.75
+    got = run_gemm(dtype_in, dtype_out, RM, CM, RM, m, n, k, a, b, c, alpha, beta, rw.GEMM_AUTO)
+    want = orc.gemm(dtype_in, dtype_out, RM, CM, RM, RM, m, n, k, a, b, c, alpha, beta)
+    check(dtype_in, dtype_out, got, want, tol_for(dtype_in))
+
+
 # ---------------------------------------------------------------- config 2: 8192^3, 4 layouts x 2 types
 @pytest.mark.parametrize("la", [RM, CM])
 @pytest.mark.parametrize("lb", [RM, CM])
