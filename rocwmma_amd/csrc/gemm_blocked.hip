@@ -118,6 +118,28 @@ namespace rocwmma_amd
                 if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
                     return rc;
             }
+            // Fewer rows than a whole 128 x 64 tile (and other multiples of 16 that leave one partly filled row of
+            // tiles): the same ring of four 128-byte stages with partly filled tiles, when that is one round of
+            // workgroups with enough K to stream.  The rows that are not there cost matrix instructions, not
+            // bytes: 64 x 14336 x 4096 int8 22.1 -> 18.2 us, fp8 24.3 -> 16.4; 96 rows int8 27.0 -> 18.7, fp8
+            // 29.0 -> 17.1, f16 37.8 -> 30.1; 64 x 8192 x 8192 f16 69 -> 55.  Not below 4 KiB of K per row
+            // (64 x 14336 x 2048 int8 9.2 -> 10.1 us), and 16-bit types with up to 64 rows only from 16 KiB
+            // (64 x 14336 x 4096 f16 27.8 -> 31.7 us on it).
+            if constexpr(AK && BK)
+            {
+                constexpr bool Fp8e = sizeof(InT) == 1u && !std::is_same<InT, int8_t>::value;
+                using NarrowLinesEdge = std::conditional_t<!Fp8e,
+                                                           BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 4, 2, 4, 1, 16, true, false, false, 128>,
+                                                           BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 1, 32, true, false, false, 128>>;
+                const uint32_t tiles = ceilDiv(g.m, NarrowLinesEdge::MacroM) * ceilDiv(g.n, NarrowLinesEdge::MacroN);
+                const size_t   minK  = (sizeof(InT) == 2u && g.m <= 64u) ? 16384u : 4096u;
+                if(static_cast<size_t>(g.k) * sizeof(InT) >= minK && tiles <= computeUnits() && 4u * tiles > computeUnits())
+                {
+                    int rc = launchCfg<NarrowLinesEdge>(g, stream);
+                    if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                        return rc;
+                }
+            }
             // multiples of 64 that are not multiples of 128: 64 x 64 tiles, one 32 x 32 block per wave
             // (K-contiguous operands only: the dim-major LDS tile is at least 128 wide)
             if constexpr(AK && BK)

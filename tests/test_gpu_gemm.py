@@ -579,6 +579,28 @@ def test_blocked_kernel_128x64_tiles_on_whole_line_stages(dtype_in, dtype_out, m
     check(dtype_in, dtype_out, got, want, tol_for(dtype_in))
 
 
+@pytest.mark.parametrize("dtype_in,dtype_out,m,n,k,beta", [
+    (orc.I8, orc.I32, 64, 8448, 4096, 0.0), (orc.I8, orc.I32, 112, 4240, 4096, 2.0), (orc.I8, orc.I8, 80, 8320, 4224, 0.0),
+    (orc.E4M3, orc.F32, 80, 8320, 4096, 0.5), (orc.E5M2, orc.F32, 16, 8448, 4224, 0.0),
+    (orc.F16, orc.F32, 96, 8448, 2048, 1.0), (orc.F16, orc.F16, 64, 4176, 8192, 0.0),
+    (orc.BF16, orc.F32, 144, 4224, 2112, 0.0),
+])
+def test_blocked_kernel_partly_filled_128x64_tiles_on_whole_line_stages(dtype_in, dtype_out, m, n, k, beta):
+    """Row counts that leave a partly filled row of 128 x 64 tiles (and an n that leaves a partly filled
+    column), one round of workgroups, at least 4 KiB of K per row, both operands K-contiguous."""
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(0x5EED0311, orc.I8, m * k), uniform_bits(0x5EED0312, orc.I8, k * n)
+    elif dtype_in in (orc.E4M3, orc.E5M2):
+        a, b = normal_fp8_bits(0x5EED0311, dtype_in, m * k), normal_fp8_bits(0x5EED0312, dtype_in, k * n)
+    else:
+        a, b = uniform_bits(0x5EED0311, dtype_in, m * k), uniform_bits(0x5EED0312, dtype_in, k * n)
+    c = uniform_bits(0x5EED0313, dtype_out, m * n) if beta else None
+    alpha = 1.0 if dtype_in == orc.I8 else 0.75
+    got = run_gemm(dtype_in, dtype_out, RM, CM, RM, m, n, k, a, b, c, alpha, beta, rw.GEMM_BLOCKED)
+    want = orc.gemm(dtype_in, dtype_out, RM, CM, RM, RM, m, n, k, a, b, c, alpha, beta)
+    check(dtype_in, dtype_out, got, want, tol_for(dtype_in))
+
+
 # ---------------------------------------------------------------- config 2: 8192^3, 4 layouts x 2 types
 @pytest.mark.parametrize("la", [RM, CM])
 @pytest.mark.parametrize("lb", [RM, CM])
