@@ -152,6 +152,10 @@ namespace rocwmma_amd
     // k a multiple of 128.  256 x 256 tiles of 16-wide blocks when gemmMxBlockedUsesLargeTile(), else 128 x 128
     // tiles of 32-wide blocks: the scales must have been packed for that.
     bool gemmMxBlockedUsesLargeTile(GemmArgs const& args);
+    // True when launchGemmBlocked runs a problem with K-contiguous operands (A row-major, B col-major) of
+    // `elemBytes`-byte elements on partly filled 128 x 64 tiles over the ring of four 128-byte stages:
+    // one round of workgroups with enough K to stream.  (The weight-streaming kernels leave those to it.)
+    bool gemmBlockedTakesPartlyFilledLineTiles(uint32_t m, uint32_t n, uint32_t k, uint32_t elemBytes);
     int  launchGemmMxBlocked(int dtypeIn, GemmArgs const& args, const void* packedA, const void* packedB, hipStream_t stream);
 
     // The blocked kernel with the fused epilogue (float types, row-major C/D; args.bias / args.activation)

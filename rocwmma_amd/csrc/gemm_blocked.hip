@@ -131,9 +131,8 @@ namespace rocwmma_amd
                 using NarrowLinesEdge = std::conditional_t<!Fp8e,
                                                            BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 4, 2, 4, 1, 16, true, false, false, 128>,
                                                            BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 1, 32, true, false, false, 128>>;
-                const uint32_t tiles = ceilDiv(g.m, NarrowLinesEdge::MacroM) * ceilDiv(g.n, NarrowLinesEdge::MacroN);
-                const size_t   minK  = (sizeof(InT) == 2u && g.m <= 64u) ? 16384u : 4096u;
-                if(static_cast<size_t>(g.k) * sizeof(InT) >= minK && tiles <= computeUnits() && 4u * tiles > computeUnits())
+                static_assert(NarrowLinesEdge::MacroM == 128u && NarrowLinesEdge::MacroN == 64u, "gemmBlockedTakesPartlyFilledLineTiles");
+                if(gemmBlockedTakesPartlyFilledLineTiles(g.m, g.n, g.k, sizeof(InT)))
                 {
                     int rc = launchCfg<NarrowLinesEdge>(g, stream);
                     if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
@@ -218,6 +217,14 @@ namespace rocwmma_amd
             return launchCfg<Mid>(g, stream, ex);
         }
     } // namespace
+
+    bool gemmBlockedTakesPartlyFilledLineTiles(uint32_t m, uint32_t n, uint32_t k, uint32_t elemBytes)
+    {
+        const uint32_t tiles  = ceilDiv(m, 128u) * ceilDiv(n, 64u);
+        const size_t   kBytes = static_cast<size_t>(k) * elemBytes;
+        const size_t   minK   = (elemBytes == 2u && m <= 64u) ? 16384u : 4096u;
+        return kBytes % 128u == 0u && kBytes >= minK && tiles <= computeUnits() && 4u * tiles > computeUnits();
+    }
 
     bool gemmMxBlockedUsesLargeTile(GemmArgs const& g)
     {

@@ -502,8 +502,10 @@ namespace rocwmma_amd
             // From 64 rows on the blocked kernel is as fast or faster, in one launch and without atomic adds
             // (its 64 x 64 tiles at 64 rows: 21 against 21 us; its partly filled 128 x 128 tiles at 80, 96,
             // 112 rows of int8 against 14336 x 4096: 25.5, 25.4, 26.4 us against 26.8, 29.0, 32.3 us here);
-            // 48 rows stay (20.8 against 24.6 us).
-            if(g.m >= 64u)
+            // 48 rows stayed (20.8 against 24.6 us) until the blocked kernel got partly filled 128 x 64 tiles on
+            // whole-line stages: where it runs those (one round of workgroups, 4 KiB of K and more) it takes 48
+            // rows as well, 17.7 / 16.9 us int8 / fp8 against 20.9 / 22.5 us here.
+            if(g.m >= 64u || gemmBlockedTakesPartlyFilledLineTiles(g.m, g.n, g.k, E))
                 return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
             // K slices: whole 1 KiB copies per row and whole batches of fragment steps per slice, the
             // A slice within 128 KiB of LDS; as few slices as fill the compute units
