@@ -112,7 +112,8 @@ int rocwmma_amd_device_info(int* compute_units, int* clock_mhz, int* is_gfx950);
  * type in all four A/B layout pairs (m, n that do not fill whole tiles run on partly filled edge tiles)
  * and is chosen automatically, as are the weight-streaming kernels for up to 48 rows of A against a
  * col-major B.
- * One of those (48 rows, or a 16-bit A of 16 / 32 rows too large for the LDS) runs as two launches on the
+ * One of those (48 rows against few columns or little K, or a 16-bit A of 16 / 32 rows too large for the
+ * LDS; wide 48-row problems run on the blocked kernel) runs as two launches on the
  * stream and adds its K slices into D with atomic adds: I32 results are exact, F32 results can differ
  * in the last bit from run to run.
  * Alignment: base pointers and leading dimensions must be multiples of 16 bytes.
