@@ -51,6 +51,13 @@ def library():
         path = library_path()
         if not os.path.exists(path):
             raise RuntimeError(f"{path} is missing: build it with `python rocwmma_amd/build.py`")
+        # PyTorch brings a HIP runtime of its own.  Loaded first, this library would bind to the system's,
+        # and a device made current through one runtime is not current in the other (device_info then
+        # reports that no gfx950 device is current): where PyTorch is installed it is imported first.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(path)
         i, u, vp, f = ctypes.c_int, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_float
         L.rocwmma_amd_version.restype = i
