@@ -601,6 +601,29 @@ def test_blocked_kernel_partly_filled_128x64_tiles_on_whole_line_stages(dtype_in
     check(dtype_in, dtype_out, got, want, tol_for(dtype_in))
 
 
+@pytest.mark.parametrize("m", [128, 80])
+def test_whole_line_128x64_tiles_padded_leading_dimensions_in_place(m):
+    """The 128 x 64 tiles on 128-byte stages (whole, m = 128, and partly filled, m = 80) with padded lda / ldb /
+    ldd and C = D: the window must match the oracle bit for bit (int8), the padding of D must stay untouched."""
+    import torch
+
+    n, k = 4240, 4096
+    lda, ldb, ldd = k + 64, k + 128, n + 48
+    rng = np.random.default_rng(0x5EED0321)
+    A = rng.integers(-128, 128, (m, lda), dtype=np.int8)
+    B = rng.integers(-128, 128, (n, ldb), dtype=np.int8)  # col-major B: n columns of ldb
+    C = rng.integers(-1000, 1000, (m, ldd), dtype=np.int32)
+    d = to_device(C.copy())
+    rw.gemm(orc.I8, orc.I32, RM, CM, RM, m, n, k, to_device(A), to_device(B), d, d, 1.0, 3.0,
+            lda=lda, ldb=ldb, ldc=ldd, ldd=ldd, algo=rw.GEMM_BLOCKED)
+    torch.cuda.synchronize()
+    got = d.cpu().numpy().reshape(m, ldd)
+    want = orc.gemm(orc.I8, orc.I32, RM, CM, RM, RM, m, n, k, np.ascontiguousarray(A[:, :k]), np.ascontiguousarray(B[:, :k]),
+                    np.ascontiguousarray(C[:, :n]), 1.0, 3.0)
+    assert np.array_equal(np.ascontiguousarray(got[:, :n]).reshape(-1), want)
+    assert np.array_equal(got[:, n:], C[:, n:])
+
+
 # ---------------------------------------------------------------- config 2: 8192^3, 4 layouts x 2 types
 @pytest.mark.parametrize("la", [RM, CM])
 @pytest.mark.parametrize("lb", [RM, CM])
