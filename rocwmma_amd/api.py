@@ -25,7 +25,7 @@ ACT_NONE, ACT_RELU, ACT_GELU = range(3)
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
 _AUX_LIB_NAME = "librocwmma_amd_aux.so"
 AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_bench_mfma_ceiling",
-               "rocwmma_amd_bench_stream"]
+               "rocwmma_amd_bench_stream", "rocwmma_amd_bench_phase_trace"]
 (MFMA_F16_16X16X32, MFMA_F16_32X32X16, MFMA_BF16_16X16X32, MFMA_BF16_32X32X16, MFMA_I8_16X16X64, MFMA_I8_32X32X32,
  MFMA_F8_16X16X128, MFMA_F8_32X32X64, MFMA_F8_16X16X128_SCALED) = range(9)
 
@@ -116,6 +116,8 @@ def aux_library():
         L.rocwmma_amd_bench_mfma_ceiling.restype = i
         L.rocwmma_amd_bench_stream.argtypes = [i, vp, vp, ctypes.c_size_t, vp]
         L.rocwmma_amd_bench_stream.restype = i
+        L.rocwmma_amd_bench_phase_trace.argtypes = [i, i, i, u, u, u, vp, vp, vp, vp, f, f, vp, ctypes.c_size_t, vp]
+        L.rocwmma_amd_bench_phase_trace.restype = i
         _aux = L
     return _aux
 
@@ -295,6 +297,14 @@ def bench_stream(mode, src, dst, nbytes, stream=None):
     device tensors or raw addresses."""
     _check(aux_library().rocwmma_amd_bench_stream(mode, _ptr(src), _ptr(dst), nbytes,
                                                   stream if stream is not None else _stream()), "bench_stream")
+
+
+def bench_phase_trace(dtype_in, layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta, trace):
+    """Runs the blocked GEMM's 256 x 256 kernel with time stamps in its main loop (include/rocwmma_amd_aux.h);
+    `trace`: a device tensor of (m / 256) * (n / 256) * 64 int64 words."""
+    _check(aux_library().rocwmma_amd_bench_phase_trace(dtype_in, layout_a, layout_b, m, n, k, _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+                                                       alpha, beta, _ptr(trace), trace.numel() * trace.element_size(), _stream()),
+           "bench_phase_trace")
 
 
 def bench_mfma_ceiling(shape, trips, waves_per_simd, operands, out):

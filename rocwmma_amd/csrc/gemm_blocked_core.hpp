@@ -253,7 +253,19 @@ namespace rocwmma_amd
         {
             MxPacked      mx;
             FusedEpilogue fused;
+#ifdef ROCWMMA_AMD_PHASE_TRACE
+            // Benchmark builds only (phase_trace.hip): where the ring-of-two main loops leave their time stamps,
+            // eight 64-bit words per wave: shader clocks spent in the phase in front of the barrier, in the wait
+            // for copies and LDS reads, at the barrier, in the phase behind it, in the whole loop, and the
+            // number of stages.
+            unsigned long long* trace;
+#endif
         };
+#ifdef ROCWMMA_AMD_PHASE_TRACE
+#define ROCWMMA_AMD_TRACE(...) __VA_ARGS__
+#else
+#define ROCWMMA_AMD_TRACE(...)
+#endif
 
         // ---- stream-K support ------------------------------------------------------------------
         // Which part of a tile's K range a call of gemmTile computes.
@@ -827,6 +839,8 @@ namespace rocwmma_amd
                     }
                 };
                 readFrags(f[0], 0u, 0u);
+                ROCWMMA_AMD_TRACE(unsigned long long trFront = 0, trWait = 0, trBarrier = 0, trBehind = 0;
+                                  const unsigned long long trStart = __builtin_readcyclecounter(); unsigned long long trPrev = trStart;)
                 for(uint32_t i = 0; i < stages; ++i)
                 {
 #pragma unroll
@@ -843,10 +857,15 @@ namespace rocwmma_amd
                         scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                         __builtin_amdgcn_sched_barrier(0);
                     }
+                    ROCWMMA_AMD_TRACE(const unsigned long long tr1 = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0);)
                     lds::waitCopiesAndReads<0u>(); // stage i+1 has landed, stage i is in registers
                     pinFrags(f[(N - 1u) & 1u]);
+                    ROCWMMA_AMD_TRACE(__builtin_amdgcn_sched_barrier(0); const unsigned long long tr2 = __builtin_readcyclecounter();
+                                      __builtin_amdgcn_sched_barrier(0);)
                     lds::barrier();
                     __builtin_amdgcn_sched_barrier(0);
+                    ROCWMMA_AMD_TRACE(const unsigned long long tr3 = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0);
+                                      trFront += tr1 - trPrev, trWait += tr2 - tr1, trBarrier += tr3 - tr2;)
                     issueStage(i % 2u, i + 3u < stages);
                     if constexpr(Cfg::Scaled)
                     {
@@ -870,9 +889,14 @@ namespace rocwmma_amd
                     scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                     scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::Copies>();
                     __builtin_amdgcn_sched_barrier(0);
+                    ROCWMMA_AMD_TRACE(trPrev = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); trBehind += trPrev - tr3;)
                 }
                 lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
                 lds::barrier();
+                ROCWMMA_AMD_TRACE(if(ex.trace && lane == 0u) {
+                    unsigned long long* t = ex.trace + (static_cast<size_t>(blockIdx.x) * Cfg::Waves + wave) * 8u;
+                    t[0] = trFront, t[1] = trWait, t[2] = trBarrier, t[3] = trBehind, t[4] = __builtin_readcyclecounter() - trStart, t[5] = stages;
+                })
             }
             else if constexpr(Cfg::KSteps == 2u)
             {
