@@ -105,9 +105,27 @@ namespace rocwmma_amd
                 // (128 x 64 tiles with a K-contiguous B, 64 x 128 with a K-contiguous A)
                 using Half = std::conditional_t<BK, BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 3>,
                                                 BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 2, 4, 3>>;
+                // The same tiles on the ring of four 128-byte stages (see NarrowLines above) for the 8-bit types with
+                // at least 4 KiB of K per row: 128 x 14336 x 4096 int8 27.5 -> 24.8 us (A row / B row) and 24.8 -> 22.5
+                // (A col / B col), fp8 28.6 -> 24.0 and 26.1 -> 18.6, 256 x 8192 x 8192 int8 41.8 -> 37.6 and 41.5 ->
+                // 36.9.  (f16 / bf16: between 6 % faster and 11 % slower, left on the 64-byte ring; 2 KiB of K: up to
+                // 9 % slower.)
+                constexpr bool Fp8h = sizeof(InT) == 1u && !std::is_same<InT, int8_t>::value;
+                using HalfLines = std::conditional_t<
+                    BK,
+                    std::conditional_t<!Fp8h, BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 4, 2, 4, 1, 16, false, false, false, 128>,
+                                       BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 1, 4, 1, 32, false, false, false, 128>>,
+                    std::conditional_t<!Fp8h, BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 4, 4, 1, 16, false, false, false, 128>,
+                                       BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 1, 2, 4, 1, 32, false, false, false, 128>>>;
                 if(g.m % Small::MacroM == 0u && g.n % Small::MacroN == 0u
                    && 2u * (g.m / Small::MacroM) * (g.n / Small::MacroN) <= computeUnits())
                 {
+                    if constexpr(sizeof(InT) == 1u)
+                    {
+                        const int rcl = g.k >= 4096u ? launchCfg<HalfLines>(g, stream) : ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+                        if(rcl != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                            return rcl;
+                    }
                     int rc = launchCfg<Half>(g, stream);
                     if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
                         return rc;

@@ -601,6 +601,23 @@ def test_blocked_kernel_partly_filled_128x64_tiles_on_whole_line_stages(dtype_in
     check(dtype_in, dtype_out, got, want, tol_for(dtype_in))
 
 
+@pytest.mark.parametrize("la,lb", [(RM, RM), (CM, CM)])
+@pytest.mark.parametrize("dtype_in,m,n,k", [(orc.I8, 128, 8448, 4096), (orc.E4M3, 256, 4224, 4224), (orc.E5M2, 128, 8320, 4096)])
+def test_8bit_types_one_operand_dim_major_on_whole_line_stages(dtype_in, m, n, k, la, lb):
+    """128 x 64 / 64 x 128 tiles with one operand in the other major on the ring of four 128-byte stages:
+    8-bit types, one round of workgroups, at least 4 KiB of K per row."""
+    if dtype_in == orc.I8:
+        a, b = uniform_bits(0x5EED0331, orc.I8, m * k), uniform_bits(0x5EED0332, orc.I8, k * n)
+    else:
+        a, b = normal_fp8_bits(0x5EED0331, dtype_in, m * k), normal_fp8_bits(0x5EED0332, dtype_in, k * n)
+    out = OUT_OF[dtype_in]
+    c = uniform_bits(0x5EED0333, out, m * n)
+    alpha, beta = (1.0, -1.0) if dtype_in == orc.I8 else (0.5, 1.0)
+    got = run_gemm(dtype_in, out, la, lb, RM, m, n, k, a, b, c, alpha, beta, rw.GEMM_BLOCKED)
+    want = orc.gemm(dtype_in, out, la, lb, RM, RM, m, n, k, a, b, c, alpha, beta)
+    check(dtype_in, out, got, want, tol_for(dtype_in))
+
+
 @pytest.mark.parametrize("m", [128, 80])
 def test_whole_line_128x64_tiles_padded_leading_dimensions_in_place(m):
     """The 128 x 64 tiles on 128-byte stages (whole, m = 128, and partly filled, m = 80) with padded lda / ldb /
