@@ -131,6 +131,25 @@ namespace rocwmma_amd
                         return rc;
                 }
             }
+            // fp8, both operands K-contiguous, one round of more than half as many 128 x 128 tiles as there are
+            // compute units, at least 4 KiB of K: the tile on the ring of four 128-byte stages (128 KiB of LDS, one
+            // workgroup per compute unit).  256 x 14336 x 4096 30.9 -> 25.5 us, 2048 x 2048 x 4096 26.2 -> 23.0,
+            // 256 x 16384 x 8192 53.7 -> 42.7, 128 x 28672 x 4096 27.0 -> 24.6; with more tiles than compute units it loses to
+            // the two-workgroup ring of two, 512 x 14336 x 4096 43.6 -> 48.1.  (int8 and the 16-bit types, whose
+            // 32-wide blocks would make four MFMA steps of such a stage, ran it with 16-wide blocks: int8 3 %
+            // faster to 12 % slower, f16 6-12 % slower; they stay on the 64-byte ring.)
+            if constexpr(AK && BK && sizeof(InT) == 1u && !std::is_same<InT, int8_t>::value)
+            {
+                using SmallLines = BlockedConfig<InT, OutT, CompT, AK, BK, 2, 2, 2, 2, 4, 1, 32, false, false, false, 128>;
+                if(g.m % Small::MacroM == 0u && g.n % Small::MacroN == 0u && g.k >= 4096u
+                   && (g.m / Small::MacroM) * (g.n / Small::MacroN) <= computeUnits()
+                   && 2u * (g.m / Small::MacroM) * (g.n / Small::MacroN) > computeUnits())
+                {
+                    int rc = launchCfg<SmallLines>(g, stream);
+                    if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                        return rc;
+                }
+            }
             {
                 int rc = launchByRounds<Small, Small2>(g, stream);
                 if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)

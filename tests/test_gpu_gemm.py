@@ -561,6 +561,8 @@ def test_config3_quantised_inference_shapes(dtype_in, m):
     (orc.E4M3, orc.F32, 128, 8448, 2048, 0.0), (orc.E5M2, orc.F32, 128, 8320, 2176, -0.5),
     (orc.F16, orc.F32, 128, 8448, 1024, 1.0), (orc.F16, orc.F16, 256, 4224, 1088, 0.0),
     (orc.BF16, orc.F32, 128, 8320, 1152, 0.0),
+    # fp8 on 128 x 128 tiles of the same ring: more than half as many tiles as compute units, 4 KiB of K
+    (orc.E4M3, orc.F32, 256, 8320, 4096, 0.5), (orc.E5M2, orc.F32, 384, 5632, 4224, 0.0),
 ])
 def test_blocked_kernel_128x64_tiles_on_whole_line_stages(dtype_in, dtype_out, m, n, k, beta):
     """One round of 128 x 64 tiles (more than a quarter, at most the number of compute units) with at least
