@@ -143,10 +143,22 @@ def _check(rc, where):
         raise RocwmmaError(rc, where)
 
 
-def _stream():
-    import torch
+_raw_stream = None
 
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+def _stream():
+    """The current PyTorch stream of the current device as a raw handle."""
+    global _raw_stream
+    if _raw_stream is None:
+        import torch
+
+        fast = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        if fast is not None:
+            # (no Stream object per call: a launch from Python costs a few microseconds, and this is one of them)
+            _raw_stream = lambda: fast(torch.cuda.current_device())
+        else:
+            _raw_stream = lambda: torch.cuda.current_stream().cuda_stream
+    return ctypes.c_void_p(_raw_stream())
 
 
 def _ptr(t):
