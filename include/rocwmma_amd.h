@@ -9,7 +9,9 @@
  * Conventions (all entry points):
  *   - every pointer is a DEVICE pointer owned by the caller; nothing is allocated or freed;
  *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the null stream) and
- *     the call returns without waiting for it;
+ *     the call returns without waiting for it; a call enqueues kernels only (no memset or copy
+ *     nodes), so it may be recorded into a HIP graph and replayed
+ *     (tests/test_gpu_graph_replay.py);
  *   - leading dimensions are in elements;
  *   - the return value is a rocwmma_amd_status (0 = success); a non-zero status means nothing
  *     was launched.  The reference's hosts exit() on HIP errors (samples/common.hpp:34-46) and
