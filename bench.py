@@ -108,9 +108,6 @@ def parse_args():
                     help="skip the MFMA-only ceiling loops and the all-zero-operand run (counter runs)")
     ap.add_argument("--record-traffic", default=None, metavar="KEY:FAMILY:FETCH:WRITE:COPY_FETCH:COPY_WRITE",
                     help="no GPU work: rewrite the entry of profiles/traffic.json for one case from counter readings")
-    ap.add_argument("--phase-trace", action="store_true",
-                    help="run only the headline GEMM's kernel built with time stamps in its main loop (f16, four layout "
-                         "pairs, and int8) and print where a stage's shader clocks go, per half of the waves")
     ap.add_argument("--only", default=None,
                     help="run one case only: a headline case such as f16_rc (dtype_{r|c}{r|c} = A,B layout) or an "
                          "extra case by its JSON key (gemm_fp8_m4096, gemv_8192x8192_n8, ...): for profiling")
@@ -207,43 +204,6 @@ def main():
         ms = event_ms(lambda: dst.copy_(src), 5, torch)
         print(json.dumps({"calibrate_copy_bytes_each_way": src.numel() * 4, "ms": round(ms, 4),
                           "gbs": round(2 * src.numel() * 4 / ms / 1e6, 1)}))
-        return
-
-    if args.phase_trace:
-        # The 256 x 256 kernel with shader-clock time stamps at the phase boundaries of its ring-of-two loop
-        # (librocwmma_amd_aux.so).  Waves 0-3 of a workgroup are the first wave of each SIMD, waves 4-7 the second.
-        import numpy as np
-
-        rows = {}
-        for tag, code, la, lb in (("f16_rc", rw.F16, RM, CM), ("f16_rr", rw.F16, RM, RM), ("f16_cr", rw.F16, CM, RM),
-                                  ("f16_cc", rw.F16, CM, CM), ("i8_rc", rw.I8, RM, CM)):
-            if code == rw.I8:
-                A = torch.randint(-128, 128, (S * S,), device=dev, dtype=torch.int8, generator=gen)
-                B = torch.randint(-128, 128, (S * S,), device=dev, dtype=torch.int8, generator=gen)
-                C = torch.zeros(S * S, device=dev, dtype=torch.int32)
-            else:
-                A = (torch.rand(S * S, device=dev, generator=gen) * 2 - 1).to(torch.float16)
-                B = (torch.rand(S * S, device=dev, generator=gen) * 2 - 1).to(torch.float16)
-                C = torch.rand(S * S, device=dev, generator=gen) * 2 - 1
-            D = torch.empty_like(C)
-            trace = torch.zeros((S // 256) * (S // 256) * 64, device=dev, dtype=torch.int64)
-            fn = lambda: rw.bench_phase_trace(code, la, lb, S, S, S, A, B, C, D, 1.0, 1.0, trace)
-            fn(), fn()
-            ms = event_ms(fn, max(args.steps, 5), torch)
-            t = trace.cpu().numpy().reshape(-1, 8, 8).astype(np.float64)
-            stages = t[0, 0, 5]
-            per = lambda sel, j: round(float(t[:, sel, j].mean() / stages), 1)
-            rows[tag] = {"ms_with_time_stamps": round(ms, 4), "stages": int(stages),
-                         "clocks_per_stage": round(float(t[:, :, 4].mean() / stages), 1),
-                         "mfma_clocks_per_stage_and_simd": 2048,
-                         "waves_0_3": {"front": per(slice(0, 4), 0), "wait": per(slice(0, 4), 1), "barrier": per(slice(0, 4), 2),
-                                       "behind": per(slice(0, 4), 3)},
-                         "waves_4_7": {"front": per(slice(4, 8), 0), "wait": per(slice(4, 8), 1), "barrier": per(slice(4, 8), 2),
-                                       "behind": per(slice(4, 8), 3)}}
-            del A, B, C, D, trace
-        print(json.dumps({"phase_trace": rows, "size": S, "device": info,
-                          "note": "shader clocks per stage of 128 bytes of K and wave, averaged over the workgroups: phase in "
-                                  "front of the barrier / wait for copies and LDS reads / barrier / phase behind it"}))
         return
 
     if args.only and args.only not in HEADLINE_TAGS:

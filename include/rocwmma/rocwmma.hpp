@@ -260,7 +260,7 @@ namespace rocwmma
             DataT                     x[Traits::Size]; // element array
         };
         static_assert(sizeof(typename Traits::AccessT) == sizeof(typename Traits::StorageT),
-                      "Storage type and access type should be views into the same raw data");
+                      "the packed register view and the element array of a fragment must have the same size");
 
         constexpr static uint32_t num_elements = Traits::Size;
         using element_type                     = DataT;
@@ -282,8 +282,8 @@ namespace rocwmma
                          uint32_t                                                       ldm)
     {
         static_assert(!std::is_same<DataLayoutT, void>::value,
-                      "Must provide layout information. Either statically assign data layout in "
-                      "fragment declaration or use the run-time function overload.");
+                      "this fragment type has no data layout: name one in the fragment's template arguments, or call the "
+                      "overload that takes the layout at run time");
         using Config = detail::FragConfig<MatrixT, BlockM, BlockN, BlockK, DataT>;
         using IO     = typename Config::template IO<DataLayoutT>;
         detail::FragmentMover<IO, DataT>::load(frag.x, data, ldm);
@@ -309,8 +309,8 @@ namespace rocwmma
                           uint32_t                                                             ldm)
     {
         static_assert(!std::is_same<DataLayoutT, void>::value,
-                      "Must provide data layout. Either statically assign data layout in "
-                      "fragment declaration or use the run-time function overload.");
+                      "this fragment type has no data layout: name one in the fragment's template arguments, or call the "
+                      "overload that takes the layout at run time");
         using Config = detail::FragConfig<MatrixT, BlockM, BlockN, BlockK, DataT>;
         using IO     = typename Config::template IO<DataLayoutT>;
         detail::FragmentMover<IO, DataT>::store(data, frag.x, ldm);

@@ -211,12 +211,35 @@ int rocwmma_amd_gemm_streamk(int         dtype_in,
                              void*       stream);
 
 /*
+ * Reports whether a stream-K launch on `workspace` (NULL: the static scratch of
+ * rocwmma_amd_gemm_streamk_static on the current device) gave up waiting since the last query.
+ *
+ * In the stream-K kernel the workgroup that owns a shared tile waits for the workgroups that computed the
+ * other parts of its K range.  Workgroups draw their ranges in the order they start (a ticket counter in
+ * the workspace), and a range only ever waits for ranges of earlier tickets, which compute the awaited
+ * part first and without waiting themselves, so the wait ends whatever order the device starts workgroups
+ * in.  It is bounded all the same (2^22 polls): should it run out, the owner stops waiting, D holds wrong
+ * values for that tile, and the kernel leaves the value 0x54494D45 in the word at byte offset
+ * units * (65536 * 4) + units * 4 of the workspace (units = compute units of the device; the flags
+ * start at units * 65536 * 4).  Launches never clear that word; this call does, after reporting it, so a later launch
+ * cannot hide an earlier failure.  A workspace that has never been written reads as "no time-out" unless
+ * it happens to hold that value.
+ *
+ * Waits for `stream` (the launches to be checked must have been enqueued there or be complete), copies four
+ * bytes to the host, allocates nothing; not for use under graph capture.  *timed_out receives 0 or 1.
+ * Has no counterpart in the reference (its kernels never wait for one another).
+ */
+int rocwmma_amd_gemm_streamk_timed_out(void* workspace, size_t workspace_bytes, void* stream, int* timed_out);
+
+/*
  * rocwmma_amd_gemm_streamk without a workspace argument and without any allocation: for callers that
  * cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses that
  * forbid it).  It has no counterpart in the reference.  The workspace is a static device array inside
  * the library: 64 MiB + 1.25 KiB, enough for devices of up to 256 compute units
  * (ROCWMMA_AMD_SCRATCH_TOO_SMALL on larger ones), which every GPU the library runs on holds until
  * the process ends.  The entry point calls no hipMalloc / hipFree and no allocating library routine;
+ * the first call on a device for a type and layout pair resolves the array's device address and sets the
+ * kernel's LDS attribute (host-side queries, no allocation): make that call outside a graph capture;
  * the flags in the scratch are cleared by a small kernel on `stream` in front of the GEMM.  All calls
  * on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two
  * threads) race, so serialise them, or give the overlapping ones workspaces of their own through

@@ -104,33 +104,6 @@ int rocwmma_amd_bench_mfma_ceiling(int         shape,
  */
 int rocwmma_amd_bench_stream(int mode, const void* src, void* dst, size_t bytes, void* stream);
 
-/*
- * Phase trace of the blocked GEMM's 256 x 256 kernel: D = alpha * A * B + beta * C as rocwmma_amd_gemm
- * computes it for f16 / bf16 (f32 C and D) and int8 (int32 C and D) with dense leading dimensions and a
- * row-major C, m and n multiples of 256, k in whole 128-byte stages, on a build of that kernel that reads
- * the shader clock at the phase boundaries of its main loop.  `trace` (device memory, trace_bytes >=
- * (m / 256) * (n / 256) * 8 waves * 8 words of 8 bytes) receives per wave of every workgroup: clocks in
- * the phase in front of the stage barrier, in the wait for copies and LDS reads, at the barrier, in the
- * phase behind it, in the whole loop, and the number of stages (two words unused).  The time stamps
- * cost a few per cent, so the figures say where a stage's time goes, not how long the product kernel takes.
- * Has no counterpart in the reference.
- */
-int rocwmma_amd_bench_phase_trace(int         dtype_in,
-                                  int         layout_a,
-                                  int         layout_b,
-                                  uint32_t    m,
-                                  uint32_t    n,
-                                  uint32_t    k,
-                                  const void* a,
-                                  const void* b,
-                                  const void* c,
-                                  void*       d,
-                                  float       alpha,
-                                  float       beta,
-                                  void*       trace,
-                                  size_t      trace_bytes,
-                                  void*       stream);
-
 #ifdef __cplusplus
 }
 #endif

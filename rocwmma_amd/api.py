@@ -20,12 +20,13 @@ EXPORTS = [
     "rocwmma_amd_gemm_ex", "rocwmma_amd_gemv", "rocwmma_amd_dlrm_fwd", "rocwmma_amd_dlrm_bwd",
     "rocwmma_amd_gemm_streamk", "rocwmma_amd_gemm_streamk_workspace_size", "rocwmma_amd_gemm_streamk_static",
     "rocwmma_amd_gemm_mx", "rocwmma_amd_gemm_mx_workspace_size", "rocwmma_amd_gemm_bias_act",
+    "rocwmma_amd_gemm_streamk_timed_out",
 ]
 ACT_NONE, ACT_RELU, ACT_GELU = range(3)
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
 _AUX_LIB_NAME = "librocwmma_amd_aux.so"
 AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_bench_mfma_ceiling",
-               "rocwmma_amd_bench_stream", "rocwmma_amd_bench_phase_trace"]
+               "rocwmma_amd_bench_stream"]
 (MFMA_F16_16X16X32, MFMA_F16_32X32X16, MFMA_BF16_16X16X32, MFMA_BF16_32X32X16, MFMA_I8_16X16X64, MFMA_I8_32X32X32,
  MFMA_F8_16X16X128, MFMA_F8_32X32X64, MFMA_F8_16X16X128_SCALED) = range(9)
 
@@ -74,6 +75,8 @@ def library():
         L.rocwmma_amd_gemm_streamk.restype = i
         L.rocwmma_amd_gemm_streamk_static.argtypes = gemm_args
         L.rocwmma_amd_gemm_streamk_static.restype = i
+        L.rocwmma_amd_gemm_streamk_timed_out.argtypes = [vp, ctypes.c_size_t, vp, ctypes.POINTER(i)]
+        L.rocwmma_amd_gemm_streamk_timed_out.restype = i
         L.rocwmma_amd_gemm_bias_act.argtypes = gemm_args[:-1] + [vp, i, vp]
         L.rocwmma_amd_gemm_bias_act.restype = i
         L.rocwmma_amd_gemm_mx.argtypes = [i, i, i, i, u, u, u, vp, u, vp, u, vp, u, vp, u, vp, u, vp, u, f, f, vp, ctypes.c_size_t, vp]
@@ -116,8 +119,6 @@ def aux_library():
         L.rocwmma_amd_bench_mfma_ceiling.restype = i
         L.rocwmma_amd_bench_stream.argtypes = [i, vp, vp, ctypes.c_size_t, vp]
         L.rocwmma_amd_bench_stream.restype = i
-        L.rocwmma_amd_bench_phase_trace.argtypes = [i, i, i, u, u, u, vp, vp, vp, vp, f, f, vp, ctypes.c_size_t, vp]
-        L.rocwmma_amd_bench_phase_trace.restype = i
         _aux = L
     return _aux
 
@@ -228,6 +229,16 @@ def gemm_streamk_static(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n,
     return d
 
 
+def gemm_streamk_timed_out(workspace=None):
+    """rocwmma_amd_gemm_streamk_timed_out: True when an owner's bounded wait ran out in a stream-K launch on
+    `workspace` (None: the library's static scratch) since the last query.  Waits for torch's current stream."""
+    flag = ctypes.c_int(-1)
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check(library().rocwmma_amd_gemm_streamk_timed_out(_ptr(workspace), nbytes, _stream(), ctypes.byref(flag)),
+           "gemm_streamk_timed_out")
+    return bool(flag.value)
+
+
 def gemm_bias_act(dtype_in, dtype_out, layout_a, layout_b, layout_c, m, n, k, a, b, c, d, alpha, beta, bias, activation,
                   lda=None, ldb=None, ldc=None, ldd=None):
     """rocwmma_amd_gemm_bias_act on device tensors: D = act(alpha*A*B + beta*C + bias[column]);
@@ -309,14 +320,6 @@ def bench_stream(mode, src, dst, nbytes, stream=None):
     device tensors or raw addresses."""
     _check(aux_library().rocwmma_amd_bench_stream(mode, _ptr(src), _ptr(dst), nbytes,
                                                   stream if stream is not None else _stream()), "bench_stream")
-
-
-def bench_phase_trace(dtype_in, layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta, trace):
-    """Runs the blocked GEMM's 256 x 256 kernel with time stamps in its main loop (include/rocwmma_amd_aux.h);
-    `trace`: a device tensor of (m / 256) * (n / 256) * 64 int64 words."""
-    _check(aux_library().rocwmma_amd_bench_phase_trace(dtype_in, layout_a, layout_b, m, n, k, _ptr(a), _ptr(b), _ptr(c), _ptr(d),
-                                                       alpha, beta, _ptr(trace), trace.numel() * trace.element_size(), _stream()),
-           "bench_phase_trace")
 
 
 def bench_mfma_ceiling(shape, trips, waves_per_simd, operands, out):

@@ -254,6 +254,15 @@ int rocwmma_amd_gemm_streamk(int         dtype_in,
     return launchGemmStreamK(dtype_in, dtype_out, la, lb, args, workspace, workspace_bytes, asStream(stream));
 }
 
+int rocwmma_amd_gemm_streamk_timed_out(void* workspace, size_t workspace_bytes, void* stream, int* timed_out)
+{
+    if(!timed_out || (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0u))
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return streamKTimedOut(workspace, workspace_bytes, asStream(stream), timed_out);
+}
+
 int rocwmma_amd_gemm_streamk_static(int         dtype_in,
                                     int         dtype_out,
                                     int         layout_a,

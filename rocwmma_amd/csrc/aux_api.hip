@@ -14,7 +14,6 @@ namespace rocwmma_amd
     int benchMfmaCeiling(int shape, uint32_t trips, uint32_t wavesPerSimd, const void* operands, float* out, double* ops,
                          hipStream_t stream);
     int benchStream(int mode, const void* src, void* dst, size_t bytes, hipStream_t stream);
-    int benchPhaseTrace(int dtypeIn, int layoutA, int layoutB, GemmArgs const& g, unsigned long long* trace, hipStream_t stream);
 
     namespace
     {
@@ -105,38 +104,6 @@ int rocwmma_amd_bench_stream(int mode, const void* src, void* dst, size_t bytes,
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
     return benchStream(mode, src, dst, bytes, asStream(stream));
-}
-
-int rocwmma_amd_bench_phase_trace(int         dtype_in,
-                                  int         layout_a,
-                                  int         layout_b,
-                                  uint32_t    m,
-                                  uint32_t    n,
-                                  uint32_t    k,
-                                  const void* a,
-                                  const void* b,
-                                  const void* c,
-                                  void*       d,
-                                  float       alpha,
-                                  float       beta,
-                                  void*       trace,
-                                  size_t      trace_bytes,
-                                  void*       stream)
-{
-    if(!a || !b || !d || !trace || (!c && beta != 0.0f) || !validLayout(layout_a) || !validLayout(layout_b) || m == 0u || n == 0u
-       || k == 0u)
-        return ROCWMMA_AMD_INVALID_ARGUMENT;
-    if(m % 256u != 0u || n % 256u != 0u || (static_cast<size_t>(k) * dtypeSize(dtype_in)) % 128u != 0u)
-        return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-    if(trace_bytes < static_cast<size_t>(m / 256u) * (n / 256u) * 8u * 8u * sizeof(unsigned long long))
-        return ROCWMMA_AMD_INVALID_ARGUMENT;
-    if(!aligned16(a) || !aligned16(b) || (c && !aligned16(c)) || !aligned16(d) || !aligned16(trace))
-        return ROCWMMA_AMD_BAD_ALIGNMENT;
-    if(!isGfx950Current())
-        return ROCWMMA_AMD_NO_DEVICE;
-    const bool ak = layout_a == ROCWMMA_AMD_ROW_MAJOR, bk = layout_b == ROCWMMA_AMD_COL_MAJOR;
-    GemmArgs   args{m, n, k, a, b, c, d, ak ? k : m, bk ? k : n, n, n, alpha, beta, ROCWMMA_AMD_ROW_MAJOR};
-    return benchPhaseTrace(dtype_in, layout_a, layout_b, args, static_cast<unsigned long long*>(trace), asStream(stream));
 }
 
 } // extern "C"

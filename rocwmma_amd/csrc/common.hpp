@@ -124,6 +124,9 @@ namespace rocwmma_amd
     size_t streamKWorkspaceBytes(uint32_t workgroups);
     int    launchGemmStreamK(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, void* workspace,
                              size_t workspaceBytes, hipStream_t stream);
+    // Whether an owner's bounded wait ran out in a launch on this workspace (nullptr: the library's own scratch) since
+    // the last query; waits for `stream` first.
+    int    streamKTimedOut(void* workspace, size_t workspaceBytes, hipStream_t stream, int* timedOut);
     // the same on the library's own scratch (a static device array): allocates nothing
     int    launchGemmStreamKStatic(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& args, hipStream_t stream);
 

@@ -7,20 +7,25 @@
 // two LDS buffers, next K slab prefetched while the current one is multiplied), re-tiled and
 // re-plumbed for CDNA4:
 //
-//   reference (gfx9 params)                      this kernel
-//   macro tile 128 x 128 x 16, 4 waves           256 x 256 x (64 bytes of K) x 4-stage LDS ring, 8 waves
-//                                                (two per SIMD: one keeps the matrix pipe fed
-//                                                while the other waits at a barrier)
-//   wave tile 2 x 2 blocks of 32x32x16 (2 MFMA)  2 x 4 blocks of 32x32, one wide-K MFMA per step
-//   global -> VGPR -> shuffle -> LDS             global -> LDS directly (global_load_lds_dwordx4)
-//   LDS -> VGPR -> shuffle (AOS<->SOA)           swizzled ds_read_b128, or ds_read_b64_tr_b16
+//   reference (gfx9 params)                      this kernel (256 x 256 configuration)
+//   macro tile 128 x 128 x 16, 4 waves           256 x 256 x (128 bytes of K) x ring of two LDS stages, 8 waves
+//                                                (two per SIMD: one keeps the matrix pipe fed while the
+//                                                other issues the stage's copies or waits at the barrier)
+//   wave tile 2 x 2 blocks of 32x32x16 (2 MFMA)  4 x 8 blocks of 16x16, wide-K MFMAs (16x16x32 f16 / bf16,
+//                                                16x16x64 int8, 16x16x128 fp8), 64 per wave and stage
+//   global -> VGPR -> shuffle -> LDS             global -> LDS directly (buffer_load_dwordx4 ... lds), issued by
+//                                                the first wave of each SIMD for itself and its partner
+//   LDS -> VGPR -> shuffle (AOS<->SOA)           swizzled ds_read_b128, or ds_read_b64_tr_b16 / _b8
 //                                                for operands whose K is not contiguous
-//   2 LDS buffers, wait + barrier per step       copies 3 stages ahead, one bare barrier per stage
-//   8 MFMA between barriers                      16 MFMA (128 passes) per wave between barriers
+//   2 LDS buffers, wait + barrier per step       copies one stage ahead, one barrier per 128-byte stage
+//   8 MFMA between barriers                      64 MFMA (1024 clocks of matrix-pipe work) per wave between barriers
 //   C read / D written in fragment layout       C staged through LDS (full-row non-temporal
 //                                                copies), D written in fragment layout
 //   grid (m/128, n/128)                          1-D grid, tiles dealt to XCDs in L2-friendly patches
 //                                                (9 % faster than the plain order at 8192^3)
+//
+// The smaller configurations (128 x 128, 128 x 64, 64 x 64 tiles of 4 waves) come with a ring of four stages
+// of 64 bytes of K (copies three stages ahead), a ring of four stages of 128 bytes, or the ring of two.
 //
 // Column-major C/D is handled by the caller as the transposed problem (D^T = B^T A^T).
 #ifndef ROCWMMA_AMD_CSRC_GEMM_BLOCKED_CORE_HPP
@@ -253,19 +258,7 @@ namespace rocwmma_amd
         {
             MxPacked      mx;
             FusedEpilogue fused;
-#ifdef ROCWMMA_AMD_PHASE_TRACE
-            // Benchmark builds only (phase_trace.hip): where the ring-of-two main loops leave their time stamps,
-            // eight 64-bit words per wave: shader clocks spent in the phase in front of the barrier, in the wait
-            // for copies and LDS reads, at the barrier, in the phase behind it, in the whole loop, and the
-            // number of stages.
-            unsigned long long* trace;
-#endif
         };
-#ifdef ROCWMMA_AMD_PHASE_TRACE
-#define ROCWMMA_AMD_TRACE(...) __VA_ARGS__
-#else
-#define ROCWMMA_AMD_TRACE(...)
-#endif
 
         // ---- stream-K support ------------------------------------------------------------------
         // Which part of a tile's K range a call of gemmTile computes.
@@ -277,11 +270,14 @@ namespace rocwmma_amd
         };
 
         // Workspace of the stream-K kernel: one slot of raw accumulators (MacroM x MacroN x 4 bytes, in
-        // register order) and one flag per workgroup, then one word that records a wait that ran out.
+        // register order) and one flag per workgroup, then one word that records a wait that ran out
+        // (kStreamKTimedOut; never cleared by a launch, only by the query that reports it) and the ticket
+        // counter the workgroups of a launch draw their ranges from.
+        constexpr uint32_t kStreamKTimedOut = 0x54494D45u; // "TIME": a value, not a bit, so that an uninitialised workspace does not read as a time-out
         struct StreamKPart
         {
             char*     slots; // slot i at slots + i * slotBytes
-            uint32_t* flags; // flag i set to 1 once slot i is complete; [workgroups] = time-out marker
+            uint32_t* flags; // flag i set to 1 once slot i is complete; [workgroups] = time-out marker, [workgroups + 1] = tickets
             uint32_t  slotBytes;
             uint32_t  mySlot; // contributor: where the accumulators go
             uint32_t  firstSlot, slotCount; // owner: the slots to add, in this order
@@ -336,7 +332,7 @@ namespace rocwmma_amd
                             __builtin_amdgcn_s_sleep(8);
                             if(++spins > (1u << 22))
                             {
-                                __hip_atomic_store(sk.flags + sk.timeoutWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                __hip_atomic_store(sk.flags + sk.timeoutWord, kStreamKTimedOut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                 break;
                             }
                         }
@@ -367,21 +363,27 @@ namespace rocwmma_amd
             }
         }
 
-        // Main loop schedule (per wave; S = 4 LDS stages of 64 bytes of K, F0/F1 = fragment
-        // register sets of the first / last MFMA step of a stage):
+        // Main loop schedules (per wave), by ring:
         //
-        //   prologue : copies for stages 0..2 in flight; wait for stage 0; barrier; read F0(0)
-        //   iteration i:
-        //       issue copies of stage i+3 (into the ring slot everybody finished reading at
-        //         the barrier of iteration i-1)
-        //       [two-step stages] read F1(i) while the MFMAs of F0(i) run
-        //       wait: stage i+1 landed (copies of stages i+2, i+3 may stay in flight) and own
-        //         LDS reads returned;  barrier
-        //       read F0(i+1) while the MFMAs of the last step of stage i run
+        //   ring of two stages of 128 bytes of K (the 256 x 256 tile; N = 2 or 4 MFMA steps per stage):
+        //     prologue : copies of stages 0 and 1 in flight; wait for stage 0; barrier; read F(0, step 0)
+        //     stage i  : steps 0 .. N-2: read the next step's fragments while this step's MFMAs run
+        //                wait: stage i+1 landed and own LDS reads returned;  barrier
+        //                issue the copies of stage i+2 into stage i's slot, read F(i+1, step 0) while the
+        //                  MFMAs of step N-1 run
+        //     (fp8 16x16x128, one step per stage: the A fragments of a stage are held whole, the B fragments
+        //     stream through column buffers; see that branch)
         //
-        // So every LDS read has a full MFMA step (16 instructions, 512 cycles) to return, every
-        // global -> LDS copy has almost three iterations, and the barrier is the only
-        // synchronisation per stage.
+        //   ring of S = 4 stages (64 or 128 bytes of K; F0 / F1 = fragment sets of a stage's two steps):
+        //     prologue : copies for stages 0..2 in flight; wait for stage 0; barrier; read F0(0)
+        //     stage i  : issue copies of stage i+3 (into the slot everybody finished reading at the
+        //                  barrier of stage i-1); read F1(i) while the MFMAs of F0(i) run
+        //                wait: stage i+1 landed (stages i+2, i+3 may stay in flight) and own LDS reads
+        //                  returned;  barrier
+        //                read F0(i+1) while the MFMAs of F1(i) run
+        //
+        // Every LDS read has a full MFMA step to return, and the barrier is the only synchronisation per
+        // stage.
         // One macro tile (or, with Part != Whole, a part of its K range): tile (tm, tn) of the tile grid,
         // `stages` pipeline stages of K starting at stage `stage0`.
         template <typename Cfg, TilePart Part = TilePart::Whole>
@@ -839,8 +841,6 @@ namespace rocwmma_amd
                     }
                 };
                 readFrags(f[0], 0u, 0u);
-                ROCWMMA_AMD_TRACE(unsigned long long trFront = 0, trWait = 0, trBarrier = 0, trBehind = 0;
-                                  const unsigned long long trStart = __builtin_readcyclecounter(); unsigned long long trPrev = trStart;)
                 for(uint32_t i = 0; i < stages; ++i)
                 {
 #pragma unroll
@@ -857,15 +857,10 @@ namespace rocwmma_amd
                         scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    ROCWMMA_AMD_TRACE(const unsigned long long tr1 = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0);)
                     lds::waitCopiesAndReads<0u>(); // stage i+1 has landed, stage i is in registers
                     pinFrags(f[(N - 1u) & 1u]);
-                    ROCWMMA_AMD_TRACE(__builtin_amdgcn_sched_barrier(0); const unsigned long long tr2 = __builtin_readcyclecounter();
-                                      __builtin_amdgcn_sched_barrier(0);)
                     lds::barrier();
                     __builtin_amdgcn_sched_barrier(0);
-                    ROCWMMA_AMD_TRACE(const unsigned long long tr3 = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0);
-                                      trFront += tr1 - trPrev, trWait += tr2 - tr1, trBarrier += tr3 - tr2;)
                     issueStage(i % 2u, i + 3u < stages);
                     if constexpr(Cfg::Scaled)
                     {
@@ -889,14 +884,9 @@ namespace rocwmma_amd
                     scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                     scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::Copies>();
                     __builtin_amdgcn_sched_barrier(0);
-                    ROCWMMA_AMD_TRACE(trPrev = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); trBehind += trPrev - tr3;)
                 }
                 lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
                 lds::barrier();
-                ROCWMMA_AMD_TRACE(if(ex.trace && lane == 0u) {
-                    unsigned long long* t = ex.trace + (static_cast<size_t>(blockIdx.x) * Cfg::Waves + wave) * 8u;
-                    t[0] = trFront, t[1] = trWait, t[2] = trBarrier, t[3] = trBehind, t[4] = __builtin_readcyclecounter() - trStart, t[5] = stages;
-                })
             }
             else if constexpr(Cfg::KSteps == 2u)
             {

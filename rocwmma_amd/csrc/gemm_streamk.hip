@@ -14,10 +14,15 @@
 //
 // The sums are taken in a fixed order, so results do not change from run to run (int32 results are
 // exact, f32 results differ from the one-tile kernel's only in the rounding of the partial sums).
-// A part that waits looks at workgroups with lower ids only, which the dispatcher started earlier
-// and which compute the awaited part before anything else: no workgroup waits for one that cannot
-// run.  The reference's GEMM hosts have no counterpart (plain 2-D grids,
-// samples/perf_hgemm.cpp:810-812).
+// Deadlock freedom does not lean on the dispatcher's order: a workgroup draws a ticket from a counter
+// in the workspace when it starts, and ranges are numbered against the tickets.  A part that waits
+// looks only at ranges of workgroups with earlier tickets, which are therefore resident, and which
+// compute the awaited part before anything else and without waiting for anyone: no workgroup waits for
+// one that cannot run, whatever order the workgroups start in and whatever else occupies the device.
+// (The whole rounds are dealt by workgroup id, which is what places a tile on an XCD.)  The owner's
+// wait is bounded all the same; a wait that runs out leaves kStreamKTimedOut in the workspace, which
+// rocwmma_amd_gemm_streamk_timed_out reports to the caller.  The reference's GEMM hosts have no
+// counterpart (plain 2-D grids, samples/perf_hgemm.cpp:810-812).
 #include "gemm_blocked_core.hpp"
 
 using namespace rocwmma;
@@ -52,8 +57,16 @@ namespace rocwmma_amd
             const uint32_t splitTiles    = tilesM * tilesN - roundTiles; // tile ids behind them: shared by K range
 
             // this workgroup's range of the (split tile, stage) sequence; ranges are numbered against
-            // the workgroup ids, so the parts a range waits for belong to lower ids
-            const uint32_t range = workgroups - 1u - blockIdx.x;
+            // the order the workgroups start in (a ticket drawn here), so the parts a range waits for
+            // belong to workgroups that are already running
+            extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
+            if(threadIdx.x == 0u)
+                *reinterpret_cast<uint32_t*>(ldsRaw)
+                    = __hip_atomic_fetch_add(flags + workgroups + 1u, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            const uint32_t ticket = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const uint32_t*>(ldsRaw));
+            __syncthreads(); // (the first copies overwrite the word)
+            const uint32_t range = workgroups - 1u - ticket;
             const uint64_t units = static_cast<uint64_t>(splitTiles) * stagesPerTile;
             auto           rangeStart = [&](uint32_t r) { return static_cast<uint32_t>(units * r / workgroups); };
             uint32_t       u    = rangeStart(range);
@@ -108,12 +121,14 @@ namespace rocwmma_amd
             }
         }
 
-        // Clears the flags (and the time-out marker) of a launch.  A kernel, not a memset: the entry
-        // points may be recorded into a HIP graph.
-        __global__ void clearFlagsKernel(uint32_t* flags, uint32_t count)
+        // Clears the flags and the ticket counter of a launch, not the time-out marker between them (a later
+        // launch must not hide an earlier failure: the query clears it).  A kernel, not a memset: the
+        // entry points may be recorded into a HIP graph.
+        __global__ void clearFlagsKernel(uint32_t* flags, uint32_t workgroups)
         {
-            for(uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < count; i += gridDim.x * blockDim.x)
-                flags[i] = 0u;
+            for(uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < workgroups + 2u; i += gridDim.x * blockDim.x)
+                if(i != workgroups)
+                    flags[i] = 0u;
         }
 
         // The 256 x 256 configurations of the one-tile kernel (ring of two 128-byte K stages).
@@ -156,7 +171,7 @@ namespace rocwmma_amd
                                    static_cast<int>(Cfg::LdsBytes))
                != hipSuccess)
                 return ROCWMMA_AMD_LAUNCH_FAILED;
-            hipLaunchKernelGGL(clearFlagsKernel, dim3(1), dim3(256), 0, stream, flags, workgroups + 1u);
+            hipLaunchKernelGGL(clearFlagsKernel, dim3(1), dim3(256), 0, stream, flags, workgroups);
             hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(Cfg::Threads), Cfg::LdsBytes, stream, g.m, g.n, g.k,
                                static_cast<typename Cfg::InT const*>(g.a), static_cast<typename Cfg::InT const*>(g.b),
                                static_cast<typename Cfg::OutT const*>(g.c), static_cast<typename Cfg::OutT*>(g.d), g.lda, g.ldb,
@@ -192,7 +207,7 @@ namespace rocwmma_amd
     namespace
     {
         constexpr uint32_t kScratchWorkgroups = 256u;
-        constexpr size_t   kScratchBytes = static_cast<size_t>(kScratchWorkgroups) * kStreamKSlotBytes + 1280u; // slots + 257 flag words
+        constexpr size_t   kScratchBytes = static_cast<size_t>(kScratchWorkgroups) * kStreamKSlotBytes + 1280u; // slots + 258 words (flags, marker, tickets)
         __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
         void* scratchOfCurrentDevice()
@@ -224,8 +239,37 @@ namespace rocwmma_amd
 
     size_t streamKWorkspaceBytes(uint32_t workgroups)
     {
-        // slots, then the flags and the time-out marker, rounded to 256 bytes
-        return static_cast<size_t>(workgroups) * kStreamKSlotBytes + ((static_cast<size_t>(workgroups) + 1u) * 4u + 255u) / 256u * 256u;
+        // slots, then the flags, the time-out marker and the ticket counter, rounded to 256 bytes
+        return static_cast<size_t>(workgroups) * kStreamKSlotBytes + ((static_cast<size_t>(workgroups) + 2u) * 4u + 255u) / 256u * 256u;
+    }
+
+    int streamKTimedOut(void* workspace, size_t workspaceBytes, hipStream_t stream, int* timedOut)
+    {
+        const uint32_t workgroups = computeUnits();
+        if(!workspace)
+        {
+            if(streamKWorkspaceBytes(workgroups) > kScratchBytes)
+                return ROCWMMA_AMD_SCRATCH_TOO_SMALL;
+            workspace      = scratchOfCurrentDevice();
+            workspaceBytes = kScratchBytes;
+            if(!workspace)
+                return ROCWMMA_AMD_LAUNCH_FAILED;
+        }
+        if(workspaceBytes < streamKWorkspaceBytes(workgroups))
+            return ROCWMMA_AMD_INVALID_ARGUMENT;
+        uint32_t* marker = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + static_cast<size_t>(workgroups) * kStreamKSlotBytes)
+                           + workgroups;
+        uint32_t word = 0u;
+        if(hipStreamSynchronize(stream) != hipSuccess || hipMemcpy(&word, marker, sizeof(word), hipMemcpyDeviceToHost) != hipSuccess)
+            return ROCWMMA_AMD_LAUNCH_FAILED;
+        *timedOut = word == kStreamKTimedOut ? 1 : 0;
+        if(word == kStreamKTimedOut) // reported once
+        {
+            const uint32_t zero = 0u;
+            if(hipMemcpy(marker, &zero, sizeof(zero), hipMemcpyHostToDevice) != hipSuccess)
+                return ROCWMMA_AMD_LAUNCH_FAILED;
+        }
+        return ROCWMMA_AMD_OK;
     }
 
     int launchGemmStreamK(int dtypeIn, int dtypeOut, int layoutA, int layoutB, GemmArgs const& g, void* workspace,

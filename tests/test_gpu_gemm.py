@@ -150,12 +150,15 @@ def test_8bit_types_k_contiguous(dtype_in, algo):
 
 @pytest.mark.parametrize("dtype_in", [orc.I8, orc.E4M3])
 @pytest.mark.parametrize("la,lb", [(RM, RM), (CM, CM), (CM, RM)])
-def test_8bit_types_other_layouts_wave_tile(dtype_in, la, lb):
+@pytest.mark.parametrize("algo", [rw.GEMM_AUTO, rw.GEMM_WAVE_TILE])
+def test_8bit_types_other_layouts_small(dtype_in, la, lb, algo):
+    """A small problem with a dim-major 8-bit operand: whatever AUTO picks for it (the blocked kernel's partly
+    filled tiles), and the wave-tile kernel when asked for by name."""
     m, n, k = 64, 96, 256
     a = uniform_bits(41, orc.I8, m * k) if dtype_in == orc.I8 else normal_fp8_bits(41, dtype_in, m * k)
     b = uniform_bits(42, orc.I8, k * n) if dtype_in == orc.I8 else normal_fp8_bits(42, dtype_in, k * n)
     out = OUT_OF[dtype_in]
-    got = run_gemm(dtype_in, out, la, lb, RM, m, n, k, a, b, None, 1.0, 0.0, rw.GEMM_AUTO)
+    got = run_gemm(dtype_in, out, la, lb, RM, m, n, k, a, b, None, 1.0, 0.0, algo)
     want = orc.gemm(dtype_in, out, la, lb, RM, RM, m, n, k, a, b, None, 1.0, 0.0)
     check(dtype_in, out, got, want, tol_for(dtype_in))
 
@@ -394,11 +397,8 @@ def test_blocked_kernel_tile_ladder(dtype_in, m, n):
 def test_blocked_kernel_more_workgroups_than_compute_units(dtype_in, m, n, k, la, lb):
     """128 x 128 and 64 x 64 tilings with more tiles than a 256-unit device has compute units run on the
     ring of two 128-byte K stages (with K in whole stages; the last case, K = 96, stays on the ring of
-    four); an odd number of stages and every layout pair the types allow."""
-    if dtype_in in (orc.I8, orc.E4M3) and (la, lb) != (RM, CM):
-        pytest.skip("8-bit operands: the blocked kernel takes the K-contiguous pairing only")
-    if (m % 128 != 0) and (la, lb) != (RM, CM):
-        pytest.skip("64 x 64 tiles: K-contiguous operands only")
+    four); an odd number of stages and three layout pairs.  (Multiples of 64 that are not multiples of 128
+    run 64 x 64 tiles with both operands K-contiguous and partly filled 128 x 128 tiles otherwise.)"""
     if dtype_in in (orc.E4M3,):
         a, b = normal_fp8_bits(81, dtype_in, m * k), normal_fp8_bits(82, dtype_in, k * n)
     else:
@@ -448,8 +448,6 @@ def test_blocked_kernel_partly_filled_edge_tiles(dtype_in, dtype_out, m, n, k, l
     allocated to size and framed by a guard region that must stay untouched."""
     import torch
 
-    if dtype_in in (orc.I8, orc.E4M3, orc.E5M2) and (la, lb) != (RM, CM):
-        pytest.skip("8-bit operands: the blocked kernel takes the K-contiguous pairing only")
     if dtype_in in (orc.E4M3, orc.E5M2):
         a, b = normal_fp8_bits(85, dtype_in, m * k), normal_fp8_bits(86, dtype_in, k * n)
     elif dtype_in == orc.I8 and dtype_out == orc.I8:

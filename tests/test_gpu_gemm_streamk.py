@@ -22,14 +22,17 @@ def workspace():
     size = rw.gemm_streamk_workspace_size()
     assert size >= 256 * 256 * 4
     # garbage on purpose: the entry point must not depend on the workspace's contents
-    return torch.randint(0, 255, (size,), dtype=torch.uint8, device="cuda")
+    # (bytes below 0x45: the garbage cannot spell the time-out value)
+    return torch.randint(0, 0x45, (size,), dtype=torch.uint8, device="cuda")
 
 
-def timed_out(workspace):
-    """The kernel's bounded wait records a wait that ran out in the word behind the flags."""
+TIMED_OUT = 0x54494D45  # what a wait that ran out leaves in the workspace (include/rocwmma_amd.h)
+
+
+def marker_word(workspace):
+    """The word behind the flags that records a wait that ran out (offset documented in include/rocwmma_amd.h)."""
     cus = rw.device_info()["compute_units"]
-    flags = workspace[cus * 256 * 256 * 4:].view(__import__("torch").int32)
-    return int(flags[cus].item()) != 0
+    return workspace[cus * 256 * 256 * 4:].view(__import__("torch").int32)[cus:cus + 1]
 
 
 def run_streamk(dtype_in, la, lb, lc, m, n, k, a, b, c, alpha, beta, workspace):
@@ -40,8 +43,7 @@ def run_streamk(dtype_in, la, lb, lc, m, n, k, a, b, c, alpha, beta, workspace):
     d = to_device(sentinel)
     rw.gemm_streamk(dtype_in, dtype_out, la, lb, lc, m, n, k, to_device(a), to_device(b),
                     None if c is None else to_device(c), d, alpha, beta, workspace)
-    torch.cuda.synchronize()
-    assert not timed_out(workspace), "a stream-K owner gave up waiting for a contributor"
+    assert not rw.gemm_streamk_timed_out(workspace), "a stream-K owner gave up waiting for a contributor"
     return to_host(d, orc.storage_dtype(dtype_out))
 
 
@@ -136,3 +138,24 @@ def test_argument_errors(workspace):
     with pytest.raises(rw.RocwmmaError) as e:  # 8-bit operands: K-contiguous pairing only
         rw.gemm_streamk(rw.I8, rw.I32, RM, RM, RM, m, n, k, da, db, None, d.view(torch.int32), 1.0, 0.0, workspace)
     assert e.value.status == 3
+
+
+def test_timed_out_query_reports_once_and_launches_do_not_clear_it(workspace):
+    """No kernel is made to wait: the host itself writes the value a wait that ran out would leave, behind
+    a finished launch.  The next launch must not clear it; the query reports it once and clears it."""
+    import torch
+
+    m, n, k = 1024, 1024, 2048
+    a, b, c = inputs(orc.I8, m, n, k, 0x5EED0733)
+    want = run_streamk(orc.I8, RM, CM, RM, m, n, k, a, b, c, 1.0, 0.0, workspace)  # (asserts: no time-out)
+    assert not rw.gemm_streamk_timed_out(workspace)
+    marker_word(workspace).fill_(TIMED_OUT)
+    torch.cuda.synchronize()
+    d = to_device(np.zeros(m * n, dtype=np.int32))
+    rw.gemm_streamk(orc.I8, orc.I32, RM, CM, RM, m, n, k, to_device(a), to_device(b), None, d, 1.0, 0.0, workspace)
+    assert np.array_equal(to_host(d, np.int32), want)
+    assert rw.gemm_streamk_timed_out(workspace), "a later launch hid an earlier time-out"
+    assert not rw.gemm_streamk_timed_out(workspace), "the query reports a time-out once"
+    with pytest.raises(rw.RocwmmaError) as e:  # a workspace that cannot hold the marker
+        rw.gemm_streamk_timed_out(workspace[:4096])
+    assert e.value.status == 1

@@ -45,3 +45,23 @@ def test_static_scratch_entry_point_two_calls_in_a_row(dtype_in, dtype_out, la, 
     # first call: 20 tiles, every one shared by a dozen workgroups; second call, smaller: 12 tiles
     _both(dtype_in, dtype_out, la, lb, 1280, 1024, 4096, 0x5EED0900, alpha, beta, workspace)
     _both(dtype_in, dtype_out, la, lb, 768, 1024, 3072, 0x5EED0910, alpha, beta, workspace)
+    assert not rw.gemm_streamk_timed_out(None), "a stream-K owner on the static scratch gave up waiting"
+
+
+def test_static_scratch_entry_point_leaves_free_device_memory_unchanged():
+    """After a warm-up call (which resolves the scratch's address and sets the kernel's LDS attribute), calls of
+    the entry point must not change what the device reports as free memory."""
+    import torch
+
+    m, n, k = 1024, 1024, 2048
+    a, b = to_device(uniform_bits(1, orc.I8, m * k)), to_device(uniform_bits(2, orc.I8, k * n))
+    d = torch.empty(m * n, dtype=torch.int32, device="cuda")
+    call = lambda: rw.gemm_streamk_static(orc.I8, orc.I32, RM, CM, RM, m, n, k, a, b, None, d, 1.0, 0.0)
+    call()
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    call()
+    call()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
