@@ -97,10 +97,14 @@ int rocwmma_amd_bench_mfma_ceiling(int         shape,
 
 /*
  * Memory-stream ceiling probe: one plain kernel that reads (mode 0), writes (mode 1) or copies (mode 2)
- * `bytes` bytes (a multiple of 32 KiB) with 16-byte accesses, 16 workgroups of 256 threads per compute
- * unit.  mode 0 reads `src` (and needs 4 writable bytes at `dst`), mode 1 writes `dst`, mode 2 copies
- * `src` to `dst`.  The bandwidth-bound workloads are priced against what this reaches for their byte
- * counts on the same device.  Has no counterpart in the reference.
+ * `bytes` bytes (a multiple of 64 KiB) with 16-byte accesses (reads: 16 workgroups of 256 threads per compute
+ * unit; writes and copies: workgroups of 1024 threads; each tuned by a sweep over accesses per lane, workgroup
+ * size and count, plain / non-temporal accesses).  mode 0 reads `src` (and needs 4 writable bytes at `dst`),
+ * mode 1 writes `dst`, mode 2 copies `src` to `dst`, mode 3 copies `src` to `dst` and reads a tenth as much again
+ * from the `bytes` bytes behind `src`'s first `bytes` (so `src` holds 2 * bytes; 4 writable bytes behind `dst`'s
+ * `bytes`): 1.1 bytes read per byte written, the mix of the DLRM backward pass.  The bandwidth-bound workloads
+ * are priced against what this reaches for their byte counts on the same device.  Has no counterpart in the
+ * reference.
  */
 int rocwmma_amd_bench_stream(int mode, const void* src, void* dst, size_t bytes, void* stream);
 

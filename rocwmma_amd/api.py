@@ -312,7 +312,7 @@ def selftest_coop_gemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta):
     return d
 
 
-STREAM_READ, STREAM_WRITE, STREAM_COPY = 0, 1, 2
+STREAM_READ, STREAM_WRITE, STREAM_COPY, STREAM_COPY_READ_MORE = 0, 1, 2, 3
 
 
 def bench_stream(mode, src, dst, nbytes, stream=None):

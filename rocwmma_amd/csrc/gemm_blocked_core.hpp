@@ -1157,6 +1157,26 @@ namespace rocwmma_amd
                 }
                 return bv;
             };
+            // With 16-wide blocks a wave's bias values (four per block and lane) are few enough to be fetched once,
+            // in front of everything else the epilogue requests, and kept for every row of blocks; fetched per
+            // block, each load's latency sat in front of that block's stores (8192^3 f16 with a bias: +26 us,
+            // hoisted: +3 us).  The 32-wide blocks (16 values per block and lane) keep the per-block loads: held
+            // for all blocks they spilled.
+            constexpr bool HoistBias = Cfg::Fused && 4u * Runs * Cfg::BlocksN <= 32u;
+            BiasOfBlock    biasRow[HoistBias ? Cfg::BlocksN : 1u];
+            if constexpr(HoistBias)
+            {
+#pragma unroll
+                for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                    biasRow[bj] = loadBias(bj);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            auto biasOf = [&](uint32_t bj) {
+                if constexpr(HoistBias)
+                    return biasRow[bj];
+                else
+                    return loadBias(bj);
+            };
             auto finish = [&](BiasOfBlock const& bv, uint32_t e, CompT v) -> CompT {
                 if constexpr(Cfg::Fused)
                     return applyActivation(v + bv.v[e], ex.fused.activation);
@@ -1244,7 +1264,7 @@ namespace rocwmma_amd
 #pragma unroll
                         for(uint32_t bj = 0; bj < GB; ++bj)
                         {
-                            const BiasOfBlock bv = loadBias(bj0 + bj);
+                            const BiasOfBlock bv = biasOf(bj0 + bj);
 #pragma unroll
                             for(uint32_t e = 0; e < io[bj].num_elements; ++e)
                                 acc[bi][bj0 + bj].x[e]
@@ -1284,7 +1304,7 @@ namespace rocwmma_amd
                     for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
                     {
                         auto& io = fc[bi % 2u][bj];
-                        const BiasOfBlock bv = loadBias(bj);
+                        const BiasOfBlock bv = biasOf(bj);
 #pragma unroll
                         for(uint32_t e = 0; e < io.num_elements; ++e)
                             io.x[e] = static_cast<OutT>(finish(bv, e, alpha * acc[bi][bj].x[e] + beta * static_cast<CompT>(io.x[e])));
@@ -1322,7 +1342,7 @@ namespace rocwmma_amd
 #pragma unroll
                             for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
                             {
-                                const BiasOfBlock bv = loadBias(bj);
+                                const BiasOfBlock bv = biasOf(bj);
 #pragma unroll
                                 for(uint32_t e = 0; e < acc[bi][bj].num_elements; ++e)
                                     acc[bi][bj].x[e] = finish(bv, e, alpha * acc[bi][bj].x[e]);
@@ -1338,7 +1358,7 @@ namespace rocwmma_amd
 #pragma unroll
                         for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
                         {
-                            const BiasOfBlock bv = loadBias(bj);
+                            const BiasOfBlock bv = biasOf(bj);
 #pragma unroll
                             for(uint32_t e = 0; e < fd[bj].num_elements; ++e)
                                 fd[bj].x[e] = static_cast<OutT>(finish(bv, e, alpha * acc[bi][bj].x[e]));

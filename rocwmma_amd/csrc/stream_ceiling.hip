@@ -32,45 +32,71 @@ namespace rocwmma_amd
                 sink[0] = acc;
         }
 
-        __global__ void __launch_bounds__(kStreamThreads) streamWriteKernel(u32x4* __restrict__ dst, size_t vecs)
+        // Write and copy: workgroups of 1024 threads, four 16-byte accesses per lane and trip.  The variants were
+        // swept over 1-16 accesses per lane, 256-1024 threads, 2-64 workgroups per compute unit and plain /
+        // non-temporal accesses on 1.75 GiB: the write reaches most with plain stores and one workgroup per
+        // compute unit (5.9 TB/s; one access per lane on 16 workgroups of 256 threads per unit: 4.0), the copy
+        // with non-temporal loads and stores on 8 workgroups per unit (5.75 TB/s; plain stores, 256 threads: 5.0).
+        constexpr uint32_t kWideThreads = 1024;
+        constexpr uint32_t kWideUnroll  = 4;
+
+        __global__ void __launch_bounds__(kWideThreads) streamWriteKernel(u32x4* __restrict__ dst, size_t vecs)
         {
-            size_t       i      = static_cast<size_t>(blockIdx.x) * kStreamThreads + threadIdx.x;
-            const size_t stride = static_cast<size_t>(gridDim.x) * kStreamThreads;
+            size_t       i      = static_cast<size_t>(blockIdx.x) * kWideThreads * kWideUnroll + threadIdx.x;
+            const size_t stride = static_cast<size_t>(gridDim.x) * kWideThreads * kWideUnroll;
             const u32x4  v      = {1u, 2u, 3u, 4u};
-            for(; i < vecs; i += stride)
-                dst[i] = v;
+            for(; i + kWideThreads * (kWideUnroll - 1u) < vecs; i += stride)
+#pragma unroll
+                for(uint32_t u = 0; u < kWideUnroll; ++u)
+                    dst[i + u * kWideThreads] = v;
         }
 
-        __global__ void __launch_bounds__(kStreamThreads)
-            streamCopyKernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t vecs)
+        // ExtraReads: every tenth trip also reads a trip's worth of data that is not written anywhere (from the
+        // `vecs` vectors behind the copied ones): 1.1 bytes read per byte written, the mix of the DLRM backward
+        // pass (7870 bytes read, 7168 written per sample), which a plain 1 : 1 copy slightly under-prices because
+        // reads are the cheaper half.
+        template <bool ExtraReads>
+        __global__ void __launch_bounds__(kWideThreads)
+            streamCopyKernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t vecs, uint32_t* sink)
         {
-            constexpr uint32_t U      = 4;
-            size_t             i      = static_cast<size_t>(blockIdx.x) * kStreamThreads * U + threadIdx.x;
-            const size_t       stride = static_cast<size_t>(gridDim.x) * kStreamThreads * U;
-            for(; i + kStreamThreads * (U - 1u) < vecs; i += stride)
+            size_t       i      = static_cast<size_t>(blockIdx.x) * kWideThreads * kWideUnroll + threadIdx.x;
+            const size_t stride = static_cast<size_t>(gridDim.x) * kWideThreads * kWideUnroll;
+            uint32_t     acc    = 0;
+            for(uint32_t trip = blockIdx.x; i + kWideThreads * (kWideUnroll - 1u) < vecs; i += stride, ++trip)
             {
-                u32x4 v[U];
+                u32x4 v[kWideUnroll];
 #pragma unroll
-                for(uint32_t u = 0; u < U; ++u)
-                    v[u] = __builtin_nontemporal_load(src + i + u * kStreamThreads);
+                for(uint32_t u = 0; u < kWideUnroll; ++u)
+                    v[u] = __builtin_nontemporal_load(src + i + u * kWideThreads);
+                if(ExtraReads && trip % 10u == 0u)
+                {
 #pragma unroll
-                for(uint32_t u = 0; u < U; ++u)
-                    dst[i + u * kStreamThreads] = v[u];
+                    for(uint32_t u = 0; u < kWideUnroll; ++u)
+                    {
+                        const u32x4 x = __builtin_nontemporal_load(src + vecs + i + u * kWideThreads);
+                        acc += x[0] ^ x[1] ^ x[2] ^ x[3];
+                    }
+                }
+#pragma unroll
+                for(uint32_t u = 0; u < kWideUnroll; ++u)
+                    __builtin_nontemporal_store(v[u], dst + i + u * kWideThreads);
             }
+            if(ExtraReads && acc == 0x12345678u) // (keeps the extra loads alive; practically never true)
+                sink[0] = acc;
         }
     } // namespace
 
-    // mode 0: read `bytes` from src; 1: write `bytes` to dst; 2: copy `bytes` from src to dst.
-    // bytes must be a multiple of 32 KiB (whole trips of the unrolled loops for every workgroup size used).
+    // mode 0: read `bytes` from src; 1: write `bytes` to dst; 2: copy `bytes` from src to dst; 3: copy with a tenth more reads.
+    // bytes must be a multiple of 64 KiB (whole trips of the unrolled loops for every workgroup size used).
     int benchStream(int mode, const void* src, void* dst, size_t bytes, hipStream_t stream)
     {
-        if(bytes == 0u || bytes % 32768u != 0u)
+        if(bytes == 0u || bytes % 65536u != 0u)
             return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
         const size_t   vecs = bytes / 16u;
         const uint32_t cus  = computeUnits();
         // enough workgroups to keep every compute unit's request queues full, but no more trips than data
-        const size_t   perTrip = static_cast<size_t>(kStreamThreads) * (mode == 0 ? kStreamUnroll : (mode == 2 ? 4u : 1u));
-        size_t         grid    = static_cast<size_t>(cus) * 16u;
+        const size_t   perTrip = mode == 0 ? static_cast<size_t>(kStreamThreads) * kStreamUnroll : static_cast<size_t>(kWideThreads) * kWideUnroll;
+        size_t         grid    = static_cast<size_t>(cus) * (mode == 0 ? 16u : (mode >= 2 ? 8u : 1u));
         if(grid > vecs / perTrip)
             grid = vecs / perTrip;
         if(grid == 0u)
@@ -86,14 +112,21 @@ namespace rocwmma_amd
         case 1:
             if(!dst)
                 return ROCWMMA_AMD_INVALID_ARGUMENT;
-            hipLaunchKernelGGL(streamWriteKernel, dim3(static_cast<uint32_t>(grid)), dim3(kStreamThreads), 0, stream,
+            hipLaunchKernelGGL(streamWriteKernel, dim3(static_cast<uint32_t>(grid)), dim3(kWideThreads), 0, stream,
                                static_cast<u32x4*>(dst), vecs);
             break;
         case 2:
             if(!src || !dst)
                 return ROCWMMA_AMD_INVALID_ARGUMENT;
-            hipLaunchKernelGGL(streamCopyKernel, dim3(static_cast<uint32_t>(grid)), dim3(kStreamThreads), 0, stream,
-                               static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), vecs);
+            hipLaunchKernelGGL(streamCopyKernel<false>, dim3(static_cast<uint32_t>(grid)), dim3(kWideThreads), 0, stream,
+                               static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), vecs, static_cast<uint32_t*>(nullptr));
+            break;
+        case 3: // copy `bytes` and read a tenth as much again from behind them (src holds 2 * bytes; 4 bytes of dst + bytes are the sink)
+            if(!src || !dst)
+                return ROCWMMA_AMD_INVALID_ARGUMENT;
+            hipLaunchKernelGGL(streamCopyKernel<true>, dim3(static_cast<uint32_t>(grid)), dim3(kWideThreads), 0, stream,
+                               static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), vecs,
+                               reinterpret_cast<uint32_t*>(static_cast<char*>(dst) + bytes));
             break;
         default:
             return ROCWMMA_AMD_INVALID_ARGUMENT;
