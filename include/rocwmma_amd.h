@@ -356,6 +356,60 @@ int rocwmma_amd_gemm_mx(int         dtype_in,
                         void*       stream);
 
 /*
+ * The two halves of rocwmma_amd_gemm_mx's blocked path as calls of their own, for callers whose scales
+ * outlive a call (a weight matrix multiplied again and again): re-ordering the scales takes a launch of
+ * its own (6-7 us for the 1.9 MB of scales of a 4096 x 14336 x 4096 problem), a fifth of the time of a
+ * 128-row problem.  They have no counterpart in the reference.
+ *
+ * rocwmma_amd_gemm_mx_pack_scales re-orders the scales of a problem of this shape and these layouts into
+ * `workspace` (as for rocwmma_amd_gemm_mx: 256-byte aligned, at least rocwmma_amd_gemm_mx_workspace_size
+ * bytes).  scale_a or scale_b may be NULL: that operand's part of the workspace is left as it is (pack the
+ * weights' scales once, the tokens' scales per call).  The packed order depends on m, n and k (which tile
+ * the GEMM will run on), so a workspace serves calls with the shape it was packed for.
+ * ROCWMMA_AMD_UNSUPPORTED_SHAPE for problems the blocked kernels do not take (see rocwmma_amd_gemm_mx:
+ * row-major A / col-major B, or the transposed pairing for a col-major C; m, n multiples of 16; k a
+ * multiple of 128).
+ *
+ * rocwmma_amd_gemm_mx_packed is rocwmma_amd_gemm_mx on a workspace filled by rocwmma_amd_gemm_mx_pack_scales
+ * for the same m, n, k and layouts: one launch, the GEMM.  It does not write the workspace, so calls that
+ * share one may overlap.  Same shape rule; it never falls back to another kernel.
+ */
+int rocwmma_amd_gemm_mx_pack_scales(int         layout_a,
+                                    int         layout_b,
+                                    int         layout_c,
+                                    uint32_t    m,
+                                    uint32_t    n,
+                                    uint32_t    k,
+                                    const void* scale_a,
+                                    uint32_t    ld_scale_a,
+                                    const void* scale_b,
+                                    uint32_t    ld_scale_b,
+                                    void*       workspace,
+                                    size_t      workspace_bytes,
+                                    void*       stream);
+
+int rocwmma_amd_gemm_mx_packed(int         dtype_in,
+                               int         layout_a,
+                               int         layout_b,
+                               int         layout_c,
+                               uint32_t    m,
+                               uint32_t    n,
+                               uint32_t    k,
+                               const void* a,
+                               uint32_t    lda,
+                               const void* b,
+                               uint32_t    ldb,
+                               const void* c,
+                               uint32_t    ldc,
+                               void*       d,
+                               uint32_t    ldd,
+                               float       alpha,
+                               float       beta,
+                               const void* workspace,
+                               size_t      workspace_bytes,
+                               void*       stream);
+
+/*
  * Skinny GEMV / GEMM:  Y = alpha * A * X + beta * Y,  in place on Y.
  *
  * Stands in for sgemv_rocwmma_d and its host (samples/simple_sgemv.cpp:103-155,207-227), whose

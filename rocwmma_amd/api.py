@@ -20,7 +20,7 @@ EXPORTS = [
     "rocwmma_amd_gemm_ex", "rocwmma_amd_gemv", "rocwmma_amd_dlrm_fwd", "rocwmma_amd_dlrm_bwd",
     "rocwmma_amd_gemm_streamk", "rocwmma_amd_gemm_streamk_workspace_size", "rocwmma_amd_gemm_streamk_static",
     "rocwmma_amd_gemm_mx", "rocwmma_amd_gemm_mx_workspace_size", "rocwmma_amd_gemm_bias_act",
-    "rocwmma_amd_gemm_streamk_timed_out",
+    "rocwmma_amd_gemm_streamk_timed_out", "rocwmma_amd_gemm_mx_pack_scales", "rocwmma_amd_gemm_mx_packed",
 ]
 ACT_NONE, ACT_RELU, ACT_GELU = range(3)
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
@@ -83,6 +83,10 @@ def library():
         L.rocwmma_amd_gemm_mx_workspace_size.argtypes = [u, u, u]
         L.rocwmma_amd_gemm_mx_workspace_size.restype = ctypes.c_size_t
         L.rocwmma_amd_gemm_mx.restype = i
+        L.rocwmma_amd_gemm_mx_pack_scales.argtypes = [i, i, i, u, u, u, vp, u, vp, u, vp, ctypes.c_size_t, vp]
+        L.rocwmma_amd_gemm_mx_pack_scales.restype = i
+        L.rocwmma_amd_gemm_mx_packed.argtypes = [i, i, i, i, u, u, u, vp, u, vp, u, vp, u, vp, u, f, f, vp, ctypes.c_size_t, vp]
+        L.rocwmma_amd_gemm_mx_packed.restype = i
         L.rocwmma_amd_gemm_streamk_workspace_size.argtypes = []
         L.rocwmma_amd_gemm_streamk_workspace_size.restype = ctypes.c_size_t
         L.rocwmma_amd_gemv.argtypes = [u, u, u, vp, u, vp, u, vp, u, f, f, vp]
@@ -277,6 +281,32 @@ def gemm_mx(dtype_in, layout_a, layout_b, layout_c, m, n, k, a, scale_a, b, scal
                                        alpha, beta, _ptr(workspace),
                                        0 if workspace is None else workspace.numel() * workspace.element_size(), _stream())
     _check(rc, "gemm_mx")
+    return d
+
+
+def gemm_mx_pack_scales(layout_a, layout_b, layout_c, m, n, k, scale_a, scale_b, workspace, ld_scale_a=None, ld_scale_b=None):
+    """rocwmma_amd_gemm_mx_pack_scales: re-orders the scales of a problem into `workspace` for gemm_mx_packed;
+    scale_a or scale_b may be None (that operand's part of the workspace is left as it is)."""
+    rc = library().rocwmma_amd_gemm_mx_pack_scales(layout_a, layout_b, layout_c, m, n, k, _ptr(scale_a),
+                                                   ld_scale_a if ld_scale_a is not None else k // 32, _ptr(scale_b),
+                                                   ld_scale_b if ld_scale_b is not None else k // 32, _ptr(workspace),
+                                                   workspace.numel() * workspace.element_size(), _stream())
+    _check(rc, "gemm_mx_pack_scales")
+    return workspace
+
+
+def gemm_mx_packed(dtype_in, layout_a, layout_b, layout_c, m, n, k, a, b, c, d, alpha, beta, workspace,
+                   lda=None, ldb=None, ldc=None, ldd=None):
+    """rocwmma_amd_gemm_mx_packed: the block-scaled GEMM on a workspace filled by gemm_mx_pack_scales."""
+    lda = lda if lda is not None else (k if layout_a == ROW_MAJOR else m)
+    ldb = ldb if ldb is not None else (n if layout_b == ROW_MAJOR else k)
+    nat = n if layout_c == ROW_MAJOR else m
+    ldc = ldc if ldc is not None else nat
+    ldd = ldd if ldd is not None else nat
+    rc = library().rocwmma_amd_gemm_mx_packed(dtype_in, layout_a, layout_b, layout_c, m, n, k, _ptr(a), lda, _ptr(b), ldb,
+                                              _ptr(c), ldc, _ptr(d), ldd, alpha, beta, _ptr(workspace),
+                                              workspace.numel() * workspace.element_size(), _stream())
+    _check(rc, "gemm_mx_packed")
     return d
 
 

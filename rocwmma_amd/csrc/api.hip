@@ -334,6 +334,32 @@ int rocwmma_amd_gemm_bias_act(int          dtype_in,
     return launchGemmWaveTile(dtype_in, dtype_out, layout_a, layout_b, args, asStream(stream));
 }
 
+namespace
+{
+    // The blocked block-scaled kernels take: row-major A / col-major B for a row-major C (the transposed
+    // problem for a col-major C), k in whole 128-byte stages, operand spans inside a copy's window.
+    // Fills in the problem as those kernels see it (and the scales swapped with it).
+    bool mxBlockedProblem(int layout_a, int layout_b, GemmArgs const& args, MxScales const& scales, GemmArgs& blocked, MxScales& sc)
+    {
+        blocked = args;
+        sc      = scales;
+        int la = layout_a, lb = layout_b;
+        if(blocked.layoutC == ROCWMMA_AMD_COL_MAJOR)
+        {
+            std::swap(sc.a, sc.b);
+            std::swap(sc.lda, sc.ldb);
+        }
+        transposeForColMajorC(blocked, la, lb);
+        return la == ROCWMMA_AMD_ROW_MAJOR && lb == ROCWMMA_AMD_COL_MAJOR && args.k % 128u == 0u
+               && static_cast<uint64_t>(blocked.lda) * 128u < 0x7FFF0000ull && static_cast<uint64_t>(blocked.ldb) * 128u < 0x7FFF0000ull;
+    }
+
+    bool mxWorkspaceFits(const void* workspace, size_t bytes, uint32_t m, uint32_t n, uint32_t k)
+    {
+        return workspace && bytes >= mxPackedScaleBytes(m, n, k) && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0u;
+    }
+} // namespace
+
 size_t rocwmma_amd_gemm_mx_workspace_size(uint32_t m, uint32_t n, uint32_t k)
 {
     return mxPackedScaleBytes(m, n, k);
@@ -386,19 +412,11 @@ int rocwmma_amd_gemm_mx(int         dtype_in,
         if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE && rc != ROCWMMA_AMD_UNSUPPORTED_TYPE)
             return rc;
     }
-    if(workspace && workspace_bytes >= mxPackedScaleBytes(m, n, k) && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0u)
+    if(mxWorkspaceFits(workspace, workspace_bytes, m, n, k))
     {
-        GemmArgs blocked = args;
-        MxScales sc      = scales;
-        int      la = layout_a, lb = layout_b;
-        if(blocked.layoutC == ROCWMMA_AMD_COL_MAJOR)
-        {
-            std::swap(sc.a, sc.b);
-            std::swap(sc.lda, sc.ldb);
-        }
-        transposeForColMajorC(blocked, la, lb);
-        if(la == ROCWMMA_AMD_ROW_MAJOR && lb == ROCWMMA_AMD_COL_MAJOR && k % 128u == 0u
-           && static_cast<uint64_t>(lda) * 128u < 0x7FFF0000ull && static_cast<uint64_t>(ldb) * 128u < 0x7FFF0000ull)
+        GemmArgs blocked;
+        MxScales sc;
+        if(mxBlockedProblem(layout_a, layout_b, args, scales, blocked, sc))
         {
             char* packedA = static_cast<char*>(workspace);
             char* packedB = packedA + mxPackedScaleOffsetB(blocked.m, k);
@@ -412,6 +430,86 @@ int rocwmma_amd_gemm_mx(int         dtype_in,
         }
     }
     return launchGemmMxWaveTile(dtype_in, layout_a, layout_b, args, scales, asStream(stream));
+}
+
+int rocwmma_amd_gemm_mx_pack_scales(int         layout_a,
+                                    int         layout_b,
+                                    int         layout_c,
+                                    uint32_t    m,
+                                    uint32_t    n,
+                                    uint32_t    k,
+                                    const void* scale_a,
+                                    uint32_t    ld_scale_a,
+                                    const void* scale_b,
+                                    uint32_t    ld_scale_b,
+                                    void*       workspace,
+                                    size_t      workspace_bytes,
+                                    void*       stream)
+{
+    if(!validLayout(layout_a) || !validLayout(layout_b) || !validLayout(layout_c) || m == 0u || n == 0u || k == 0u
+       || (!scale_a && !scale_b))
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(m % 16u != 0u || n % 16u != 0u || k % 128u != 0u)
+        return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+    if((scale_a && ld_scale_a < k / 32u) || (scale_b && ld_scale_b < k / 32u))
+        return ROCWMMA_AMD_BAD_LEADING_DIM;
+    if(!mxWorkspaceFits(workspace, workspace_bytes, m, n, k))
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    // (only the shape, the layouts and the scales matter here: dense leading dimensions stand in for the operands')
+    GemmArgs args{m, n, k, nullptr, nullptr, nullptr, nullptr, layout_a == ROCWMMA_AMD_ROW_MAJOR ? k : m,
+                  layout_b == ROCWMMA_AMD_ROW_MAJOR ? n : k, 0u, 0u, 1.0f, 0.0f, layout_c};
+    MxScales scales{static_cast<const uint8_t*>(scale_a), static_cast<const uint8_t*>(scale_b), ld_scale_a, ld_scale_b};
+    GemmArgs blocked;
+    MxScales sc;
+    if(!mxBlockedProblem(layout_a, layout_b, args, scales, blocked, sc))
+        return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+    char* packedA = static_cast<char*>(workspace);
+    char* packedB = packedA + mxPackedScaleOffsetB(blocked.m, k);
+    return launchMxPackScales(sc, blocked.m, blocked.n, k, packedA, packedB, !gemmMxBlockedUsesLargeTile(blocked), asStream(stream));
+}
+
+int rocwmma_amd_gemm_mx_packed(int         dtype_in,
+                               int         layout_a,
+                               int         layout_b,
+                               int         layout_c,
+                               uint32_t    m,
+                               uint32_t    n,
+                               uint32_t    k,
+                               const void* a,
+                               uint32_t    lda,
+                               const void* b,
+                               uint32_t    ldb,
+                               const void* c,
+                               uint32_t    ldc,
+                               void*       d,
+                               uint32_t    ldd,
+                               float       alpha,
+                               float       beta,
+                               const void* workspace,
+                               size_t      workspace_bytes,
+                               void*       stream)
+{
+    if(dtype_in != ROCWMMA_AMD_E4M3 && dtype_in != ROCWMMA_AMD_E5M2)
+        return ROCWMMA_AMD_UNSUPPORTED_TYPE;
+    int rc = checkGemm(dtype_in, ROCWMMA_AMD_F32, layout_a, layout_b, layout_c, m, n, k, a, lda, b, ldb, c, ldc, d, ldd, alpha, beta);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(m % 16u != 0u || n % 16u != 0u || k % 128u != 0u)
+        return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+    if(!mxWorkspaceFits(workspace, workspace_bytes, m, n, k))
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    GemmArgs args{m, n, k, a, b, c, d, lda, ldb, c ? ldc : ldd, ldd, alpha, beta, layout_c};
+    GemmArgs blocked;
+    MxScales sc, none{};
+    if(!mxBlockedProblem(layout_a, layout_b, args, none, blocked, sc))
+        return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+    const char* packedA = static_cast<const char*>(workspace);
+    const char* packedB = packedA + mxPackedScaleOffsetB(blocked.m, k);
+    return launchGemmMxBlocked(dtype_in, blocked, packedA, packedB, asStream(stream));
 }
 
 int rocwmma_amd_gemm(int         dtype_in,

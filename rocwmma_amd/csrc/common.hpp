@@ -87,7 +87,7 @@ namespace rocwmma_amd
     ROCWMMA_DEVICE ROCWMMA_INLINE float applyActivation(float v, int activation)
     {
         if(activation == ROCWMMA_AMD_ACT_RELU)
-            return v > 0.0f ? v : 0.0f;
+            return v < 0.0f ? 0.0f : v; // (a NaN stays a NaN, as with a maximum that propagates NaNs)
         if(activation == ROCWMMA_AMD_ACT_GELU)
         {
             // x * Phi(x) with Phi(x) = erfc(-x / sqrt 2) / 2 and, for z >= 0, erfc(z) = (a1 t + ... + a5 t^5)

@@ -212,9 +212,13 @@ namespace rocwmma_amd
     int launchMxPackScales(MxScales const& s, uint32_t m, uint32_t n, uint32_t k, void* packedA, void* packedB, bool wide32,
                            hipStream_t stream)
     {
+        // (an operand without scales is left as it is in the workspace: a caller with fixed weights packs
+        // those once and the tokens' scales per call)
         const uint32_t pairs   = (k + 255u) / 256u;
-        const uint32_t groupsA = (m + 63u) / 64u;
-        const uint32_t groupsB = (n + 63u) / 64u;
+        const uint32_t groupsA = s.a ? (m + 63u) / 64u : 0u;
+        const uint32_t groupsB = s.b ? (n + 63u) / 64u : 0u;
+        if(groupsA + groupsB == 0u)
+            return ROCWMMA_AMD_OK;
         const dim3     grid(groupsA + groupsB);
         if(wide32)
             hipLaunchKernelGGL(mxPackScalesKernel<true>, grid, dim3(256), 0, stream, s, m, n, k / 32u, pairs, groupsA,

@@ -92,3 +92,29 @@ def test_no_bias_and_no_activation_is_the_plain_gemm_bit_for_bit():
     want = orc.gemm(orc.F16, orc.F32, RM, CM, RM, RM, m, n, k, a, b, c, 1.5, -0.5)
     check(orc.F32, got, want, 1e-3)
     assert np.array_equal(got.view(np.uint32), to_host(d, np.float32).view(np.uint32))
+
+
+@pytest.mark.parametrize("act", [rw.ACT_RELU, rw.ACT_GELU])
+@pytest.mark.parametrize("m,n,k", [(208, 304, 256), (64, 96, 48)])
+def test_activations_at_non_finite_and_large_arguments(act, m, n, k):
+    """What the activations do at +-Inf, NaN and large |x| (fed in through C with beta = 1), on the blocked kernel
+    and on the wave-tile kernel: ReLU(-Inf) = 0, ReLU(+Inf) = +Inf, ReLU(NaN) = NaN; GELU(+Inf) = +Inf,
+    GELU(NaN) = NaN, GELU(-Inf) = NaN (x * Phi(x) = -Inf * 0, in the oracle's float64 formula as well),
+    GELU(x) = x for large x and -0 for large negative x."""
+    a, b, c, bias = case(500, orc.F16, orc.F32, m, n, k)
+    c = c.copy()
+    special = np.array([np.inf, -np.inf, np.nan, 1e30, -1e30, 40.0, -40.0, 6.0, -6.0], dtype=np.float32)
+    c[: special.size * 7 : 7] = special
+    got = run(orc.F16, orc.F32, RM, CM, RM, m, n, k, a, b, c, 1.0, 1.0, bias, act)
+    want = orc.gemm_bias_act(orc.F16, orc.F32, RM, CM, RM, m, n, k, a, b, c, 1.0, 1.0, bias, act)
+    assert np.array_equal(np.isnan(got), np.isnan(want)), (got[: special.size * 7 : 7], want[: special.size * 7 : 7])
+    assert np.array_equal(np.isinf(got), np.isinf(want))
+    ok = np.isfinite(want)
+    assert np.array_equal(np.sign(got[np.isinf(want)]), np.sign(want[np.isinf(want)]))
+    err, inf, nan = orc.compare_equal(orc.F32, got[ok], orc.F32, want[ok])
+    assert not inf and not nan and err <= 1e-3, (err, inf, nan)
+    sp = got[: special.size * 7 : 7]
+    if act == rw.ACT_RELU:
+        assert sp[0] == np.inf and sp[1] == 0.0 and np.isnan(sp[2]) and sp[4] == 0.0
+    else:
+        assert sp[0] == np.inf and np.isnan(sp[1]) and np.isnan(sp[2]) and sp[3] > 9e29 and abs(sp[4]) == 0.0 and abs(sp[6]) == 0.0

@@ -205,3 +205,97 @@ def test_full_size_quantised_inference_shape_sampled_rows():
     ref = af @ bsum
     size = np.abs(af) @ np.abs(orc.mx_dequantise(dtype, b, sb, RM, n, k).astype(np.float64)).sum(axis=0)
     assert np.max(np.abs(got.astype(np.float64).sum(axis=1) - ref) / size) < 1e-5
+
+
+@pytest.mark.parametrize("m,n,k", [(4096, 2048, 512), (128, 1040, 640), (512, 768, 256)])
+def test_scales_packed_once_and_reused(m, n, k):
+    """rocwmma_amd_gemm_mx_pack_scales + rocwmma_amd_gemm_mx_packed against rocwmma_amd_gemm_mx with a workspace
+    (which packs on every call), bit for bit, on the 256 x 256 tiles and on the mid-size tiles; then new token
+    scales packed into the same workspace without touching the weights' part."""
+    import torch
+
+    rng = np.random.default_rng(77)
+    a, b = exact_int_bits(orc.E4M3, m, k, RM), exact_int_bits(orc.E4M3, k, n, CM)
+    sa, sb = scales(71, m, k, 125, 129), scales(72, n, k, 125, 129)
+    want = run_mx(orc.E4M3, RM, CM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0, True)
+    ws = torch.randint(0, 255, (rw.gemm_mx_workspace_size(m, n, k),), dtype=torch.uint8, device="cuda")
+    rw.gemm_mx_pack_scales(RM, CM, RM, m, n, k, to_device(sa), to_device(sb), ws)
+    da, db = to_device(a), to_device(b)
+    for _ in range(2):  # the GEMM leaves the workspace as it is
+        d = to_device(np.full(m * n, np.nan, dtype=np.float32))
+        rw.gemm_mx_packed(orc.E4M3, RM, CM, RM, m, n, k, da, db, None, d, 1.0, 0.0, ws)
+        assert np.array_equal(to_host(d, np.float32).view(np.uint32), want.view(np.uint32))
+    # new tokens' scales only: the weights' packed scales stay
+    sa2 = scales(73, m, k, 125, 129)
+    rw.gemm_mx_pack_scales(RM, CM, RM, m, n, k, to_device(sa2), None, ws)
+    d = to_device(np.full(m * n, np.nan, dtype=np.float32))
+    rw.gemm_mx_packed(orc.E4M3, RM, CM, RM, m, n, k, da, db, None, d, 1.0, 0.0, ws)
+    want2 = run_mx(orc.E4M3, RM, CM, RM, m, n, k, a, sa2, b, sb, None, 1.0, 0.0, True)
+    assert np.array_equal(to_host(d, np.float32).view(np.uint32), want2.view(np.uint32))
+    want_cpu = orc.gemm_mx(orc.E4M3, RM, CM, RM, RM, m, n, k, a, sa2, b, sb, None, 1.0, 0.0, rows=np.arange(0, m, 61, dtype=np.uint32))
+    rows = np.arange(0, m, 61)
+    assert np.array_equal(want2.reshape(m, n)[rows], want_cpu.reshape(m, n)[rows])
+
+
+def test_packed_entry_points_reject_what_the_blocked_kernels_do_not_take():
+    import torch
+
+    m, n, k = 128, 256, 256
+    ws = torch.empty(rw.gemm_mx_workspace_size(m, n, k), dtype=torch.uint8, device="cuda")
+    sa, sb = to_device(scales(1, m, k, 127, 127)), to_device(scales(2, n, k, 127, 127))
+    with pytest.raises(rw.RocwmmaError) as e:  # both operands row-major: one block per wave only
+        rw.gemm_mx_pack_scales(RM, RM, RM, m, n, k, sa, sb, ws)
+    assert e.value.status == 3
+    with pytest.raises(rw.RocwmmaError) as e:  # nothing to pack
+        rw.gemm_mx_pack_scales(RM, CM, RM, m, n, k, None, None, ws)
+    assert e.value.status == 1
+    with pytest.raises(rw.RocwmmaError) as e:  # workspace too small
+        rw.gemm_mx_pack_scales(RM, CM, RM, m, n, k, sa, sb, ws[:256])
+    assert e.value.status == 1
+    a = to_device(exact_int_bits(orc.E4M3, m, k, RM))
+    b = to_device(exact_int_bits(orc.E4M3, k, n, CM))
+    d = torch.empty(m * n, device="cuda")
+    with pytest.raises(rw.RocwmmaError) as e:  # k not in whole 128-byte stages
+        rw.gemm_mx_packed(orc.E4M3, RM, CM, RM, m, n, 192, a, b, None, d, 1.0, 0.0, ws)
+    assert e.value.status == 3
+
+
+@pytest.mark.parametrize("workspace", [False, True])
+@pytest.mark.parametrize("m,n,k", [(64, 96, 256), (256, 256, 256)])
+def test_end_points_of_the_scale_range_in_live_positions(m, n, k, workspace):
+    """E8M0 bytes 0 (2^-127) and 254 (2^127) on blocks that hold non-zero elements: A's blocks of every third row at
+    2^-127 (and of the rows behind them at 2^-126) against B's at 2^127 in the first K block, unit scales elsewhere.
+    Elements 0, -1, -2 in A and 0, -1 in B, so every product and every partial sum is exact and must match bit for
+    bit; a kernel that flushed the small scale or saturated the large one before multiplying would not."""
+    a = exact_int_bits(orc.E4M3, m, k, RM)
+    bmat = -((np.arange(k)[:, None] + np.arange(n)[None, :]) % 2).astype(np.float32)  # k x n, values 0 / -1
+    b = orc.encode(orc.E4M3, np.ascontiguousarray(bmat.T).reshape(-1))  # col-major
+    sa = np.full((m, k // 32), 127, dtype=np.uint8)
+    sb = np.full((n, k // 32), 127, dtype=np.uint8)
+    sa[::3, 0] = 0
+    sb[:, 0] = 254
+    sa[1::3, 0] = 1  # 2^-126 against 2^127: the block's products are doubled
+    sa[2::3, 0] = 2  # and here times four (a unit scale against 2^127 would overflow)
+    got = run_mx(orc.E4M3, RM, CM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0, workspace)
+    # (the oracle dequantises each operand on its own; every element times its scale is representable here)
+    want = orc.gemm_mx(orc.E4M3, RM, CM, RM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0)
+    assert np.isfinite(want).all() and np.abs(want).max() < 2.0 ** 24
+    # rows whose first block is scaled by 2^-127 * 2^127 = 1 equal the product with unit scales everywhere
+    unit = orc.gemm_mx(orc.E4M3, RM, CM, RM, RM, m, n, k, a, np.full_like(sa, 127), b, np.full_like(sb, 127), None, 1.0, 0.0)
+    assert np.array_equal(want.reshape(m, n)[::3], unit.reshape(m, n)[::3])
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("workspace", [False, True])
+def test_nan_scale_poisons_its_row_only(workspace):
+    """Scale byte 255 is NaN: every output that block contributes to is NaN, every other output is untouched."""
+    m, n, k = 64, 96, 256
+    a, b = exact_int_bits(orc.E4M3, m, k, RM), exact_int_bits(orc.E4M3, k, n, CM)
+    sa, sb = scales(31, m, k, 126, 128), scales(32, n, k, 126, 128)
+    sa[5, 1] = 255
+    sb[17, 0] = 255
+    got = run_mx(orc.E4M3, RM, CM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0, workspace).reshape(m, n)
+    want = orc.gemm_mx(orc.E4M3, RM, CM, RM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0).reshape(m, n)
+    assert np.isnan(want[5]).all() and np.isnan(want[:, 17]).all() and np.isnan(want).sum() == n + m - 1
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(got[~np.isnan(want)], want[~np.isnan(want)])
