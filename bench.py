@@ -666,6 +666,31 @@ def run_extras(rw, torch, dev, gen, only=None):
                                    "note": "E4M3 operands, E8M0 scales per 32 elements of K, scale re-ordering included"}
         del Am, Bm, SAm, SBm, Dm, ws
 
+    # ... its 128-token shape (mid-size scaled tiles): scales re-ordered on every call against scales packed once
+    if wanted("gemm_mxfp8_m128"):
+        m = 128
+        Am = (torch.randn(m * k, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+        Bm = (torch.randn(k * n, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+        SAm = torch.randint(124, 131, (m * (k // 32),), device=dev, dtype=torch.uint8, generator=gen)
+        SBm = torch.randint(124, 131, (n * (k // 32),), device=dev, dtype=torch.uint8, generator=gen)
+        Dm = torch.empty(m * n, device=dev, dtype=torch.float32)
+        ws = torch.empty(rw.gemm_mx_workspace_size(m, n, k), device=dev, dtype=torch.uint8)
+
+        def fn_each():
+            rw.gemm_mx(rw.E4M3, RM, CM, RM, m, n, k, Am, SAm, Bm, SBm, None, Dm, 1.0, 0.0, workspace=ws)
+
+        def fn_packed():
+            rw.gemm_mx_packed(rw.E4M3, RM, CM, RM, m, n, k, Am, Bm, None, Dm, 1.0, 0.0, ws)
+
+        fn_each()
+        ms_each = event_ms(fn_each, iters, torch)
+        rw.gemm_mx_pack_scales(RM, CM, RM, m, n, k, SAm, SBm, ws)
+        fn_packed()
+        ms_packed = event_ms(fn_packed, iters, torch)
+        out["gemm_mxfp8_m128"] = {"ms": round(ms_each, 4), "ms_scales_packed_once": round(ms_packed, 4),
+                                  "note": "E4M3 operands, E8M0 scales per 32 elements of K; weights cache resident"}
+        del Am, Bm, SAm, SBm, Dm, ws
+
     # ... and its 16-token shape (weight streaming): weights and their scales rotated over 5 buffers
     if wanted("gemm_mxfp8_m16"):
         m = 16

@@ -249,6 +249,16 @@ namespace rocwmma_amd
             // at most one 128 x 128 tile per two compute units (few token rows against a wide weight matrix):
             // 128 x 64 tiles put twice as many workgroups to work
             using Narrow = BlockedConfig<InT, float32_t, float32_t, true, true, 2, 2, 2, 1, 2, 3, 32, true, true>;
+            // One round of 128 x 64 tiles with at least 4 KiB of K per row: the tile on the ring of four 128-byte
+            // stages (whole-line requests, three stages in flight), as for the unscaled types (NarrowLinesEdge
+            // above): 128 x 14336 x 4096 31 -> 21 us on scales packed beforehand.
+            using NarrowLines = BlockedConfig<InT, float32_t, float32_t, true, true, 2, 2, 2, 1, 4, 1, 32, true, true, false, 128>;
+            if(gemmBlockedTakesPartlyFilledLineTiles(g.m, g.n, g.k, 1u))
+            {
+                const int rc = launchCfg<NarrowLines>(g, stream, ex);
+                if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+                    return rc;
+            }
             if(2u * ceilDiv(g.m, 128u) * ceilDiv(g.n, 128u) <= computeUnits())
                 return launchCfg<Narrow>(g, stream, ex);
             return launchCfg<Mid>(g, stream, ex);

@@ -148,8 +148,11 @@ namespace rocwmma_amd
                                             && 2u * Block * GroupBlocks * Block * sizeof(OutT) * Waves <= LdsBytes;
 
             static_assert(Block == 32u || Block == 16u, "MFMA blocks are 32 or 16 wide");
-            static_assert(!Scaled || (KPackBytes == 32u && AKMajor && BKMajor && Stages_ == 2u && (Block == 32u || !Edges_)),
-                          "block scales: fp8 on K-contiguous operands in the ring of two (16x16x128 on whole tiles, or 32x32x64)");
+            static_assert(!Scaled
+                              || (KPackBytes == 32u && AKMajor && BKMajor && (Block == 32u || !Edges_)
+                                  && (Stages_ == 2u || (Stages_ == 4u && StageKB == 128u && Block == 32u))),
+                          "block scales: fp8 on K-contiguous operands in the ring of two (16x16x128 on whole tiles, or 32x32x64), "
+                          "or 32x32x64 in the ring of four 128-byte stages");
             static_assert(Block == 32u || KPackBytes == 16u || ((PairReads || Scaled) && AKMajor && BKMajor && Stages_ == 2u),
                           "16-wide blocks: 16 bytes of K per lane (16-bit types, int8), or fp8 16x16x128 on K-contiguous "
                           "operands in the ring of two");
@@ -884,6 +887,104 @@ namespace rocwmma_amd
                     scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
                     scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::Copies>();
                     __builtin_amdgcn_sched_barrier(0);
+                }
+                lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
+                lds::barrier();
+            }
+            else if constexpr(Cfg::KSteps == 2u && Cfg::Scaled)
+            {
+                // Ring of four stages of 128 bytes of K with block scales (32-wide blocks, two instruction steps per
+                // stage): the loop below with the scale loads joining its count of vector-memory operations in
+                // flight.  Two stages per trip, so that a trip is one pair of stages of the packed scales (one dword
+                // per block and lane, byte = step of the pair) and everything that depends on a stage's parity is a
+                // constant: the next pair's scales are requested at the head of a trip, two stages before they take
+                // over.  Every trip issues its stages (past the end of K the last stage again, into a slot nobody
+                // reads), so the body and its counts are uniform.
+                static_assert(S == 4u && Cfg::StageKB == 128u && Cfg::Block == 32u && Part == TilePart::Whole, "scaled ring of four: 128-byte stages of 32-wide blocks");
+                uint32_t        sA[Cfg::BlocksM] = {}, sB[Cfg::BlocksN] = {}, sAnext[Cfg::BlocksM] = {}, sBnext[Cfg::BlocksN] = {};
+                // (dword of block b of an operand, pair p, lane l: (((b / 2) * pairs + p) * 64 + l) * 2 + b % 2)
+                const uint32_t* mxA = static_cast<const uint32_t*>(mx.a)
+                                      + (static_cast<size_t>((row0 + waveM * Cfg::WaveM) / 64u) * mx.pairs * 64u + lane) * 2u
+                                      + ((row0 + waveM * Cfg::WaveM) / 32u) % 2u;
+                const uint32_t* mxB = static_cast<const uint32_t*>(mx.b)
+                                      + (static_cast<size_t>((col0 + waveN * Cfg::WaveN) / 64u) * mx.pairs * 64u + lane) * 2u
+                                      + ((col0 + waveN * Cfg::WaveN) / 32u) % 2u;
+                static_assert(Cfg::BlocksM == 1u || Cfg::BlocksM % 2u == 0u, "a wave's row blocks: one, or whole groups of two");
+                static_assert(Cfg::BlocksN == 1u || Cfg::BlocksN % 2u == 0u, "a wave's column blocks: one, or whole groups of two");
+                auto loadScales32 = [&](uint32_t(&a_)[Cfg::BlocksM], uint32_t(&b_)[Cfg::BlocksN], uint32_t pair) {
+#pragma unroll
+                    for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+                        a_[bi] = mxA[(static_cast<size_t>(bi / 2u) * mx.pairs + pair) * 128u + bi % 2u];
+#pragma unroll
+                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                        b_[bj] = mxB[(static_cast<size_t>(bj / 2u) * mx.pairs + pair) * 128u + bj % 2u];
+                };
+                auto multiplyScaled = [&](Frags const& fr, auto stepC) {
+#if ROCWMMA_ARCH_GFX950 // (the instruction table exists in the device pass only)
+                    using Op  = detail::MfmaScaled<detail::TypeInfo<InT>::cls, detail::TypeInfo<InT>::cls, 32u>;
+                    using Acc = typename Op::Acc;
+                    constexpr uint32_t shift = 8u * decltype(stepC)::value; // the step's byte within the pair of stages
+#pragma unroll
+                    for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+#pragma unroll
+                        for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                        {
+                            Acc& v = *reinterpret_cast<Acc*>(acc[bi][bj].x);
+                            // (the accumulator is kept transposed: the instruction's first multiplicand is B)
+                            v = Op::template exec<0, 0>(fr.b[bj].x, fr.a[bi].x, v, sB[bj] >> shift, sA[bi] >> shift);
+                        }
+#else
+                    (void)fr, (void)stepC;
+#endif
+                };
+                // (in front of the first copies and kept there: the wait for stage 0 covers them)
+                loadScales32(sA, sB, 0u);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for(uint32_t st = 0; st < S - 1u; ++st)
+                    issueStage(st, st + 1u < stages);
+                lds::waitCopiesAndReads<(S - 2u) * Cfg::Copies>();
+                lds::barrier();
+                Frags f0, f1;
+                readFrags(f0, 0u, 0u);
+                auto stage = [&](uint32_t i, auto parityC) {
+                    constexpr uint32_t parity = decltype(parityC)::value;
+                    const uint32_t     slot   = (i + S - 1u) % S;
+                    const bool         adv    = i + S < stages;
+                    issueA(slot, adv);
+                    readFrags(f1, i % S, 1u);
+                    multiplyScaled(f0, std::integral_constant<uint32_t, parity * 2u>{});
+                    scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
+                    scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::CopiesA>();
+                    __builtin_amdgcn_sched_barrier(0);
+                    // Stage i+1 has landed once only stage i+2 and the A half of stage i+3 are in flight.  The scale
+                    // loads of a trip's head sit between those two in issue order, but loads into registers do not
+                    // complete in order with copies into LDS (counting them as in flight let a wait pass with a copy of
+                    // stage i+1 outstanding whenever they had returned first: wrong results on a cold cache), so they
+                    // are not counted: with them outstanding the wait holds a little longer, never too short.
+                    lds::waitCopiesAndReads<(S - 3u) * Cfg::Copies + Cfg::CopiesA>();
+                    lds::barrier();
+                    __builtin_amdgcn_sched_barrier(0);
+                    issueB(slot, adv);
+                    readFrags(f0, (i + 1u) % S, 0u);
+                    multiplyScaled(f1, std::integral_constant<uint32_t, parity * 2u + 1u>{});
+                    scheduleInterleaved<Cfg::MfmasPerStep / 2u, Cfg::ReadsPerStep, 0u>();
+                    scheduleInterleaved<Cfg::MfmasPerStep - Cfg::MfmasPerStep / 2u, 0u, Cfg::CopiesB>();
+                    __builtin_amdgcn_sched_barrier(0);
+                };
+                for(uint32_t i = 0; i < stages; i += 2u)
+                {
+                    loadScales32(sAnext, sBnext, i / 2u + 1u < mx.pairs ? i / 2u + 1u : mx.pairs - 1u);
+                    __builtin_amdgcn_sched_barrier(0);
+                    stage(i, std::integral_constant<uint32_t, 0u>{});
+                    if(i + 1u < stages)
+                        stage(i + 1u, std::integral_constant<uint32_t, 1u>{});
+#pragma unroll
+                    for(uint32_t bi = 0; bi < Cfg::BlocksM; ++bi)
+                        sA[bi] = sAnext[bi];
+#pragma unroll
+                    for(uint32_t bj = 0; bj < Cfg::BlocksN; ++bj)
+                        sB[bj] = sBnext[bj];
                 }
                 lds::waitCopiesAndReads<0u>(); // the surplus copies still target this workgroup's LDS
                 lds::barrier();

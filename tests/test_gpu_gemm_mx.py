@@ -299,3 +299,24 @@ def test_nan_scale_poisons_its_row_only(workspace):
     assert np.isnan(want[5]).all() and np.isnan(want[:, 17]).all() and np.isnan(want).sum() == n + m - 1
     assert np.array_equal(np.isnan(got), np.isnan(want))
     assert np.array_equal(got[~np.isnan(want)], want[~np.isnan(want)])
+
+
+@pytest.mark.parametrize("dtype", [orc.E4M3, orc.E5M2])
+@pytest.mark.parametrize("m,n,k", [(128, 4160, 4096), (48, 8192, 4224), (112, 14336, 4096)])
+def test_one_round_of_narrow_tiles_on_the_ring_of_four_line_stages(dtype, m, n, k):
+    """One round of 128 x 64 tiles with at least 4 KiB of K per row (on a 256-unit device): the scaled tile on the
+    ring of four 128-byte stages, whose scale loads join the count of operations in flight.  An even and an odd
+    number of stages, a partly filled row of tiles, every scale different: exact pattern bit for bit, random
+    operands within the fp8 tolerance against sampled oracle rows."""
+    a = exact_int_bits(dtype, m, k, RM)
+    b = exact_int_bits(dtype, k, n, CM)
+    sa, sb = scales(101, m, k, 125, 129), scales(102, n, k, 125, 129)
+    rows = np.arange(0, m, 5, dtype=np.uint32)
+    got = run_mx(dtype, RM, CM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0, True)
+    want = orc.gemm_mx(dtype, RM, CM, RM, RM, m, n, k, a, sa, b, sb, None, 1.0, 0.0, rows=rows)
+    check(np.ascontiguousarray(got.reshape(m, n)[rows]).ravel(), np.ascontiguousarray(want.reshape(m, n)[rows]).ravel(), 0.0)
+    a, b = uniform_bits(103, dtype, m * k), uniform_bits(104, dtype, k * n)
+    c = uniform_bits(105, orc.F32, m * n)
+    got = run_mx(dtype, RM, CM, RM, m, n, k, a, sa, b, sb, c, 0.5, 2.0, True)
+    want = orc.gemm_mx(dtype, RM, CM, RM, RM, m, n, k, a, sa, b, sb, c, 0.5, 2.0, rows=rows)
+    check(np.ascontiguousarray(got.reshape(m, n)[rows]).ravel(), np.ascontiguousarray(want.reshape(m, n)[rows]).ravel(), 1e-2)
