@@ -444,7 +444,9 @@ int rocwmma_amd_gemv(uint32_t    m,
  *   output : batch x (k + m(m-1)/2):  [ input[b,0,:] , Z[1,0], Z[2,0], Z[2,1], Z[3,0], ... ]
  *            with Z = input[b] * input[b]^T.
  * Unlike the reference kernel this one needs no f32 m x m scratch (`acc`) and accepts any
- * m <= 32 (the reference GPU kernels need m % 16 == 0, test/dlrm/dlrm_kernel_base_impl.hpp:146-150).
+ * m <= 128 (the reference GPU kernels need m % 16 == 0, test/dlrm/dlrm_kernel_base_impl.hpp:146-150;
+ * its tests run m = 32 and 128 among others, test/dlrm/test/dlrm_test_params.hpp:51-58).  Up to 32 rows are
+ * one matrix-instruction operand per sample (the benchmark configuration, m = 27); more run as tiles of 32.
  * k must be 32, 64, 128 or 256; input and output must be 16-byte aligned.
  */
 int rocwmma_amd_dlrm_fwd(const void* input,

@@ -568,7 +568,7 @@ static int checkDlrm(uint32_t m, uint32_t k, uint32_t batch)
 {
     if(m == 0u || batch == 0u)
         return ROCWMMA_AMD_INVALID_ARGUMENT;
-    if(m > 32u || (k != 32u && k != 64u && k != 128u && k != 256u))
+    if(m > 128u || (k != 32u && k != 64u && k != 128u && k != 256u))
         return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
     return ROCWMMA_AMD_OK;
 }

@@ -402,6 +402,282 @@ namespace rocwmma_amd
             }
         }
 
+        // ------------------------------------------------------------------ more than 32 feature rows
+        // 32 < m <= 128 (the reference's DLRM tests also run m = 128, test/dlrm/test/dlrm_test_params.hpp:51-58): the
+        // same wave-per-sample structure with the sample's rows cut into tiles of 32.  Forward: Z block (I, J), J <= I,
+        // is F_I F_J^T, one 32 x 32 accumulator at a time.  Backward: row tile I of the gradient is the sum over
+        // contraction tiles J of G_IJ F_J, with the G fragments of a row tile rebuilt once from the packed triangle
+        // and the result staged per wave.  One or two samples per workgroup, whatever fits the LDS.  These shapes
+        // are not a benchmark configuration; the kernels are written for parity, with the data paths of the ones above.
+        constexpr uint32_t kMaxTiledM = 128;
+
+        template <uint32_t K, uint32_t Samples>
+        __global__ void __launch_bounds__(64 * Samples)
+            dlrmFwdTiledKernel(const float16_t* __restrict__ input, float16_t* __restrict__ output, uint32_t m, uint32_t batch)
+        {
+            constexpr uint32_t KSteps = K / 16u;
+            using Tile                = FeatureTile<K>;
+            using FragA               = fragment<matrix_a, 32, 32, 16, float16_t, row_major>;
+            using FragAcc             = fragment<accumulator, 32, 32, 16, float32_t>;
+            using AccMap              = detail::AccMap<32, 32, 32>;
+
+            extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
+            const uint32_t width     = K + (m * (m - 1u)) / 2u;
+            const uint32_t tiles     = (m + 31u) / 32u;
+            const uint32_t tileBytes = (((Samples - 1u) * m + tiles * 32u) * Tile::rowBytes + 1023u) & ~1023u;
+            char*          ldsIn     = ldsRaw;
+            const uint32_t sample0   = blockIdx.x * Samples;
+            float16_t* const outBlock = output + static_cast<size_t>(sample0) * width;
+            float16_t*       ldsOut   = reinterpret_cast<float16_t*>(ldsRaw + tileBytes + (reinterpret_cast<uintptr_t>(outBlock) & 15u));
+
+            const uint32_t lane  = threadIdx.x & 63u;
+            const uint32_t wave  = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            const uint32_t nHere = min(Samples, batch - sample0);
+
+            Tile::template asyncLoad<false>(ldsIn, input + static_cast<size_t>(sample0) * m * K, nHere * m * Tile::rowBytes,
+                                            wave, Samples, lane);
+            lds::waitCopiesAndReads<0>();
+            __syncthreads();
+
+            if(wave < nHere)
+            {
+                const uint32_t row    = lane & 31u;
+                const uint32_t kGroup = lane >> 5;
+                float16_t*     out    = ldsOut + wave * width;
+                {
+                    const uint32_t   R0   = wave * m;
+                    const float16_t* row0 = reinterpret_cast<const float16_t*>(ldsIn + R0 * Tile::rowBytes);
+                    const uint32_t   swz0 = Tile::chunkSwizzle(R0);
+#pragma unroll
+                    for(uint32_t e = lane; e < K; e += 64u)
+                        out[e] = row0[(((e / 8u) ^ swz0) << 3) + e % 8u];
+                }
+                const uint32_t spare = (Samples - wave) * width + wave; // behind the last sample's row
+                // operand of tile T: matrix row = lane % 32 (rows >= m belong to the next sample or are stale LDS:
+                // they only reach Gram entries with an index >= m, which are dropped)
+                auto loadTile = [&](FragA(&f)[KSteps], uint32_t T) {
+                    const uint32_t R   = wave * m + T * 32u + row;
+                    const uint32_t swz = Tile::chunkSwizzle(R);
+#pragma unroll
+                    for(uint32_t ks = 0; ks < KSteps; ++ks)
+                        *reinterpret_cast<u32x4_t*>(f[ks].x)
+                            = *reinterpret_cast<const u32x4_t*>(ldsIn + R * Tile::rowBytes + (((ks * 2u + kGroup) ^ swz) << 4));
+                };
+#pragma unroll 1
+                for(uint32_t I = 0; I < tiles; ++I)
+                {
+                    FragA fI[KSteps];
+                    loadTile(fI, I);
+                    const uint32_t Rg       = I * 32u + row; // row of Z
+                    const uint32_t rowStart = K + (Rg * (Rg - 1u)) / 2u;
+#pragma unroll 1
+                    for(uint32_t J = 0; J <= I; ++J)
+                    {
+                        FragA fJ[KSteps];
+                        loadTile(fJ, J);
+                        FragAcc acc;
+                        fill_fragment(acc, 0.0f);
+#pragma unroll
+                        for(uint32_t ks = 0; ks < KSteps; ++ks)
+                            mma_sync(acc, fI[ks], applyTranspose(fJ[ks]), acc);
+#pragma unroll
+                        for(uint32_t e = 0; e < FragAcc::num_elements; ++e)
+                        {
+                            const uint32_t Cg = J * 32u + AccMap::colOf(e, lane);
+                            out[(Rg < m && Cg < Rg) ? rowStart + Cg : spare] = static_cast<float16_t>(acc.x[e]);
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+            copyOut(outBlock, ldsOut, nHere * width);
+        }
+
+        template <uint32_t K, uint32_t Samples>
+        __global__ void __launch_bounds__(64 * Samples) dlrmBwdTiledKernel(const float16_t* __restrict__ input,
+                                                                                const float16_t* __restrict__ upstream,
+                                                                                float16_t* __restrict__ grad,
+                                                                                float16_t* __restrict__ mlpGrad,
+                                                                                uint32_t m,
+                                                                                uint32_t batch)
+        {
+            constexpr uint32_t NBlocks  = K / 32u; // 32-column blocks of the m x K result
+            constexpr uint32_t MaxTiles = kMaxTiledM / 32u;
+            using Tile                  = FeatureTile<K>;
+            using Stage                 = GradStage<K>;
+            using FragG                 = fragment<matrix_a, 32, 32, 16, float16_t, row_major>;
+            using FragF                 = fragment<matrix_b, 32, 32, 16, float16_t, row_major>;
+            using FragAcc               = fragment<accumulator, 32, 32, 16, float32_t>;
+            using AccMap                = detail::AccMap<32, 32, 32>;
+
+            extern __shared__ __attribute__((aligned(1024))) char ldsRaw[];
+            const uint32_t width     = K + (m * (m - 1u)) / 2u;
+            const uint32_t tiles     = (m + 31u) / 32u;
+            const uint32_t tileBytes = (((Samples - 1u) * m + tiles * 32u) * Tile::rowBytes + 1023u) & ~1023u;
+            const uint32_t upBytesLds = (Samples * width * 2u + 2u + 255u) & ~255u;
+            char*          ldsF      = ldsRaw;
+            float16_t*     ldsUp     = reinterpret_cast<float16_t*>(ldsRaw + tileBytes);
+            char*          ldsStage  = ldsRaw + tileBytes + upBytesLds; // per wave: 32 rows of the gradient
+
+            const uint32_t lane    = threadIdx.x & 63u;
+            const uint32_t wave    = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            const uint32_t sample0 = blockIdx.x * Samples;
+            const uint32_t nHere   = min(Samples, batch - sample0);
+
+            Tile::template asyncLoad<true>(ldsF, input + static_cast<size_t>(sample0) * m * K, nHere * m * Tile::rowBytes, wave, Samples,
+                                           lane);
+            // upstream gradients: 4-byte direct copies.  With one sample per workgroup and an odd row width a
+            // block can start on an odd half: it is then copied from the half in front of it (the previous
+            // sample's last) and read one half on.
+            const float16_t* upBlock = upstream + static_cast<size_t>(sample0) * width;
+            const uint32_t   upSkew  = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(upBlock) & 2u) / 2u; // 0 or 1 halves
+            {
+                const float16_t*      from    = upBlock - upSkew;
+                const uint32_t        upBytes = (nHere * width + upSkew) * 2u;
+                const uint32_t        whole   = upBytes & ~3u;
+                const lds::BufferRsrc rsrc
+                    = __builtin_amdgcn_make_buffer_rsrc(const_cast<float16_t*>(from), 0, static_cast<int>(whole), 0x00020000);
+                for(uint32_t copy = wave; copy * 256u < whole; copy += Samples)
+                    if(copy * 256u + lane * 4u < whole)
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds::LdsPtr)(reinterpret_cast<char*>(ldsUp) + copy * 256u), 4,
+                                                                 static_cast<int>(copy * 256u + lane * 4u), 0, 0, 2 /* nt */);
+                if(whole != upBytes && threadIdx.x == 0u)
+                    ldsUp[whole / 2u] = from[whole / 2u];
+            }
+            lds::waitCopiesAndReads<0>();
+            __syncthreads();
+            const float16_t* upLds = ldsUp + upSkew;
+
+            for(uint32_t i = threadIdx.x; i < nHere * (K / 8u); i += blockDim.x)
+            {
+                const uint32_t   s   = i / (K / 8u);
+                const uint32_t   c8  = i % (K / 8u);
+                const float16_t* src = upLds + s * width + c8 * 8u;
+                float16_t        tmp[8];
+#pragma unroll
+                for(uint32_t j = 0; j < 8u; ++j)
+                    tmp[j] = src[j];
+                reinterpret_cast<u32x4_t*>(mlpGrad + static_cast<size_t>(sample0 + s) * K)[c8] = *reinterpret_cast<u32x4_t*>(tmp);
+            }
+
+            if(wave < nHere)
+            {
+                const uint32_t   row     = lane & 31u;
+                const uint32_t   kGroup  = lane >> 5;
+                const uint32_t   group   = lane >> 4;
+                const uint32_t   s16     = lane & 15u;
+                const float16_t* up      = upLds + wave * width;
+                const uint32_t   ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds::LdsPtr)ldsF));
+                char*            stage   = ldsStage + wave * (32u * Stage::rowBytes);
+                u32x4_t*         dstSample = reinterpret_cast<u32x4_t*>(grad + static_cast<size_t>(sample0 + wave) * m * K);
+#pragma unroll 1
+                for(uint32_t I = 0; I < tiles; ++I)
+                {
+                    // G operands of row tile I against every contraction tile J: row Rg, columns J*32 + ks*16 +
+                    // kGroup*8 + j, rebuilt from the packed triangle (every lane reads all of its entries, a harmless
+                    // address where there is none, and selects afterwards)
+                    const uint32_t Rg    = I * 32u + row;
+                    const uint32_t below = K + (Rg * (Rg - 1u)) / 2u;
+                    FragG          fg[MaxTiles][2];
+#pragma unroll
+                    for(uint32_t J = 0; J < MaxTiles; ++J)
+#pragma unroll
+                        for(uint32_t ks = 0; ks < 2u; ++ks)
+                        {
+                            const uint32_t c0    = J * 32u + ks * 16u + kGroup * 8u;
+                            uint32_t       above = K + (c0 * (c0 - 1u)) / 2u + Rg; // (c0 = 0: the product wraps to 0)
+#pragma unroll
+                            for(uint32_t j = 0; j < 8u; ++j)
+                            {
+                                const uint32_t  c     = c0 + j;
+                                const bool      there = (c > Rg ? c : Rg) < m && c != Rg;
+                                const float16_t g     = up[there ? (c < Rg ? below + c : above) : 0u];
+                                fg[J][ks].x[j]        = there ? g : static_cast<float16_t>(0);
+                                above += c;
+                            }
+                        }
+#pragma unroll 1
+                    for(uint32_t nb = 0; nb < NBlocks; ++nb)
+                    {
+                        FragAcc acc;
+                        fill_fragment(acc, 0.0f);
+#pragma unroll
+                        for(uint32_t J = 0; J < MaxTiles; ++J)
+                        {
+                            if(J < tiles) // (wave uniform)
+                            {
+                                // F operands: transposing reads, lane l gets column nb*32 + l%32 and contraction rows
+                                // J*32 + ks*16 + (l/32)*8 + 0..7 of this sample
+                                uint32_t ff[2][4];
+#pragma unroll
+                                for(uint32_t ks = 0; ks < 2u; ++ks)
+#pragma unroll
+                                    for(uint32_t kk = 0; kk < 2u; ++kk)
+                                    {
+                                        const uint32_t c    = J * 32u + ks * 16u + (group >> 1) * 8u + kk * 4u + (s16 >> 2);
+                                        const uint32_t R    = wave * m + c;
+                                        const uint32_t seg  = nb * 2u + (group & 1u);
+                                        const uint32_t addr = ldsBase + R * Tile::rowBytes + ((seg ^ Tile::segmentSwizzle(R)) << 5)
+                                                              + ((s16 & 3u) << 3);
+                                        typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+                                        u32x2_t v;
+                                        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+                                        ff[ks][2u * kk]      = v[0];
+                                        ff[ks][2u * kk + 1u] = v[1];
+                                    }
+                                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                                for(uint32_t ks = 0; ks < 2u; ++ks)
+                                {
+                                    FragF f;
+#pragma unroll
+                                    for(uint32_t w = 0; w < 4u; ++w)
+                                    {
+                                        // contraction rows >= m are the next sample's features or stale LDS: cleared, so
+                                        // that 0 * Inf and 0 * NaN cannot leak between samples
+                                        const uint32_t c0   = J * 32u + ks * 16u + kGroup * 8u + 2u * w;
+                                        const uint32_t keep = (c0 < m ? 0x0000FFFFu : 0u) | (c0 + 1u < m ? 0xFFFF0000u : 0u);
+                                        asm volatile("" : "+v"(ff[ks][w]));
+                                        reinterpret_cast<uint32_t*>(f.x)[w] = ff[ks][w] & keep;
+                                    }
+                                    mma_sync(acc, fg[J][ks], f, acc);
+                                }
+                            }
+                        }
+                        // into this wave's staging rows (8-byte units XOR-swizzled by the row)
+#pragma unroll
+                        for(uint32_t r4 = 0; r4 < AccMap::runs; ++r4)
+                        {
+                            const uint32_t e0 = r4 * 4u;
+                            const uint32_t r  = AccMap::rowOf(e0, lane);
+                            const uint32_t c  = nb * 32u + AccMap::colOf(e0, lane);
+                            float16_t      h[4];
+#pragma unroll
+                            for(uint32_t j = 0; j < 4u; ++j)
+                                h[j] = static_cast<float16_t>(acc.x[e0 + j]);
+                            typedef uint32_t u32x2_t __attribute__((ext_vector_type(2), may_alias));
+                            *reinterpret_cast<u32x2_t*>(stage + Stage::unitOffset(r, c / 4u)) = *reinterpret_cast<u32x2_t*>(h);
+                        }
+                    }
+                    // rows I*32 .. of this sample's gradient: one contiguous block of 16-byte pieces
+                    {
+                        constexpr uint32_t chunksPerRow = K / 8u;
+                        const uint32_t     rowsHere     = min(32u, m - I * 32u);
+                        u32x4_t*           dst          = dstSample + static_cast<size_t>(I) * 32u * chunksPerRow;
+                        for(uint32_t q = lane; q < rowsHere * chunksPerRow; q += 64u)
+                        {
+                            const uint32_t R = q / chunksPerRow, ch = q % chunksPerRow;
+                            const uint32_t s = R & Stage::mask;
+                            u32x4_t        v = *reinterpret_cast<const u32x4_t*>(stage + R * Stage::rowBytes + ((ch ^ (s >> 1)) << 4));
+                            if(s & 1u)
+                                v = u32x4_t{v[2], v[3], v[0], v[1]};
+                            dst[q] = v;
+                        }
+                    }
+                }
+            }
+        }
+
         template <uint32_t K, uint32_t Samples>
         uint32_t tileBytesFor(uint32_t m)
         {
@@ -465,9 +741,50 @@ namespace rocwmma_amd
             return batch >= 8u * cus ? 4u : 2u;
         }
 
+        constexpr uint32_t kLdsBytes = 160u * 1024u;
+
+        template <uint32_t K, uint32_t Samples>
+        int launchFwdTiledS(const void* input, void* output, uint32_t m, uint32_t batch, hipStream_t stream)
+        {
+            const uint32_t width = K + (m * (m - 1u)) / 2u, tiles = (m + 31u) / 32u;
+            const uint32_t lds   = ((((Samples - 1u) * m + tiles * 32u) * K * 2u + 1023u) & ~1023u) + ((Samples * width * 2u + 15u) & ~15u) + 32u;
+            if(lds > kLdsBytes)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            auto kernel = dlrmFwdTiledKernel<K, Samples>;
+            if(int rc = optInLds(kernel, lds))
+                return rc;
+            hipLaunchKernelGGL(kernel, dim3((batch + Samples - 1u) / Samples), dim3(64u * Samples), lds, stream,
+                               static_cast<const float16_t*>(input), static_cast<float16_t*>(output), m, batch);
+            return launchStatus();
+        }
+
+        template <uint32_t K, uint32_t Samples>
+        int launchBwdTiledS(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t batch,
+                            hipStream_t stream)
+        {
+            const uint32_t width = K + (m * (m - 1u)) / 2u, tiles = (m + 31u) / 32u;
+            const uint32_t lds   = ((((Samples - 1u) * m + tiles * 32u) * K * 2u + 1023u) & ~1023u) + ((Samples * width * 2u + 2u + 255u) & ~255u)
+                                 + Samples * 32u * K * 2u;
+            if(lds > kLdsBytes)
+                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            auto kernel = dlrmBwdTiledKernel<K, Samples>;
+            if(int rc = optInLds(kernel, lds))
+                return rc;
+            hipLaunchKernelGGL(kernel, dim3((batch + Samples - 1u) / Samples), dim3(64u * Samples), lds, stream,
+                               static_cast<const float16_t*>(input), static_cast<const float16_t*>(upstream),
+                               static_cast<float16_t*>(grad), static_cast<float16_t*>(mlpGrad), m, batch);
+            return launchStatus();
+        }
+
         template <uint32_t K>
         int launchFwd(const void* input, void* output, uint32_t m, uint32_t batch, hipStream_t stream)
         {
+            if(m > kMaxM)
+            {
+                // two samples per workgroup where the LDS holds them, else one
+                const int rc = launchFwdTiledS<K, 2>(input, output, m, batch, stream);
+                return rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE ? rc : launchFwdTiledS<K, 1>(input, output, m, batch, stream);
+            }
             switch(samplesFor(batch, true))
             {
             case 4:
@@ -481,6 +798,11 @@ namespace rocwmma_amd
         int launchBwd(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t batch,
                       hipStream_t stream)
         {
+            if(m > kMaxM)
+            {
+                const int rc = launchBwdTiledS<K, 2>(input, upstream, grad, mlpGrad, m, batch, stream);
+                return rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE ? rc : launchBwdTiledS<K, 1>(input, upstream, grad, mlpGrad, m, batch, stream);
+            }
             switch(samplesFor(batch, false))
             {
             case 8:

@@ -124,3 +124,35 @@ def test_backward_samples_are_independent_of_non_finite_neighbours(b):
     assert np.array_equal(grad[0::2], clean[0::2])
     wgrad, _ = orc.dlrm_bwd(poisoned, up, m, k, b)
     assert np.array_equal(np.isnan(orc.decode(orc.F16, grad.reshape(-1))), np.isnan(orc.decode(orc.F16, wgrad.reshape(-1))))
+
+
+@pytest.mark.parametrize("b,m,k", [(5, 128, 128), (3, 128, 256), (4, 33, 64), (7, 64, 32), (6, 100, 128), (2, 96, 256), (9, 40, 128)])
+def test_more_than_32_feature_rows_run_as_tiles_of_32(b, m, k):
+    """32 < m <= 128 (the reference's DLRM tests run m = 128, test/dlrm/test/dlrm_test_params.hpp:51-58): forward
+    and backward against the oracle; one and two samples per workgroup, odd batch sizes and odd row widths
+    (m = 33: width 592, m = 100 with k = 128: 5078), m that is not a multiple of 32."""
+    inp = uniform_bits(700 + m, orc.F16, b * m * k).reshape(b, m, k)
+    width = k + m * (m - 1) // 2
+    up = uniform_bits(701 + m, orc.F16, b * width).reshape(b, width)
+    got = gpu_fwd(inp, m, k, b)
+    want = orc.dlrm_fwd(inp, m, k, b)
+    close(got, want)
+    assert np.array_equal(got[:, :k], inp[:, 0, :])
+    grad, mlp = gpu_bwd(inp, up, m, k, b)
+    wgrad, wmlp = orc.dlrm_bwd(inp, up, m, k, b)
+    close(grad, wgrad)
+    assert np.array_equal(mlp, wmlp)
+
+
+def test_tiled_backward_samples_are_independent_of_non_finite_neighbours():
+    """As for m <= 32: rows of the next sample that a tile's operand reads beyond m must not leak (0 * Inf)."""
+    b, m, k = 4, 40, 128
+    inp = uniform_bits(801, orc.F16, b * m * k).reshape(b, m, k).copy()
+    width = k + m * (m - 1) // 2
+    up = uniform_bits(802, orc.F16, b * width).reshape(b, width)
+    want, _ = orc.dlrm_bwd(inp, up, m, k, b)
+    poisoned = inp.copy()
+    poisoned[2] = 0x7C00  # +Inf everywhere in sample 2
+    grad, _ = gpu_bwd(poisoned, up, m, k, b)
+    for s in (0, 1, 3):
+        close(grad[s], want[s])
