@@ -128,7 +128,7 @@ def test_gemv_and_dlrm_argument_validation(lib):
     assert f(64, 64, 1, None, 64, 8192, 64, 12288, 64, 1.0, 0.0, None) == 1
     g = lib.rocwmma_amd_dlrm_fwd
     assert g(None, 4096, 27, 128, 8, None) == 1
-    assert g(4096, 8192, 33, 128, 8, None) == 3
+    assert g(4096, 8192, 129, 128, 8, None) == 3
     assert g(4096, 8192, 27, 100, 8, None) == 3
     assert g(4096, 8192, 27, 128, 0, None) == 1
     h = lib.rocwmma_amd_dlrm_bwd
