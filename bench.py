@@ -349,6 +349,14 @@ def main():
         del zeros
         roofline["mfma_only_ceiling"] = ceiling
         roofline["frac_of_mfma_only_ceiling"] = round(per_case[dom]["tflops"] / ceiling[key]["data"], 4)
+        # What the device sustains when the tile's matrix instructions run next to the byte streams a 256 x 256
+        # tile of 16-bit operands needs (192 KiB of LDS reads and 64 KiB of L2 -> LDS copies per 64 of K per compute
+        # unit) and nothing else -- no barrier, no tile bookkeeping, no epilogue: the ceiling of the tiling itself on
+        # this power-managed part, on the benchmark's operands and on all-zero ones.
+        if S == 8192 and dom_dtype == "f16":
+            streams = run_streams_ceiling(rw, torch, dev, gen, dom_case[4], dom_case[5])
+            roofline["mfma_with_operand_streams"] = streams
+            roofline["frac_of_operand_streams_ceiling"] = round(per_case[dom]["tflops"] / streams["data"]["with_lds_reads_and_l2_copies"], 4)
         roofline["zero_operands"] = {
             "ms": round(ms_zero, 4), "tflops": round(flops_per_gemm / ms_zero / 1e9, 1),
             "frac": round(flops_per_gemm / ms_zero / 1e9 / dom_peak, 4),
@@ -408,6 +416,28 @@ def main():
                                f"({len(cases)} GEMMs per step), alpha=beta=1"},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "extra": extra,
     }))
+
+
+def run_streams_ceiling(rw, torch, dev, gen, A, B):
+    """TFLOP/s of the matrix-pipes-next-to-their-operand-streams probe (rocwmma_amd_bench_mfma_streams): matrix
+    instructions only, with the LDS fragment reads, with those and the global -> LDS copies; on the operands of
+    the timed GEMM and on all-zero ones.  Ten launches of four tiles per compute unit after ten warm-up launches."""
+    tables = {"data": (A[: 32768].contiguous().view(torch.uint8), A, B),
+              "zero": (torch.zeros(65536, device=dev, dtype=torch.uint8), torch.zeros_like(A), None)}
+    sink = torch.empty(rw.device_info()["compute_units"] * 512, device=dev)
+    out = {}
+    for label, (table, a_, b_) in tables.items():
+        b_ = a_ if b_ is None else b_
+        res = {}
+        for name, streams in (("mfma_only", 0), ("with_lds_reads", 1), ("with_lds_reads_and_l2_copies", 3)):
+            fn = lambda: rw.bench_mfma_streams(streams, 4, a_, b_, table, sink)
+            ops = fn()
+            for _ in range(9):
+                fn()
+            ms = event_ms(fn, 10, torch)
+            res[name] = round(ops / ms / 1e9, 1)
+        out[label] = res
+    return out
 
 
 def run_ceiling(rw, torch, dev, gen, dtypes=None):

@@ -96,6 +96,27 @@ int rocwmma_amd_bench_mfma_ceiling(int         shape,
                                    void*       stream);
 
 /*
+ * Matrix pipes next to their operand streams: what the device sustains when the matrix instructions of a
+ * 256 x 256 tile of 16-bit operands (v_mfma_f32_16x16x32_f16, eight waves of 64 x 128 per compute unit) run next
+ * to the byte streams such a tile needs per 64 of K, and nothing else: no barrier, no tile bookkeeping, no
+ * epilogue.  streams = 0: matrix instructions only; 1: with the 192 KiB of fragment reads from LDS per stage; 3: with
+ * those and the 64 KiB of global -> LDS copies per stage, walking the A / B panels in the tile order of an
+ * 8192^3 problem.  `a`, `b`: 8192 x 8192 halves each, K contiguous (needed for streams = 3); `operands`: a
+ * 64 KiB table of operand bits as for rocwmma_amd_bench_mfma_ceiling; `out`: 512 floats per compute unit;
+ * tiles_per_workgroup: tiles (of 128 stages) each compute unit walks, at most 1024 / compute units; *ops: the
+ * operations of the launch.  On a power-managed part each stream costs clock: the blocked GEMM is priced against
+ * this figure next to the matrix-pipe ceiling and the nominal peak.  Has no counterpart in the reference.
+ */
+int rocwmma_amd_bench_mfma_streams(int         streams,
+                                   uint32_t    tiles_per_workgroup,
+                                   const void* a,
+                                   const void* b,
+                                   const void* operands,
+                                   float*      out,
+                                   double*     ops,
+                                   void*       stream);
+
+/*
  * Memory-stream ceiling probe: one plain kernel that reads (mode 0), writes (mode 1) or copies (mode 2)
  * `bytes` bytes (a multiple of 64 KiB) with 16-byte accesses (reads: 16 workgroups of 256 threads per compute
  * unit; writes and copies: workgroups of 1024 threads; each tuned by a sweep over accesses per lane, workgroup

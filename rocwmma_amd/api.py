@@ -26,7 +26,7 @@ ACT_NONE, ACT_RELU, ACT_GELU = range(3)
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
 _AUX_LIB_NAME = "librocwmma_amd_aux.so"
 AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_bench_mfma_ceiling",
-               "rocwmma_amd_bench_stream"]
+               "rocwmma_amd_bench_stream", "rocwmma_amd_bench_mfma_streams"]
 (MFMA_F16_16X16X32, MFMA_F16_32X32X16, MFMA_BF16_16X16X32, MFMA_BF16_32X32X16, MFMA_I8_16X16X64, MFMA_I8_32X32X32,
  MFMA_F8_16X16X128, MFMA_F8_32X32X64, MFMA_F8_16X16X128_SCALED) = range(9)
 
@@ -122,6 +122,8 @@ def aux_library():
         L.rocwmma_amd_bench_mfma_ceiling.argtypes = [i, u, u, vp, vp, ctypes.POINTER(ctypes.c_double), vp]
         L.rocwmma_amd_bench_mfma_ceiling.restype = i
         L.rocwmma_amd_bench_stream.argtypes = [i, vp, vp, ctypes.c_size_t, vp]
+        L.rocwmma_amd_bench_mfma_streams.argtypes = [i, u, vp, vp, vp, vp, ctypes.POINTER(ctypes.c_double), vp]
+        L.rocwmma_amd_bench_mfma_streams.restype = i
         L.rocwmma_amd_bench_stream.restype = i
         _aux = L
     return _aux
@@ -350,6 +352,15 @@ def bench_stream(mode, src, dst, nbytes, stream=None):
     device tensors or raw addresses."""
     _check(aux_library().rocwmma_amd_bench_stream(mode, _ptr(src), _ptr(dst), nbytes,
                                                   stream if stream is not None else _stream()), "bench_stream")
+
+
+def bench_mfma_streams(streams, tiles_per_workgroup, a, b, operands, out):
+    """Launches the matrix-pipes-next-to-their-operand-streams probe (include/rocwmma_amd_aux.h); returns the
+    operation count of the launch."""
+    ops = ctypes.c_double(0.0)
+    _check(aux_library().rocwmma_amd_bench_mfma_streams(streams, tiles_per_workgroup, _ptr(a), _ptr(b), _ptr(operands), _ptr(out),
+                                                        ctypes.byref(ops), _stream()), "bench_mfma_streams")
+    return ops.value
 
 
 def bench_mfma_ceiling(shape, trips, waves_per_simd, operands, out):

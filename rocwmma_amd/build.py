@@ -17,7 +17,7 @@ AUX_LIB_PATH = os.path.join(HERE, "librocwmma_amd_aux.so")
 
 SOURCES = ["api.hip", "gemm_wave_tile.hip", "gemm_blocked.hip", "gemm_streamk.hip", "gemm_skinny.hip", "gemm_mx.hip", "gemm_fused.hip", "gemv.hip", "dlrm.hip"]
 # test and benchmark support: fragment-API self-test kernels and measurement probes
-AUX_SOURCES = ["aux_api.hip", "selftest.hip", "mfma_ceiling.hip", "stream_ceiling.hip"]
+AUX_SOURCES = ["aux_api.hip", "selftest.hip", "mfma_ceiling.hip", "mfma_streams.hip", "stream_ceiling.hip"]
 
 # -packed-fp32-ops off: packed FP32 instructions are not generated for this target build.
 HIPCC_FLAGS = [
