@@ -357,6 +357,18 @@ def main():
             streams = run_streams_ceiling(rw, torch, dev, gen, dom_case[4], dom_case[5])
             roofline["mfma_with_operand_streams"] = streams
             roofline["frac_of_operand_streams_ceiling"] = round(per_case[dom]["tflops"] / streams["data"]["with_lds_reads_and_l2_copies"], 4)
+            if not args.only:
+                # the same for the instructions of the 8-bit kernels (same byte streams: 128 bytes of K per row and stage),
+                # on the operand distributions of the quantised cases
+                n8 = 8192 * 16384
+                a8 = torch.randint(-128, 128, (n8,), device=dev, dtype=torch.int8, generator=gen)
+                b8 = torch.randint(-128, 128, (n8,), device=dev, dtype=torch.int8, generator=gen)
+                roofline["mfma_with_operand_streams_8bit"] = {"i8_16x16x64": run_streams_ceiling(rw, torch, dev, gen, a8, b8, rw.STREAMS_I8)}
+                del a8, b8
+                a8 = (torch.randn(n8, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+                b8 = (torch.randn(n8, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+                roofline["mfma_with_operand_streams_8bit"]["fp8_16x16x128"] = run_streams_ceiling(rw, torch, dev, gen, a8, b8, rw.STREAMS_FP8)
+                del a8, b8
         roofline["zero_operands"] = {
             "ms": round(ms_zero, 4), "tflops": round(flops_per_gemm / ms_zero / 1e9, 1),
             "frac": round(flops_per_gemm / ms_zero / 1e9 / dom_peak, 4),
@@ -404,6 +416,10 @@ def main():
             if key in extra and shape in roofline.get("mfma_only_ceiling", {}):
                 extra[key]["frac_of_mfma_only_ceiling"] = round(
                     extra[key]["tops"] / roofline["mfma_only_ceiling"][shape]["data"], 4)
+            if key in extra and shape in roofline.get("mfma_with_operand_streams_8bit", {}):
+                # (main loop only: these launches also write 224 MiB of D, a quarter of their time)
+                extra[key]["frac_of_operand_streams_ceiling"] = round(
+                    extra[key]["tops"] / roofline["mfma_with_operand_streams_8bit"][shape]["data"]["with_lds_reads_and_l2_copies"], 4)
     if args.shapes:
         extra["shapes"] = run_shapes(rw, torch, dev, gen)
 
@@ -418,11 +434,14 @@ def main():
     }))
 
 
-def run_streams_ceiling(rw, torch, dev, gen, A, B):
-    """TFLOP/s of the matrix-pipes-next-to-their-operand-streams probe (rocwmma_amd_bench_mfma_streams): matrix
+def run_streams_ceiling(rw, torch, dev, gen, A, B, kind=None):
+    """T(FL)OP/s of the matrix-pipes-next-to-their-operand-streams probe (rocwmma_amd_bench_mfma_streams): matrix
     instructions only, with the LDS fragment reads, with those and the global -> LDS copies; on the operands of
-    the timed GEMM and on all-zero ones.  Ten launches of four tiles per compute unit after ten warm-up launches."""
-    tables = {"data": (A[: 32768].contiguous().view(torch.uint8), A, B),
+    the timed GEMM (A, B: 128 MiB each, rows of 16 KiB) and on all-zero ones.  Ten launches of four tiles per compute
+    unit after ten warm-up launches."""
+    kind = rw.STREAMS_F16 if kind is None else kind
+    bytes_a = A.view(torch.uint8)
+    tables = {"data": (bytes_a[: 65536].contiguous(), A, B),
               "zero": (torch.zeros(65536, device=dev, dtype=torch.uint8), torch.zeros_like(A), None)}
     sink = torch.empty(rw.device_info()["compute_units"] * 512, device=dev)
     out = {}
@@ -430,7 +449,7 @@ def run_streams_ceiling(rw, torch, dev, gen, A, B):
         b_ = a_ if b_ is None else b_
         res = {}
         for name, streams in (("mfma_only", 0), ("with_lds_reads", 1), ("with_lds_reads_and_l2_copies", 3)):
-            fn = lambda: rw.bench_mfma_streams(streams, 4, a_, b_, table, sink)
+            fn = lambda: rw.bench_mfma_streams(streams, 4, a_, b_, table, sink, kind)
             ops = fn()
             for _ in range(9):
                 fn()

@@ -97,17 +97,20 @@ int rocwmma_amd_bench_mfma_ceiling(int         shape,
 
 /*
  * Matrix pipes next to their operand streams: what the device sustains when the matrix instructions of a
- * 256 x 256 tile of 16-bit operands (v_mfma_f32_16x16x32_f16, eight waves of 64 x 128 per compute unit) run next
- * to the byte streams such a tile needs per 64 of K, and nothing else: no barrier, no tile bookkeeping, no
- * epilogue.  streams = 0: matrix instructions only; 1: with the 192 KiB of fragment reads from LDS per stage; 3: with
- * those and the 64 KiB of global -> LDS copies per stage, walking the A / B panels in the tile order of an
- * 8192^3 problem.  `a`, `b`: 8192 x 8192 halves each, K contiguous (needed for streams = 3); `operands`: a
+ * 256 x 256 tile (eight waves of 64 x 128 per compute unit) run next to the byte streams such a tile needs per
+ * 128 bytes of K, and nothing else: no barrier, no tile bookkeeping, no epilogue.  kind = 0: 16-bit operands
+ * (v_mfma_f32_16x16x32_f16), 1: int8 (v_mfma_i32_16x16x64_i8), 2: fp8 (v_mfma_f32_16x16x128_f8f6f4, B fragments
+ * streamed through column buffers as in the kernel).  streams = 0: matrix instructions only; 1: with the
+ * 192 KiB of fragment reads from LDS per stage; 3: with those and the 64 KiB of global -> LDS copies per stage,
+ * walking the A / B panels in the tile order of an 8192 x 8192 problem with 16 KiB of K per row (K = 8192 halves or
+ * 16384 bytes).  `a`, `b`: 8192 rows of 16 KiB each, K contiguous (needed for streams = 3); `operands`: a
  * 64 KiB table of operand bits as for rocwmma_amd_bench_mfma_ceiling; `out`: 512 floats per compute unit;
  * tiles_per_workgroup: tiles (of 128 stages) each compute unit walks, at most 1024 / compute units; *ops: the
  * operations of the launch.  On a power-managed part each stream costs clock: the blocked GEMM is priced against
  * this figure next to the matrix-pipe ceiling and the nominal peak.  Has no counterpart in the reference.
  */
-int rocwmma_amd_bench_mfma_streams(int         streams,
+int rocwmma_amd_bench_mfma_streams(int         kind,
+                                   int         streams,
                                    uint32_t    tiles_per_workgroup,
                                    const void* a,
                                    const void* b,

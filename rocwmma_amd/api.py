@@ -122,7 +122,7 @@ def aux_library():
         L.rocwmma_amd_bench_mfma_ceiling.argtypes = [i, u, u, vp, vp, ctypes.POINTER(ctypes.c_double), vp]
         L.rocwmma_amd_bench_mfma_ceiling.restype = i
         L.rocwmma_amd_bench_stream.argtypes = [i, vp, vp, ctypes.c_size_t, vp]
-        L.rocwmma_amd_bench_mfma_streams.argtypes = [i, u, vp, vp, vp, vp, ctypes.POINTER(ctypes.c_double), vp]
+        L.rocwmma_amd_bench_mfma_streams.argtypes = [i, i, u, vp, vp, vp, vp, ctypes.POINTER(ctypes.c_double), vp]
         L.rocwmma_amd_bench_mfma_streams.restype = i
         L.rocwmma_amd_bench_stream.restype = i
         _aux = L
@@ -354,12 +354,15 @@ def bench_stream(mode, src, dst, nbytes, stream=None):
                                                   stream if stream is not None else _stream()), "bench_stream")
 
 
-def bench_mfma_streams(streams, tiles_per_workgroup, a, b, operands, out):
+STREAMS_F16, STREAMS_I8, STREAMS_FP8 = 0, 1, 2
+
+
+def bench_mfma_streams(streams, tiles_per_workgroup, a, b, operands, out, kind=STREAMS_F16):
     """Launches the matrix-pipes-next-to-their-operand-streams probe (include/rocwmma_amd_aux.h); returns the
     operation count of the launch."""
     ops = ctypes.c_double(0.0)
-    _check(aux_library().rocwmma_amd_bench_mfma_streams(streams, tiles_per_workgroup, _ptr(a), _ptr(b), _ptr(operands), _ptr(out),
-                                                        ctypes.byref(ops), _stream()), "bench_mfma_streams")
+    _check(aux_library().rocwmma_amd_bench_mfma_streams(kind, streams, tiles_per_workgroup, _ptr(a), _ptr(b), _ptr(operands),
+                                                        _ptr(out), ctypes.byref(ops), _stream()), "bench_mfma_streams")
     return ops.value
 
 

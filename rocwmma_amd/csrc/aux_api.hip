@@ -14,7 +14,7 @@ namespace rocwmma_amd
     int benchMfmaCeiling(int shape, uint32_t trips, uint32_t wavesPerSimd, const void* operands, float* out, double* ops,
                          hipStream_t stream);
     int benchStream(int mode, const void* src, void* dst, size_t bytes, hipStream_t stream);
-    int benchMfmaStreams(int streams, uint32_t tilesPerWorkgroup, const void* a, const void* b, const void* operands, float* out,
+    int benchMfmaStreams(int kind, int streams, uint32_t tilesPerWorkgroup, const void* a, const void* b, const void* operands, float* out,
                          double* ops, hipStream_t stream);
 
     namespace
@@ -99,7 +99,8 @@ int rocwmma_amd_bench_mfma_ceiling(int         shape,
     return benchMfmaCeiling(shape, trips, waves_per_simd, operands, out, ops, asStream(stream));
 }
 
-int rocwmma_amd_bench_mfma_streams(int         streams,
+int rocwmma_amd_bench_mfma_streams(int         kind,
+                                   int         streams,
                                    uint32_t    tiles_per_workgroup,
                                    const void* a,
                                    const void* b,
@@ -112,7 +113,7 @@ int rocwmma_amd_bench_mfma_streams(int         streams,
         return ROCWMMA_AMD_BAD_ALIGNMENT;
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
-    return benchMfmaStreams(streams, tiles_per_workgroup, a, b, operands, out, ops, asStream(stream));
+    return benchMfmaStreams(kind, streams, tiles_per_workgroup, a, b, operands, out, ops, asStream(stream));
 }
 
 int rocwmma_amd_bench_stream(int mode, const void* src, void* dst, size_t bytes, void* stream)

@@ -24,6 +24,19 @@ def test_matrix_pipes_next_to_their_operand_streams():
         assert bool(torch.isfinite(out).all())
     assert rw.bench_mfma_streams(3, 2, a, a, table, out) == 2 * 2.0 * 256 * 256 * 8192 * units
     torch.cuda.synchronize()
+    # the 8-bit kinds walk rows of the same 16 KiB: twice the K
+    a8 = torch.randint(-128, 128, (s * s * 2,), device="cuda", dtype=torch.int8)
+    f8 = (torch.randn(s * s * 2, device="cuda") * 0.1).to(torch.float8_e4m3fn)
+    for kind, panel in ((rw.STREAMS_I8, a8), (rw.STREAMS_FP8, f8)):
+        for streams in (0, 1, 3):
+            out.fill_(float("nan"))
+            ops = rw.bench_mfma_streams(streams, 1, panel, panel, panel.view(torch.uint8)[:65536].contiguous(), out, kind)
+            torch.cuda.synchronize()
+            assert ops == 2.0 * 256 * 256 * 16384 * units
+            assert bool(torch.isfinite(out).all())
+    with pytest.raises(rw.RocwmmaError) as e:  # unknown instruction kind
+        rw.bench_mfma_streams(0, 1, a, a, table, out, 3)
+    assert e.value.status == 1
     for bad in (2, 4, -1):  # copies without reads, unknown bits
         with pytest.raises(rw.RocwmmaError) as e:
             rw.bench_mfma_streams(bad, 1, a, a, table, out)
