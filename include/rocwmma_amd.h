@@ -479,6 +479,33 @@ int rocwmma_amd_dlrm_bwd(const void* input,
                          uint32_t    batch,
                          void*       stream);
 
+/*
+ * The two DLRM passes with the element type as an argument: ROCWMMA_AMD_F16 (the entry points above) or
+ * ROCWMMA_AMD_F32.  The reference's DLRM kernels and tests are templates over the element type and are
+ * instantiated for float32_t as well (test/dlrm/test/dlrm_test_params.hpp:51; fp32 data files under
+ * test/dlrm/data); semantics = dlrm_fwd_CPU / dlrm_bwd_CPU with DataT = float (test/reference_impl.hpp:83-179).
+ * Same shapes, limits and alignment as above (m <= 128, k in {32, 64, 128, 256}, 16-byte aligned pointers); the
+ * float32 kernels multiply with v_mfma_f32_32x32x2_f32 and are written for parity, not tuned.  Other element
+ * types: ROCWMMA_AMD_UNSUPPORTED_TYPE.
+ */
+int rocwmma_amd_dlrm_fwd_ex(int         dtype,
+                            const void* input,
+                            void*       output,
+                            uint32_t    m,
+                            uint32_t    k,
+                            uint32_t    batch,
+                            void*       stream);
+
+int rocwmma_amd_dlrm_bwd_ex(int         dtype,
+                            const void* input,
+                            const void* upstream_grad,
+                            void*       grad,
+                            void*       bottom_mlp_grad,
+                            uint32_t    m,
+                            uint32_t    k,
+                            uint32_t    batch,
+                            void*       stream);
+
 #ifdef __cplusplus
 }
 #endif

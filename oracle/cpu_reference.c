@@ -31,7 +31,9 @@
  *   - identity / all-ones / exact-integer closed forms, int8 against numpy int64;
  *   - f16 / bf16 / e4m3 / e5m2 codecs against numpy / the OCP closed form, all codes;
  *   - DLRM forward and backward against the reference's golden files
- *     the five fp16 files of test/dlrm/data (committed under tests/golden/ as dlrm_<name>.bin).
+ *     the five fp16 files of test/dlrm/data (committed under tests/golden/ as dlrm_<name>.bin);
+ *   - the float32 forms of the two DLRM loops against the first 16 samples of the five fp32 files of the same
+ *     directory, and against the f16 forms on f16-representable inputs (equal after one rounding).
  */
 #include <math.h>
 #include <stdint.h>
@@ -678,6 +680,77 @@ void oracle_dlrm_bwd_f16(const uint16_t* input,
         }
         free(acc);
         free(in);
+    }
+}
+
+/* ---- DLRM forward / backward, DataT = float (the same loops with the identity for the conversions; the
+ * reference's DLRM tests instantiate float32_t as well, test/dlrm/test/dlrm_test_params.hpp:51, and its data
+ * directory holds fp32 fixtures next to the fp16 ones) ----------------------------------------------------- */
+void oracle_dlrm_fwd_f32(const float* input, float* output, uint32_t m, uint32_t k, uint32_t batch)
+{
+    size_t batchOffset       = (size_t)m * k;
+    size_t outputBatchOffset = ((size_t)m * (m - 1)) / 2 + k;
+    long   b;
+#pragma omp parallel for
+    for(b = 0; b < (long)batch; b++)
+    {
+        size_t outputIdx = b * outputBatchOffset;
+        for(uint32_t i = 0; i < k; i++)
+            output[outputIdx++] = input[b * batchOffset + i];
+        for(uint32_t i = 0; i < m; i++)
+            for(uint32_t j = 0; j < i; j++) /* (the reference computes and discards j >= i) */
+            {
+                float accum = 0.0f;
+                for(uint32_t h = 0; h < k; h++)
+                    accum += input[b * batchOffset + (size_t)i * k + h] * input[b * batchOffset + (size_t)j * k + h];
+                output[outputIdx++] = accum;
+            }
+    }
+}
+
+void oracle_dlrm_bwd_f32(const float* input,
+                         const float* upstreamGrad,
+                         float*       bottomMlpGrad,
+                         float*       output,
+                         uint32_t     m,
+                         uint32_t     k,
+                         uint32_t     batch)
+{
+    size_t batchOffset = (size_t)m * k;
+    size_t accOffset   = (size_t)m * m;
+    size_t trilSize    = ((size_t)m * (m - 1)) / 2 + k;
+    long   b;
+#pragma omp parallel
+    {
+        float* acc = (float*)malloc(accOffset * sizeof(float));
+#pragma omp for
+        for(b = 0; b < (long)batch; b++)
+        {
+            for(uint32_t j = 0; j < k; j++)
+                bottomMlpGrad[b * (size_t)k + j] = upstreamGrad[b * trilSize + j];
+            size_t upstreamIdx = b * trilSize + k;
+            for(uint32_t i = 0; i < m; i++)
+                for(uint32_t j = 0; j <= i; j++)
+                {
+                    if(i == j)
+                        acc[(size_t)i * m + j] = 0.0f;
+                    else
+                    {
+                        float g                = upstreamGrad[upstreamIdx++];
+                        acc[(size_t)i * m + j] = g;
+                        acc[(size_t)j * m + i] = g;
+                    }
+                }
+            for(uint32_t i = 0; i < m; i++)
+                for(uint32_t j = 0; j < k; j++)
+                {
+                    float accum = 0.0f;
+                    for(uint32_t h = 0; h < m; h++)
+                        accum += acc[(size_t)i * m + h] * input[b * batchOffset + (size_t)h * k + j];
+                    output[b * batchOffset + (size_t)i * k + j] = accum;
+                }
+        }
+        free(acc);
     }
 }
 

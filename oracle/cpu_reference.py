@@ -42,6 +42,10 @@ def lib():
         L.oracle_dlrm_fwd_f16.restype = None
         L.oracle_dlrm_bwd_f16.argtypes = [vp, vp, vp, vp, u32, u32, u32]
         L.oracle_dlrm_bwd_f16.restype = None
+        L.oracle_dlrm_fwd_f32.argtypes = [vp, vp, u32, u32, u32]
+        L.oracle_dlrm_fwd_f32.restype = None
+        L.oracle_dlrm_bwd_f32.argtypes = [vp, vp, vp, vp, u32, u32, u32]
+        L.oracle_dlrm_bwd_f32.restype = None
         L.oracle_compare_equal.argtypes = [i, vp, i, vp, ctypes.c_size_t, ctypes.POINTER(i)]
         L.oracle_compare_equal.restype = dbl
         L.oracle_encode.argtypes = [i, vp, vp, ctypes.c_size_t]
@@ -179,26 +183,36 @@ def gemm_bias_act(dtype_in, dtype_out, layA, layB, layC, m, n, k, a, b, c, alpha
     return out
 
 
-def dlrm_fwd(inp, m, k, batch):
-    """dlrm_fwd_CPU (test/reference_impl.hpp:83-119) on f16 bit patterns."""
+def dlrm_fwd(inp, m, k, batch, dtype=F16):
+    """dlrm_fwd_CPU (test/reference_impl.hpp:83-119) on f16 bit patterns (dtype F16) or float32 values (F32)."""
+    width = m * (m - 1) // 2 + k
+    if dtype == F32:
+        inp = np.ascontiguousarray(inp, dtype=np.float32).reshape(-1)
+        assert inp.size == batch * m * k
+        out = np.zeros(batch * width, dtype=np.float32)
+        lib().oracle_dlrm_fwd_f32(_ptr(inp), _ptr(out), m, k, batch)
+        return out.reshape(batch, width)
+    assert dtype == F16
     inp = np.ascontiguousarray(inp, dtype=np.uint16).reshape(-1)
     assert inp.size == batch * m * k
-    width = m * (m - 1) // 2 + k
     out = np.zeros(batch * width, dtype=np.uint16)
     lib().oracle_dlrm_fwd_f16(_ptr(inp), _ptr(out), m, k, batch)
     return out.reshape(batch, width)
 
 
-def dlrm_bwd(inp, upstream, m, k, batch):
-    """dlrm_bwd_CPU (test/reference_impl.hpp:121-179) on f16 bit patterns.
+def dlrm_bwd(inp, upstream, m, k, batch, dtype=F16):
+    """dlrm_bwd_CPU (test/reference_impl.hpp:121-179) on f16 bit patterns (dtype F16) or float32 values (F32).
     Returns (grad[batch,m,k], bottom_mlp_grad[batch,k])."""
-    inp = np.ascontiguousarray(inp, dtype=np.uint16).reshape(-1)
-    upstream = np.ascontiguousarray(upstream, dtype=np.uint16).reshape(-1)
     width = m * (m - 1) // 2 + k
+    np_t = np.float32 if dtype == F32 else np.uint16
+    assert dtype in (F16, F32)
+    inp = np.ascontiguousarray(inp, dtype=np_t).reshape(-1)
+    upstream = np.ascontiguousarray(upstream, dtype=np_t).reshape(-1)
     assert inp.size == batch * m * k and upstream.size == batch * width
-    grad = np.zeros(batch * m * k, dtype=np.uint16)
-    mlp = np.zeros(batch * k, dtype=np.uint16)
-    lib().oracle_dlrm_bwd_f16(_ptr(inp), _ptr(upstream), _ptr(mlp), _ptr(grad), m, k, batch)
+    grad = np.zeros(batch * m * k, dtype=np_t)
+    mlp = np.zeros(batch * k, dtype=np_t)
+    fn = lib().oracle_dlrm_bwd_f32 if dtype == F32 else lib().oracle_dlrm_bwd_f16
+    fn(_ptr(inp), _ptr(upstream), _ptr(mlp), _ptr(grad), m, k, batch)
     return grad.reshape(batch, m, k), mlp.reshape(batch, k)
 
 

@@ -21,6 +21,7 @@ EXPORTS = [
     "rocwmma_amd_gemm_streamk", "rocwmma_amd_gemm_streamk_workspace_size", "rocwmma_amd_gemm_streamk_static",
     "rocwmma_amd_gemm_mx", "rocwmma_amd_gemm_mx_workspace_size", "rocwmma_amd_gemm_bias_act",
     "rocwmma_amd_gemm_streamk_timed_out", "rocwmma_amd_gemm_mx_pack_scales", "rocwmma_amd_gemm_mx_packed",
+    "rocwmma_amd_dlrm_fwd_ex", "rocwmma_amd_dlrm_bwd_ex",
 ]
 ACT_NONE, ACT_RELU, ACT_GELU = range(3)
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
@@ -95,6 +96,10 @@ def library():
         L.rocwmma_amd_dlrm_fwd.restype = i
         L.rocwmma_amd_dlrm_bwd.argtypes = [vp, vp, vp, vp, u, u, u, vp]
         L.rocwmma_amd_dlrm_bwd.restype = i
+        L.rocwmma_amd_dlrm_fwd_ex.argtypes = [i, vp, vp, u, u, u, vp]
+        L.rocwmma_amd_dlrm_fwd_ex.restype = i
+        L.rocwmma_amd_dlrm_bwd_ex.argtypes = [i, vp, vp, vp, vp, u, u, u, vp]
+        L.rocwmma_amd_dlrm_bwd_ex.restype = i
         _lib = L
     return _lib
 
@@ -321,14 +326,23 @@ def gemv(m, k, ncols, a, x, y, alpha=1.0, beta=0.0, lda=None, ldx=None, ldy=None
     return y
 
 
-def dlrm_fwd(inp, out, m, k, batch):
-    _check(library().rocwmma_amd_dlrm_fwd(_ptr(inp), _ptr(out), m, k, batch, _stream()), "dlrm_fwd")
+def dlrm_fwd(inp, out, m, k, batch, dtype=None):
+    """DLRM dot interaction, forward; dtype None: the f16 entry point, else rocwmma_amd_dlrm_fwd_ex (F16 or F32)."""
+    if dtype is None:
+        _check(library().rocwmma_amd_dlrm_fwd(_ptr(inp), _ptr(out), m, k, batch, _stream()), "dlrm_fwd")
+    else:
+        _check(library().rocwmma_amd_dlrm_fwd_ex(dtype, _ptr(inp), _ptr(out), m, k, batch, _stream()), "dlrm_fwd_ex")
     return out
 
 
-def dlrm_bwd(inp, upstream, grad, mlp_grad, m, k, batch):
-    _check(library().rocwmma_amd_dlrm_bwd(_ptr(inp), _ptr(upstream), _ptr(grad), _ptr(mlp_grad), m, k, batch,
-                                          _stream()), "dlrm_bwd")
+def dlrm_bwd(inp, upstream, grad, mlp_grad, m, k, batch, dtype=None):
+    """DLRM dot interaction, backward; dtype None: the f16 entry point, else rocwmma_amd_dlrm_bwd_ex (F16 or F32)."""
+    if dtype is None:
+        _check(library().rocwmma_amd_dlrm_bwd(_ptr(inp), _ptr(upstream), _ptr(grad), _ptr(mlp_grad), m, k, batch,
+                                              _stream()), "dlrm_bwd")
+    else:
+        _check(library().rocwmma_amd_dlrm_bwd_ex(dtype, _ptr(inp), _ptr(upstream), _ptr(grad), _ptr(mlp_grad), m, k, batch,
+                                                 _stream()), "dlrm_bwd_ex")
     return grad, mlp_grad
 
 

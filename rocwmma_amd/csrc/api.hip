@@ -12,6 +12,9 @@ namespace rocwmma_amd
     int launchGemv(uint32_t m, uint32_t k, uint32_t ncols, const void* a, uint32_t lda, const void* x, uint32_t ldx,
                    float* y, uint32_t ldy, float alpha, float beta, hipStream_t stream);
     int launchDlrmFwd(const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, hipStream_t stream);
+    int launchDlrmFwdF32(const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, hipStream_t stream);
+    int launchDlrmBwdF32(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t k, uint32_t batch,
+                         hipStream_t stream);
     int launchDlrmBwd(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t k,
                       uint32_t batch, hipStream_t stream);
 
@@ -606,6 +609,50 @@ int rocwmma_amd_dlrm_bwd(const void* input,
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
     return launchDlrmBwd(input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
+}
+
+int rocwmma_amd_dlrm_fwd_ex(int dtype, const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, void* stream)
+{
+    if(dtype == ROCWMMA_AMD_F16)
+        return rocwmma_amd_dlrm_fwd(input, output, m, k, batch, stream);
+    if(dtype != ROCWMMA_AMD_F32)
+        return ROCWMMA_AMD_UNSUPPORTED_TYPE;
+    if(!input || !output)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    int rc = checkDlrm(m, k, batch);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(!aligned16(input) || !aligned16(output))
+        return ROCWMMA_AMD_BAD_ALIGNMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return launchDlrmFwdF32(input, output, m, k, batch, asStream(stream));
+}
+
+int rocwmma_amd_dlrm_bwd_ex(int         dtype,
+                            const void* input,
+                            const void* upstream_grad,
+                            void*       grad,
+                            void*       bottom_mlp_grad,
+                            uint32_t    m,
+                            uint32_t    k,
+                            uint32_t    batch,
+                            void*       stream)
+{
+    if(dtype == ROCWMMA_AMD_F16)
+        return rocwmma_amd_dlrm_bwd(input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, stream);
+    if(dtype != ROCWMMA_AMD_F32)
+        return ROCWMMA_AMD_UNSUPPORTED_TYPE;
+    if(!input || !upstream_grad || !grad || !bottom_mlp_grad)
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    int rc = checkDlrm(m, k, batch);
+    if(rc != ROCWMMA_AMD_OK)
+        return rc;
+    if(!aligned16(input) || !aligned16(upstream_grad) || !aligned16(grad) || !aligned16(bottom_mlp_grad))
+        return ROCWMMA_AMD_BAD_ALIGNMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return launchDlrmBwdF32(input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
 }
 
 } // extern "C"

@@ -134,6 +134,16 @@ def test_gemv_and_dlrm_argument_validation(lib):
     h = lib.rocwmma_amd_dlrm_bwd
     assert h(4096, 8192, 12288, None, 27, 128, 8, None) == 1
     assert h(4096, 8192, 12290, 16384, 27, 128, 8, None) == 4
+    # the entry points with an element type: float32 and f16 only, same checks
+    gx, hx = lib.rocwmma_amd_dlrm_fwd_ex, lib.rocwmma_amd_dlrm_bwd_ex
+    F16, BF16, F32, I8 = 0, 1, 5, 4
+    assert gx(BF16, 4096, 8192, 27, 128, 8, None) == 2 and hx(I8, 4096, 8192, 12288, 16384, 27, 128, 8, None) == 2
+    for t in (F16, F32):
+        assert gx(t, None, 4096, 27, 128, 8, None) == 1
+        assert gx(t, 4096, 8192, 129, 128, 8, None) == 3
+        assert gx(t, 4096, 8192, 27, 100, 8, None) == 3
+        assert hx(t, 4096, 8192, 12288, None, 27, 128, 8, None) == 1
+        assert hx(t, 4096, 8192, 12290, 16384, 27, 128, 8, None) == 4
 
 
 def test_product_code_never_touches_the_oracle():

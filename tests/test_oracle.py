@@ -398,6 +398,44 @@ def test_dlrm_bwd_against_reference_golden_files(golden_dir):
     assert orc.compare_equal(orc.F16, orc.encode(orc.F16, g), orc.F16, want_grad)[0] > 0.1
 
 
+def test_dlrm_float32_against_reference_golden_files(golden_dir):
+    """The float32 form of the two loops against the first 16 samples of the reference's fp32 data files
+    (test/dlrm/data/*_fp32; tests/golden/extract_fp32.py).  The fixtures come from another summation order: 9.8 eps in
+    the compareEqual metric, inside the reference's 10 * eps for float32_t."""
+    b, m, k = 16, M_, K_
+    g = lambda name, shape: np.fromfile(os.path.join(golden_dir, f"dlrm_{name}.bin"), dtype=np.float32).reshape(shape)
+    inp, up = g("input_fp32", (b, m, k)), g("input_grad_fp32", (b, W_))
+    got = orc.dlrm_fwd(inp, m, k, b, orc.F32)
+    err, inf, nan = orc.compare_equal(orc.F32, got, orc.F32, g("output_fp32", (b, W_)))
+    assert not inf and not nan and err <= 10 * 2.0 ** -23
+    assert np.array_equal(got[:, :k], inp[:, 0, :])
+    swapped = np.concatenate([got[:, k:], got[:, :k]], axis=1)
+    assert orc.compare_equal(orc.F32, swapped, orc.F32, g("output_fp32", (b, W_)))[0] > 0.1
+    grad, mlp = orc.dlrm_bwd(inp, up, m, k, b, orc.F32)
+    assert np.array_equal(mlp, g("output_mlp_input_grad_fp32", (b, k))) and np.array_equal(mlp, up[:, :k])
+    err, inf, nan = orc.compare_equal(orc.F32, grad, orc.F32, g("output_input_grad_fp32", (b, m, k)))
+    assert not inf and not nan and err <= 10 * 2.0 ** -23
+    with_mlp = grad.copy()
+    with_mlp[:, 0, :] += mlp
+    assert orc.compare_equal(orc.F32, with_mlp, orc.F32, g("output_input_grad_fp32", (b, m, k)))[0] > 0.1
+
+
+def test_dlrm_float32_equals_the_f16_loops_on_f16_representable_data():
+    """On inputs that are exactly representable in f16 the two element types run the same float accumulation: the f16
+    results are the float32 results rounded once."""
+    rng = np.random.default_rng(11)
+    b, m, k = 4, 27, 64
+    F = rng.uniform(-1, 1, (b, m, k)).astype(np.float16)
+    up = rng.uniform(-1, 1, (b, m * (m - 1) // 2 + k)).astype(np.float16)
+    out16 = orc.dlrm_fwd(F.view(np.uint16), m, k, b)
+    out32 = orc.dlrm_fwd(F.astype(np.float32), m, k, b, orc.F32)
+    assert np.array_equal(out16, orc.encode(orc.F16, out32.reshape(-1)).reshape(out16.shape))
+    g16, m16 = orc.dlrm_bwd(F.view(np.uint16), up.view(np.uint16), m, k, b)
+    g32, m32 = orc.dlrm_bwd(F.astype(np.float32), up.astype(np.float32), m, k, b, orc.F32)
+    assert np.array_equal(g16, orc.encode(orc.F16, g32.reshape(-1)).reshape(g16.shape))
+    assert np.array_equal(m16.view(np.float16).astype(np.float32), m32)
+
+
 def test_dlrm_fwd_bwd_against_numpy_float64():
     rng = np.random.default_rng(7)
     b, m, k = 5, 27, 128
