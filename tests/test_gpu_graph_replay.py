@@ -129,6 +129,26 @@ def test_dlrm_replays(batch):
     _replays_match(call, [out, grad, mlp])
 
 
+@pytest.mark.parametrize("batch,m", [(64, 27), (5, 128)])
+def test_dlrm_float32_replays(batch, m):
+    import torch
+
+    k = 128
+    width = k + m * (m - 1) // 2
+    rng = np.random.default_rng(43)
+    dfe = to_device(rng.uniform(-1, 1, batch * m * k).astype(np.float32))
+    dup = to_device(rng.uniform(-1, 1, batch * width).astype(np.float32))
+    out = torch.empty(batch * width, device="cuda")
+    grad = torch.empty(batch * m * k, device="cuda")
+    mlp = torch.empty(batch * k, device="cuda")
+
+    def call():
+        rw.dlrm_fwd(dfe, out, m, k, batch, rw.F32)
+        rw.dlrm_bwd(dfe, dup, grad, mlp, m, k, batch, rw.F32)
+
+    _replays_match(call, [out, grad, mlp])
+
+
 def test_block_scaled_gemm_replays():
     """Two launches per call (scale re-ordering into the workspace, then the GEMM): both are in the graph."""
     import torch
