@@ -412,7 +412,8 @@ def main():
     if not args.no_extras and not args.only:
         extra.update(run_extras(rw, torch, dev, gen))
         # the MFMA-bound quantised case against the matrix pipes' own ceiling for its instruction
-        for key, shape in (("gemm_i8_m4096", "i8_16x16x64"), ("gemm_fp8_m4096", FP8_BLOCKED_SHAPE)):
+        for key, shape in (("gemm_i8_m4096", "i8_16x16x64"), ("gemm_fp8_m4096", FP8_BLOCKED_SHAPE),
+                           ("gemm_i8_8192cubed", "i8_16x16x64"), ("gemm_fp8_8192cubed", FP8_BLOCKED_SHAPE)):
             if key in extra and shape in roofline.get("mfma_only_ceiling", {}):
                 extra[key]["frac_of_mfma_only_ceiling"] = round(
                     extra[key]["tops"] / roofline["mfma_only_ceiling"][shape]["data"], 4)
@@ -692,6 +693,34 @@ def run_extras(rw, torch, dev, gen, only=None):
                     out[f"gemm_{tag}_m{m}"].update({"ms_graph_replay": round(msg, 4), "gbs_graph_replay": round(byts / msg / 1e6, 1),
                                                     "frac_hbm_graph_replay": round(byts / msg / 1e6 / PEAK_HBM_GBS, 4)})
         del Bq, Bf
+
+    # the headline size with the 8-bit types (A row / B col, alpha = 1, beta = 0; operands as in config 3):
+    # the size the fp8 / int8 targets are quoted on next to the f16 / bf16 one
+    for tag in ("i8", "fp8"):
+        key = f"gemm_{tag}_8192cubed"
+        if not wanted(key):
+            continue
+        sz = 8192
+        if tag == "i8":
+            A8 = torch.randint(-128, 128, (sz * sz,), device=dev, dtype=torch.int8, generator=gen)
+            B8 = torch.randint(-128, 128, (sz * sz,), device=dev, dtype=torch.int8, generator=gen)
+            D8 = torch.empty(sz * sz, device=dev, dtype=torch.int32)
+            code, ocode = rw.I8, rw.I32
+        else:
+            A8 = (torch.randn(sz * sz, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+            B8 = (torch.randn(sz * sz, device=dev, generator=gen) * 0.1).to(torch.float8_e4m3fn)
+            D8 = torch.empty(sz * sz, device=dev, dtype=torch.float32)
+            code, ocode = rw.E4M3, rw.F32
+
+        def fn8():
+            rw.gemm(code, ocode, RM, CM, RM, sz, sz, sz, A8, B8, None, D8, 1.0, 0.0)
+
+        fn8()
+        fn8()
+        ms = event_ms(fn8, iters, torch)
+        out[key] = {"ms": round(ms, 4), "tops": round(2.0 * sz ** 3 / ms / 1e9, 1),
+                    "frac_mfma": round(2.0 * sz ** 3 / ms / 1e9 / PEAK_TFLOPS[tag], 4)}
+        del A8, B8, D8
 
     # config 3's fp8 shape with block scales (one E8M0 byte per 32 elements of K): the same blocked kernel
     # on the scaled matrix instruction, plus the small kernels that re-order the scales
