@@ -613,6 +613,28 @@ def run_extras(rw, torch, dev, gen, only=None):
                             "32x32x16 blocks, 128 x 128 macro tile, single LDS buffer"}
         del Ap, Bp, Cp, Dp
 
+    # The same through the public fragment API only, laid out for this device instead of after perf_hgemm:
+    # 256 x 256 macro tile, eight waves, 16 x 16 x 32 blocks, two padded LDS buffers, the next K stage prefetched.
+    for tag, la_, lb_ in (("cr", CM, RM), ("rc", RM, CM)):
+        key = f"public_api_tiled_gemm_f16_{tag}_8192"
+        if not wanted(key):
+            continue
+        sz = 8192
+        Ap = (torch.rand(sz * sz, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        Bp = (torch.rand(sz * sz, device=dev, generator=gen) * 2 - 1).to(torch.float16)
+        Cp = torch.rand(sz * sz, device=dev, generator=gen) * 2 - 1
+        Dp = torch.empty(sz * sz, device=dev)
+
+        def fnt():
+            rw.selftest_tiled_gemm(la_, lb_, sz, sz, sz, Ap, Bp, Cp, Dp, 1.0, 1.0)
+
+        fnt()
+        ms = event_ms(fnt, 5, torch)
+        out[key] = {"ms": round(ms, 3), "tflops": round(2.0 * sz ** 3 / ms / 1e9, 1),
+                    "note": "fragment API only (load/store_matrix_coop_sync, applyDataLayout, applyTranspose, mma_sync); "
+                            "16x16x32 blocks, 256 x 256 macro tile, two LDS buffers of 64 + 8 halves per row"}
+        del Ap, Bp, Cp, Dp
+
     # the headline f16 A-row / B-col GEMM with the fused epilogue (bias per column, GELU) against the same
     # GEMM without it: what the epilogue costs when it rides on the accumulators
     if wanted("gemm_f16_rc_8192_bias_gelu"):

@@ -62,6 +62,24 @@ int rocwmma_amd_selftest_coop_gemm(int         layout_a,
                                    float       beta,
                                    void*       stream);
 
+/* A blocked GEMM written only against the public API and laid out for gfx950 instead of after perf_hgemm
+ * (256 x 256 macro tile, eight waves of 64 x 128, 16 x 16 x 32 blocks, K stages of 64 in two padded LDS buffers,
+ * the next stage prefetched with cooperative loads), f16 in / f32 out, the four A/B layout combinations, row-major
+ * C / D with leading dimension n; m, n multiples of 256, k a multiple of 64.  What a kernel ported to this device
+ * reaches through the fragment API alone; the benchmark reports it next to the perf_hgemm data flow above. */
+int rocwmma_amd_selftest_tiled_gemm(int         layout_a,
+                                    int         layout_b,
+                                    uint32_t    m,
+                                    uint32_t    n,
+                                    uint32_t    k,
+                                    const void* a,
+                                    const void* b,
+                                    const float* c,
+                                    float*      d,
+                                    float       alpha,
+                                    float       beta,
+                                    void*       stream);
+
 /* Instruction shapes of rocwmma_amd_bench_mfma_ceiling. */
 typedef enum rocwmma_amd_mfma_shape
 {

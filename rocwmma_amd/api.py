@@ -26,7 +26,7 @@ EXPORTS = [
 ACT_NONE, ACT_RELU, ACT_GELU = range(3)
 # librocwmma_amd_aux.so: test and benchmark support (include/rocwmma_amd_aux.h)
 _AUX_LIB_NAME = "librocwmma_amd_aux.so"
-AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_bench_mfma_ceiling",
+AUX_EXPORTS = ["rocwmma_amd_selftest_roundtrip", "rocwmma_amd_selftest_coop_gemm", "rocwmma_amd_selftest_tiled_gemm", "rocwmma_amd_bench_mfma_ceiling",
                "rocwmma_amd_bench_stream", "rocwmma_amd_bench_mfma_streams"]
 (MFMA_F16_16X16X32, MFMA_F16_32X32X16, MFMA_BF16_16X16X32, MFMA_BF16_32X32X16, MFMA_I8_16X16X64, MFMA_I8_32X32X32,
  MFMA_F8_16X16X128, MFMA_F8_32X32X64, MFMA_F8_16X16X128_SCALED) = range(9)
@@ -124,6 +124,8 @@ def aux_library():
         L.rocwmma_amd_selftest_roundtrip.restype = i
         L.rocwmma_amd_selftest_coop_gemm.argtypes = [i, i, u, u, u, vp, vp, vp, vp, f, f, vp]
         L.rocwmma_amd_selftest_coop_gemm.restype = i
+        L.rocwmma_amd_selftest_tiled_gemm.argtypes = [i, i, u, u, u, vp, vp, vp, vp, f, f, vp]
+        L.rocwmma_amd_selftest_tiled_gemm.restype = i
         L.rocwmma_amd_bench_mfma_ceiling.argtypes = [i, u, u, vp, vp, ctypes.POINTER(ctypes.c_double), vp]
         L.rocwmma_amd_bench_mfma_ceiling.restype = i
         L.rocwmma_amd_bench_stream.argtypes = [i, vp, vp, ctypes.c_size_t, vp]
@@ -355,6 +357,12 @@ def selftest_roundtrip(context, dtype, layout, block, blockk, coop, rows, cols, 
 def selftest_coop_gemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta):
     _check(aux_library().rocwmma_amd_selftest_coop_gemm(layout_a, layout_b, m, n, k, _ptr(a), _ptr(b), _ptr(c), _ptr(d),
                                                     alpha, beta, _stream()), "selftest_coop_gemm")
+    return d
+
+
+def selftest_tiled_gemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta):
+    _check(aux_library().rocwmma_amd_selftest_tiled_gemm(layout_a, layout_b, m, n, k, _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+                                                     alpha, beta, _stream()), "selftest_tiled_gemm")
     return d
 
 

@@ -9,6 +9,8 @@ namespace rocwmma_amd
 {
     int selftestRoundtrip(int context, int dtype, int layout, int block, int blockk, int coop, uint32_t rows, uint32_t cols,
                           const void* in, void* out, uint32_t ld, hipStream_t stream);
+    int selftestTiledGemm(int layoutA, int layoutB, uint32_t m, uint32_t n, uint32_t k, const void* a, const void* b, const float* c,
+                          float* d, float alpha, float beta, hipStream_t stream);
     int selftestCoopGemm(int layoutA, int layoutB, uint32_t m, uint32_t n, uint32_t k, const void* a, const void* b,
                          const float* c, float* d, float alpha, float beta, hipStream_t stream);
     int benchMfmaCeiling(int shape, uint32_t trips, uint32_t wavesPerSimd, const void* operands, float* out, double* ops,
@@ -82,6 +84,28 @@ int rocwmma_amd_selftest_coop_gemm(int          layout_a,
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
     return selftestCoopGemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta, asStream(stream));
+}
+
+int rocwmma_amd_selftest_tiled_gemm(int          layout_a,
+                                    int          layout_b,
+                                    uint32_t     m,
+                                    uint32_t     n,
+                                    uint32_t     k,
+                                    const void*  a,
+                                    const void*  b,
+                                    const float* c,
+                                    float*       d,
+                                    float        alpha,
+                                    float        beta,
+                                    void*        stream)
+{
+    if(!a || !b || !c || !d || !validLayout(layout_a) || !validLayout(layout_b))
+        return ROCWMMA_AMD_INVALID_ARGUMENT;
+    if(!aligned16(a) || !aligned16(b) || !aligned16(c) || !aligned16(d))
+        return ROCWMMA_AMD_BAD_ALIGNMENT;
+    if(!isGfx950Current())
+        return ROCWMMA_AMD_NO_DEVICE;
+    return selftestTiledGemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta, asStream(stream));
 }
 
 int rocwmma_amd_bench_mfma_ceiling(int         shape,

@@ -301,7 +301,174 @@ namespace rocwmma_amd
                 return launchStatus();
             }
         } // namespace flow
+        // ---- a blocked GEMM for gfx950 through the public API only ------------------------------
+        // What a kernel written against the fragment API gets when it is laid out for this device rather than
+        // after perf_hgemm: 256 x 256 macro tile, eight waves (4 x 2) of 64 x 128, 16 x 16 x 32 blocks (the
+        // full-rate f16 instruction), K stages of 64 in two LDS buffers with one barrier per stage, the next stage's
+        // slabs fetched into registers with cooperative loads while this stage is multiplied.  LDS slabs are
+        // K-contiguous rows (row-major A, transposed B) of 64 + 8 halves: the 16 rows a quarter-wave reads at one
+        // K offset are 144 bytes apart, sixteen distinct 16-byte slots, and fragments are always held in the
+        // order the matrix instruction takes them, so every LDS access is a conflict-free 16-byte one whatever
+        // the layouts in global memory (applyDataLayout / applyTranspose are re-typings).  Without the padding
+        // the same kernel runs at half the speed.
+        namespace tiled
+        {
+            constexpr uint32_t BM = 16, BN = 16, BK = 32;
+            constexpr uint32_t BlocksX = 4, BlocksY = 8;
+            constexpr uint32_t WavesX = 4, WavesY = 2;
+            constexpr uint32_t WaveTileX = BlocksX * BM, WaveTileY = BlocksY * BN;
+            constexpr uint32_t MacroX = WavesX * WaveTileX, MacroY = WavesY * WaveTileY;
+            constexpr uint32_t WaveCount = WavesX * WavesY;
+            constexpr uint32_t StageK = 64, Steps = StageK / BK;
+            constexpr uint32_t LdsLd   = StageK + 8; // halves per LDS row
+            constexpr uint32_t BufElts = (MacroX + MacroY) * LdsLd;
+            constexpr uint32_t LdsBytes = 2u * BufElts * sizeof(float16_t);
+
+            template <typename LA, typename LB>
+            __global__ void __launch_bounds__(64 * WaveCount) tiledGemmKernel(uint32_t         m,
+                                                                             uint32_t         n,
+                                                                             uint32_t         k,
+                                                                             const float16_t* a,
+                                                                             const float16_t* b,
+                                                                             const float*     c,
+                                                                             float*           d,
+                                                                             uint32_t         lda,
+                                                                             uint32_t         ldb,
+                                                                             uint32_t         ldc,
+                                                                             uint32_t         ldd,
+                                                                             float            alpha,
+                                                                             float            beta)
+            {
+                using FragA    = fragment<matrix_a, BM, BN, BK, float16_t, LA>;
+                using FragB    = fragment<matrix_b, BM, BN, BK, float16_t, LB>;
+                using FragC    = fragment<accumulator, BM, BN, BK, float, row_major>;
+                using FragAcc  = fragment<accumulator, BM, BN, BK, float>;
+                using LdsFragA = ApplyDataLayout_t<FragA, row_major>;
+                using LdsFragB = ApplyDataLayout_t<ApplyTranspose_t<FragB>, row_major>;
+                using SlabA    = fragment<matrix_a, MacroX, BN, StageK, float16_t, LA>;
+                using SlabB    = fragment<matrix_b, BM, MacroY, StageK, float16_t, LB>;
+                using MapA     = GetDataLayout_t<SlabA>;
+                using MapB     = GetDataLayout_t<SlabB>;
+
+                extern __shared__ __attribute__((aligned(16))) char ldsRaw[];
+                float16_t* lds = reinterpret_cast<float16_t*>(ldsRaw);
+
+                const uint32_t waveIndex = threadIdx.x / Constants::AMDGCN_WAVE_SIZE;
+                const uint32_t wx = waveIndex / WavesY, wy = waveIndex % WavesY;
+                const uint32_t row0 = blockIdx.x * MacroX, col0 = blockIdx.y * MacroY;
+
+                const float16_t* aPtr  = a + MapA::fromMatrixCoord(make_coord2d(row0, 0u), lda);
+                const float16_t* bPtr  = b + MapB::fromMatrixCoord(make_coord2d(0u, col0), ldb);
+                const uint32_t   stepA = MapA::fromMatrixCoord(make_coord2d(0u, StageK), lda);
+                const uint32_t   stepB = MapB::fromMatrixCoord(make_coord2d(StageK, 0u), ldb);
+
+                FragAcc acc[BlocksX][BlocksY];
+                for(uint32_t i = 0; i < BlocksX; ++i)
+                    for(uint32_t j = 0; j < BlocksY; ++j)
+                        fill_fragment(acc[i][j], 0.0f);
+
+                SlabA grA;
+                SlabB grB;
+                load_matrix_coop_sync<WaveCount>(grA, aPtr, lda, waveIndex);
+                load_matrix_coop_sync<WaveCount>(grB, bPtr, ldb, waveIndex);
+                store_matrix_coop_sync<WaveCount>(lds, applyDataLayout<row_major, WaveCount>(grA), LdsLd, waveIndex);
+                store_matrix_coop_sync<WaveCount>(lds + MacroX * LdsLd, applyDataLayout<row_major, WaveCount>(applyTranspose(grB)), LdsLd,
+                                                  waveIndex);
+                synchronize_workgroup();
+
+                uint32_t cur = 0;
+                for(uint32_t kk = 0; kk < k; kk += StageK)
+                {
+                    const bool more = kk + StageK < k;
+                    if(more)
+                    {
+                        aPtr += stepA;
+                        bPtr += stepB;
+                        load_matrix_coop_sync<WaveCount>(grA, aPtr, lda, waveIndex);
+                        load_matrix_coop_sync<WaveCount>(grB, bPtr, ldb, waveIndex);
+                    }
+                    const float16_t* ldsA = lds + cur * BufElts + wx * WaveTileX * LdsLd;
+                    const float16_t* ldsB = lds + cur * BufElts + (MacroX + wy * WaveTileY) * LdsLd;
+#pragma unroll
+                    for(uint32_t s = 0; s < Steps; ++s)
+                    {
+                        FragA fa[BlocksX];
+                        FragB fb[BlocksY];
+#pragma unroll
+                        for(uint32_t i = 0; i < BlocksX; ++i)
+                        {
+                            LdsFragA t;
+                            load_matrix_sync(t, ldsA + i * BM * LdsLd + s * BK, LdsLd);
+                            fa[i] = applyDataLayout<LA>(t);
+                        }
+#pragma unroll
+                        for(uint32_t j = 0; j < BlocksY; ++j)
+                        {
+                            LdsFragB t;
+                            load_matrix_sync(t, ldsB + j * BN * LdsLd + s * BK, LdsLd);
+                            fb[j] = applyDataLayout<LB>(applyTranspose(t));
+                        }
+#pragma unroll
+                        for(uint32_t i = 0; i < BlocksX; ++i)
+#pragma unroll
+                            for(uint32_t j = 0; j < BlocksY; ++j)
+                                mma_sync(acc[i][j], fa[i], fb[j], acc[i][j]);
+                    }
+                    if(more)
+                    {
+                        float16_t* nxt = lds + (cur ^ 1u) * BufElts;
+                        store_matrix_coop_sync<WaveCount>(nxt, applyDataLayout<row_major, WaveCount>(grA), LdsLd, waveIndex);
+                        store_matrix_coop_sync<WaveCount>(nxt + MacroX * LdsLd, applyDataLayout<row_major, WaveCount>(applyTranspose(grB)),
+                                                          LdsLd, waveIndex);
+                    }
+                    synchronize_workgroup();
+                    cur ^= 1u;
+                }
+
+                for(uint32_t i = 0; i < BlocksX; ++i)
+                    for(uint32_t j = 0; j < BlocksY; ++j)
+                    {
+                        const size_t r = row0 + wx * WaveTileX + i * BM, cc = col0 + wy * WaveTileY + j * BN;
+                        FragC        fc;
+                        load_matrix_sync(fc, c + r * ldc + cc, ldc);
+                        for(uint32_t e = 0; e < fc.num_elements; ++e)
+                            fc.x[e] = alpha * acc[i][j].x[e] + beta * fc.x[e];
+                        store_matrix_sync(d + r * ldd + cc, fc, ldd);
+                    }
+            }
+
+            template <typename LA, typename LB>
+            int launch(uint32_t m, uint32_t n, uint32_t k, const void* a, const void* b, const float* c, float* d, float alpha, float beta,
+                       hipStream_t stream)
+            {
+                auto kernel = tiledGemmKernel<LA, LB>;
+                if(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       static_cast<int>(LdsBytes))
+                   != hipSuccess)
+                    return ROCWMMA_AMD_LAUNCH_FAILED;
+                const uint32_t lda = std::is_same<LA, row_major>::value ? k : m;
+                const uint32_t ldb = std::is_same<LB, row_major>::value ? n : k;
+                hipLaunchKernelGGL(kernel, dim3(m / MacroX, n / MacroY), dim3(64 * WaveCount), LdsBytes, stream, m, n, k,
+                                   static_cast<const float16_t*>(a), static_cast<const float16_t*>(b), c, d, lda, ldb, n, n, alpha, beta);
+                return launchStatus();
+            }
+        } // namespace tiled
     } // namespace
+
+    int selftestTiledGemm(int layoutA, int layoutB, uint32_t m, uint32_t n, uint32_t k, const void* a, const void* b, const float* c,
+                          float* d, float alpha, float beta, hipStream_t stream)
+    {
+        if(m == 0u || n == 0u || k == 0u || m % tiled::MacroX != 0u || n % tiled::MacroY != 0u || k % tiled::StageK != 0u)
+            return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+        const bool ar = layoutA == ROCWMMA_AMD_ROW_MAJOR, br = layoutB == ROCWMMA_AMD_ROW_MAJOR;
+        if(ar && br)
+            return tiled::launch<row_major, row_major>(m, n, k, a, b, c, d, alpha, beta, stream);
+        if(ar && !br)
+            return tiled::launch<row_major, col_major>(m, n, k, a, b, c, d, alpha, beta, stream);
+        if(!ar && br)
+            return tiled::launch<col_major, row_major>(m, n, k, a, b, c, d, alpha, beta, stream);
+        return tiled::launch<col_major, col_major>(m, n, k, a, b, c, d, alpha, beta, stream);
+    }
 
     int selftestRoundtrip(int context, int dtype, int layout, int block, int blockk, int coop, uint32_t rows, uint32_t cols,
                           const void* in, void* out, uint32_t ld, hipStream_t stream)

@@ -101,3 +101,33 @@ def test_cooperative_flow_exact_on_integer_pattern(la, lb):
     want = orc.gemm(orc.F16, orc.F32, la, lb, RM, RM, m, n, k, a, b, c, 2.0, 2.0)
     same = np.array_equal(d.cpu().numpy(), want)
     assert same
+
+
+@pytest.mark.parametrize("la", [RM, CM])
+@pytest.mark.parametrize("lb", [RM, CM])
+def test_blocked_gemm_through_the_public_api_only(la, lb):
+    """The blocked GEMM laid out for gfx950 and written against the fragment API alone (cooperative loads and stores,
+    applyDataLayout, applyTranspose, padded LDS slabs, mma_sync on 16 x 16 x 32 blocks): against the oracle, and bit
+    for bit on the reference's integer fill; a K of three stages walks both LDS buffers and the tail."""
+    import torch
+
+    from util import exact_int_bits
+
+    m, n, k = 512, 256, 192
+    a = uniform_bits(21, orc.F16, m * k)
+    b = uniform_bits(22, orc.F16, k * n)
+    c = np.random.default_rng(23).uniform(-1, 1, m * n).astype(np.float32)
+    d = torch.full((m * n,), float("nan"), device="cuda")
+    rw.selftest_tiled_gemm(la, lb, m, n, k, to_device(a), to_device(b), to_device(c), d, 2.0, -1.5)
+    torch.cuda.synchronize()
+    want = orc.gemm(orc.F16, orc.F32, la, lb, RM, RM, m, n, k, a, b, c, 2.0, -1.5)
+    err, inf, nan = orc.compare_equal(orc.F32, d.cpu().numpy(), orc.F32, want)
+    assert not inf and not nan and err <= 1e-3, err
+    a, b, c = exact_int_bits(orc.F16, m, k, la), exact_int_bits(orc.F16, k, n, lb), exact_int_bits(orc.F32, m, n, RM)
+    d.fill_(float("nan"))
+    rw.selftest_tiled_gemm(la, lb, m, n, k, to_device(a), to_device(b), to_device(c), d, 2.0, 2.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(d.cpu().numpy(), orc.gemm(orc.F16, orc.F32, la, lb, RM, RM, m, n, k, a, b, c, 2.0, 2.0))
+    with pytest.raises(rw.RocwmmaError) as e:  # whole 256 x 256 tiles and 64-wide stages only
+        rw.selftest_tiled_gemm(la, lb, 384, n, k, to_device(a), to_device(b), to_device(c), d, 1.0, 0.0)
+    assert e.value.status == 3
