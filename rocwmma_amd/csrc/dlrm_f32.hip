@@ -7,16 +7,18 @@
 // plan -- one wave owns a sample, no m x m scratch in global memory, one launch for backward -- written for
 // parity rather than for the last byte per second:
 //
-//   * a wave copies its sample's m x K features into LDS rows of K + 4 floats (16-byte global loads; rows from m
-//     to the next multiple of 32 are zeros, so no lane ever reads another sample or past the end of the input);
+//   * operands come straight from global memory (a sample is read by one wave only, so there is nothing to share
+//     through LDS, and without LDS five waves per SIMD are resident); rows and contraction indices from m on are
+//     never read: their lanes multiply zeros, so nothing of a neighbouring sample can leak (0 * Inf);
 //   * the products run on v_mfma_f32_32x32x2_f32 through the fragment API.  Forward: block (I, J), J <= I, of
-//     Z = F F^T from the 32-row tiles I and J; a lane reads 16 bytes of K per row and LDS instruction and feeds
-//     four instructions from them (the order in which K is contracted is free as long as both multiplicands
+//     Z = F F^T from the 32-row tiles I and J; a lane loads 16 bytes of K of its row at a time and feeds four
+//     instructions from them (the order in which K is contracted is free as long as both multiplicands
 //     agree: instruction t of a group contracts k = 8 g + t and 8 g + 4 + t).  Backward: row tile I of the
 //     gradient is the sum over contraction tiles J of G_IJ F_J, G rebuilt from the packed triangle of the
-//     upstream gradient (read straight from global memory), 32 columns at a time, stored from the accumulators
-//     as 16-byte pieces;
-//   * nothing is shared between the waves of a workgroup: no barrier.
+//     upstream gradient, 32 columns at a time (32 lanes read 128 contiguous bytes of a feature row), stored
+//     from the accumulators as 16-byte pieces;
+//   * nothing is shared between the waves of a workgroup: no barrier; LDS only to put a sample's forward output
+//     row together before it is written out.
 #include "common.hpp"
 #include <rocwmma/rocwmma_transforms.hpp>
 
@@ -29,28 +31,6 @@ namespace rocwmma_amd
         typedef float f32x4_t __attribute__((ext_vector_type(4), may_alias));
 
         constexpr uint32_t kMaxM32   = 128;
-        constexpr uint32_t kMaxTiles = kMaxM32 / 32u;
-        constexpr uint32_t kRowPad   = 4; // floats: 16 consecutive rows at one column offset fall into 16 distinct 16-byte slots
-        constexpr uint32_t kLdsBytes = 160u * 1024u;
-
-        template <uint32_t K>
-        ROCWMMA_DEVICE inline void stageFeatures(float* ldsF, const float* src, uint32_t m, uint32_t rowsPad, uint32_t lane)
-        {
-            constexpr uint32_t pitch  = K + kRowPad;
-            constexpr uint32_t perRow = K / 4u;
-            for(uint32_t i = lane; i < rowsPad * perRow; i += 64u)
-            {
-                const uint32_t r = i / perRow, c4 = i % perRow;
-                f32x4_t        v = {0.0f, 0.0f, 0.0f, 0.0f};
-                if(r < m)
-                    v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(src + static_cast<size_t>(r) * K) + c4);
-                *reinterpret_cast<f32x4_t*>(ldsF + r * pitch + 4u * c4) = v;
-            }
-            // (the wave's own LDS writes are visible to its later LDS reads: the LDS serves a wave's accesses in order)
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        }
 
         template <uint32_t K, uint32_t Samples>
         __global__ void __launch_bounds__(64 * Samples)
@@ -60,25 +40,23 @@ namespace rocwmma_amd
             using FragAcc = fragment<accumulator, 32, 32, 2, float32_t>;
             using AccMap  = detail::AccMap<32, 32, 32>;
             static_assert(FragA::num_elements == 1u && FragAcc::num_elements == 16u, "one float per lane and instruction");
-            constexpr uint32_t pitch = K + kRowPad;
 
-            extern __shared__ __attribute__((aligned(16))) float ldsAll[];
-            const uint32_t lane    = threadIdx.x & 63u;
-            const uint32_t wave    = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-            const uint32_t sample  = blockIdx.x * Samples + wave;
-            const uint32_t tiles   = (m + 31u) / 32u;
-            const uint32_t rowsPad = tiles * 32u;
+            const uint32_t lane   = threadIdx.x & 63u;
+            const uint32_t wave   = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            const uint32_t sample = blockIdx.x * Samples + wave;
+            const uint32_t tiles  = (m + 31u) / 32u;
             if(sample >= batch)
                 return; // (no workgroup barrier anywhere below)
-            float*         ldsF  = ldsAll + wave * rowsPad * pitch;
             const uint32_t width = K + (m * (m - 1u)) / 2u;
-            float*         out   = output + static_cast<size_t>(sample) * width;
-
-            stageFeatures<K>(ldsF, input + static_cast<size_t>(sample) * m * K, m, rowsPad, lane);
+            const float*   feat  = input + static_cast<size_t>(sample) * m * K;
+            // the sample's output row is put together in LDS (the triangle leaves the accumulators as single floats
+            // all over the row) and written out in whole-wave pieces of 256 contiguous bytes
+            extern __shared__ __attribute__((aligned(16))) float ldsOut[];
+            float* out = ldsOut + wave * width;
 
             // bottom-MLP row: the sample's first feature row
             for(uint32_t e = lane; e < K; e += 64u)
-                out[e] = ldsF[e];
+                out[e] = feat[e];
 
             const uint32_t row = lane & 31u, half = lane >> 5;
 #pragma unroll 1
@@ -86,23 +64,50 @@ namespace rocwmma_amd
 #pragma unroll 1
                 for(uint32_t J = 0; J <= I; ++J)
                 {
-                    const float* fI = ldsF + (I * 32u + row) * pitch + 4u * half;
-                    const float* fJ = ldsF + (J * 32u + row) * pitch + 4u * half;
-                    FragAcc      acc;
+                    // (rows from m on do not exist: their lanes multiply zeros and read nothing)
+                    const bool     liveI = I * 32u + row < m, liveJ = J * 32u + row < m;
+                    const f32x4_t* fI    = reinterpret_cast<const f32x4_t*>(feat + static_cast<size_t>(I * 32u + row) * K) + half;
+                    const f32x4_t* fJ    = reinterpret_cast<const f32x4_t*>(feat + static_cast<size_t>(J * 32u + row) * K) + half;
+                    FragAcc        acc;
                     fill_fragment(acc, 0.0f);
-#pragma unroll 4
-                    for(uint32_t g = 0; g < K / 8u; ++g)
+                    constexpr uint32_t Groups = K / 8u, Batch = Groups < 8u ? Groups : 8u; // loads in flight per operand
+#pragma unroll 1
+                    for(uint32_t g0 = 0; g0 < Groups; g0 += Batch)
                     {
-                        const f32x4_t vi = *reinterpret_cast<const f32x4_t*>(fI + 8u * g);
-                        const f32x4_t vj = *reinterpret_cast<const f32x4_t*>(fJ + 8u * g);
+                        f32x4_t vi[Batch], vj[Batch];
 #pragma unroll
-                        for(uint32_t t = 0; t < 4u; ++t)
+                        for(uint32_t g = 0; g < Batch; ++g)
                         {
-                            FragA a, b;
-                            a.x[0] = vi[t];
-                            b.x[0] = vj[t];
-                            mma_sync(acc, a, applyTranspose(b), acc);
+                            vi[g] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                            if(liveI)
+                                vi[g] = fI[2u * (g0 + g)];
                         }
+                        if(I != J) // (wave uniform)
+                        {
+#pragma unroll
+                            for(uint32_t g = 0; g < Batch; ++g)
+                            {
+                                vj[g] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                                if(liveJ)
+                                    vj[g] = fJ[2u * (g0 + g)];
+                            }
+                        }
+                        else
+                        {
+#pragma unroll
+                            for(uint32_t g = 0; g < Batch; ++g)
+                                vj[g] = vi[g];
+                        }
+#pragma unroll
+                        for(uint32_t g = 0; g < Batch; ++g)
+#pragma unroll
+                            for(uint32_t t = 0; t < 4u; ++t)
+                            {
+                                FragA a, b;
+                                a.x[0] = vi[g][t];
+                                b.x[0] = vj[g][t];
+                                mma_sync(acc, a, applyTranspose(b), acc);
+                            }
                     }
                     // strict lower triangle, row by row
 #pragma unroll
@@ -114,9 +119,18 @@ namespace rocwmma_amd
                             out[K + (Rg * (Rg - 1u)) / 2u + Cg] = acc.x[e];
                     }
                 }
+            // (the wave's own LDS writes, read back by other lanes of the same wave: the LDS serves a wave's accesses in order)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            float* dst = output + static_cast<size_t>(sample) * width;
+            for(uint32_t e = lane; e < width; e += 64u)
+                dst[e] = out[e];
         }
 
-        template <uint32_t K, uint32_t Samples>
+        // MaxTiles: contraction tiles of 32 the kernel is built for (1, 2 or 4: the G values of a row tile against
+        // every contraction tile are held in registers, 16 per tile)
+        template <uint32_t K, uint32_t Samples, uint32_t MaxTiles>
         __global__ void __launch_bounds__(64 * Samples) dlrmBwdF32Kernel(const float* __restrict__ input,
                                                                             const float* __restrict__ upstream,
                                                                             float* __restrict__ grad,
@@ -129,23 +143,18 @@ namespace rocwmma_amd
             using FragAcc = fragment<accumulator, 32, 32, 2, float32_t>;
             using AccMap  = detail::AccMap<32, 32, 32>;
             static_assert(FragG::num_elements == 1u && FragF::num_elements == 1u, "one float per lane and instruction");
-            constexpr uint32_t pitch   = K + kRowPad;
             constexpr uint32_t NBlocks = K / 32u;
 
-            extern __shared__ __attribute__((aligned(16))) float ldsAll[];
-            const uint32_t lane    = threadIdx.x & 63u;
-            const uint32_t wave    = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-            const uint32_t sample  = blockIdx.x * Samples + wave;
-            const uint32_t tiles   = (m + 31u) / 32u;
-            const uint32_t rowsPad = tiles * 32u;
+            const uint32_t lane   = threadIdx.x & 63u;
+            const uint32_t wave   = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            const uint32_t sample = blockIdx.x * Samples + wave;
+            const uint32_t tiles  = (m + 31u) / 32u;
             if(sample >= batch)
                 return;
-            float*         ldsF  = ldsAll + wave * rowsPad * pitch;
             const uint32_t width = K + (m * (m - 1u)) / 2u;
+            const float*   feat  = input + static_cast<size_t>(sample) * m * K;
             const float*   up    = upstream + static_cast<size_t>(sample) * width;
             float*         dst   = grad + static_cast<size_t>(sample) * m * K;
-
-            stageFeatures<K>(ldsF, input + static_cast<size_t>(sample) * m * K, m, rowsPad, lane);
 
             // bottom-MLP gradient = the first K entries of the upstream row
             for(uint32_t e = lane; e < K; e += 64u)
@@ -157,13 +166,12 @@ namespace rocwmma_amd
             {
                 // G(Rg, c) for this lane's row and its contraction indices c = J * 32 + 2 s + half: below the
                 // diagonal the row's entries are consecutive in the packed triangle (tri(Rg) + c), above it entry
-                // (c, Rg) sits at tri(c) + Rg; zero on the diagonal and beyond m.  (Rows and contraction indices
-                // >= m meet zeros on both sides: the staged feature rows there are zeros.)
+                // (c, Rg) sits at tri(c) + Rg; zero on the diagonal and beyond m.
                 const uint32_t Rg    = I * 32u + row;
                 const uint32_t below = K + (Rg * (Rg - 1u)) / 2u;
-                float          g[kMaxTiles][16];
+                float          g[MaxTiles][16];
 #pragma unroll
-                for(uint32_t J = 0; J < kMaxTiles; ++J)
+                for(uint32_t J = 0; J < MaxTiles; ++J)
 #pragma unroll
                     for(uint32_t s = 0; s < 16u; ++s)
                     {
@@ -177,18 +185,25 @@ namespace rocwmma_amd
                     FragAcc acc;
                     fill_fragment(acc, 0.0f);
 #pragma unroll
-                    for(uint32_t J = 0; J < kMaxTiles; ++J)
+                    for(uint32_t J = 0; J < MaxTiles; ++J)
                     {
                         if(J < tiles) // (wave uniform)
                         {
-                            const float* f = ldsF + (J * 32u + half) * pitch + nb * 32u + row;
+                            // F(c, column) for the lane's contraction indices c = J * 32 + 2 s + half and its column:
+                            // 32 lanes read 128 contiguous bytes of a row; rows from m on do not exist (zeros, not
+                            // another sample's values: 0 * Inf would leak)
+                            const float* f = feat + static_cast<size_t>(J * 32u + half) * K + nb * 32u + row;
+                            float        fv[16];
+#pragma unroll
+                            for(uint32_t s = 0; s < 16u; ++s)
+                                fv[s] = J * 32u + 2u * s + half < m ? f[static_cast<size_t>(2u * s) * K] : 0.0f;
 #pragma unroll
                             for(uint32_t s = 0; s < 16u; ++s)
                             {
                                 FragG a;
                                 FragF b;
                                 a.x[0] = g[J][s];
-                                b.x[0] = f[2u * s * pitch];
+                                b.x[0] = fv[s];
                                 mma_sync(acc, a, b, acc);
                             }
                         }
@@ -208,60 +223,35 @@ namespace rocwmma_amd
             }
         }
 
-        template <typename Kernel, typename... Args>
-        int launchWithLds(Kernel kernel, uint32_t grid, uint32_t threads, uint32_t lds, hipStream_t stream, Args... args)
+        // Four samples (waves) per workgroup; nothing is shared between them.
+        constexpr uint32_t kSamples = 4;
+
+        template <uint32_t K>
+        int launchFwd32(const float* input, float* output, uint32_t m, uint32_t batch, hipStream_t stream)
         {
-            if(lds > kLdsBytes)
-                return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
+            const uint32_t lds    = kSamples * (K + (m * (m - 1u)) / 2u) * static_cast<uint32_t>(sizeof(float));
+            auto           kernel = dlrmFwdF32Kernel<K, kSamples>;
             if(lds > 65536u
                && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(lds))
                       != hipSuccess)
                 return ROCWMMA_AMD_LAUNCH_FAILED;
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, args...);
+            hipLaunchKernelGGL(kernel, dim3((batch + kSamples - 1u) / kSamples), dim3(64u * kSamples), lds, stream, input, output, m, batch);
             return launchStatus();
-        }
-
-        // Samples (waves) per workgroup: as many of 4, 2, 1 as keep a workgroup's feature tiles within 64 KiB
-        // (several workgroups per compute unit), one where a single sample needs more.
-        template <uint32_t K>
-        uint32_t samplesFor(uint32_t m)
-        {
-            const uint32_t perSample = ((m + 31u) / 32u) * 32u * (K + kRowPad) * 4u;
-            return 4u * perSample <= 65536u ? 4u : (2u * perSample <= 65536u ? 2u : 1u);
-        }
-
-        template <uint32_t K>
-        int launchFwd32(const float* input, float* output, uint32_t m, uint32_t batch, hipStream_t stream)
-        {
-            const uint32_t perSample = ((m + 31u) / 32u) * 32u * (K + kRowPad) * 4u;
-            switch(samplesFor<K>(m))
-            {
-            case 4:
-                return launchWithLds(dlrmFwdF32Kernel<K, 4>, (batch + 3u) / 4u, 256u, 4u * perSample, stream, input, output, m, batch);
-            case 2:
-                return launchWithLds(dlrmFwdF32Kernel<K, 2>, (batch + 1u) / 2u, 128u, 2u * perSample, stream, input, output, m, batch);
-            default:
-                return launchWithLds(dlrmFwdF32Kernel<K, 1>, batch, 64u, perSample, stream, input, output, m, batch);
-            }
         }
 
         template <uint32_t K>
         int launchBwd32(const float* input, const float* upstream, float* grad, float* mlpGrad, uint32_t m, uint32_t batch,
                         hipStream_t stream)
         {
-            const uint32_t perSample = ((m + 31u) / 32u) * 32u * (K + kRowPad) * 4u;
-            switch(samplesFor<K>(m))
-            {
-            case 4:
-                return launchWithLds(dlrmBwdF32Kernel<K, 4>, (batch + 3u) / 4u, 256u, 4u * perSample, stream, input, upstream, grad,
-                                     mlpGrad, m, batch);
-            case 2:
-                return launchWithLds(dlrmBwdF32Kernel<K, 2>, (batch + 1u) / 2u, 128u, 2u * perSample, stream, input, upstream, grad,
-                                     mlpGrad, m, batch);
-            default:
-                return launchWithLds(dlrmBwdF32Kernel<K, 1>, batch, 64u, perSample, stream, input, upstream, grad, mlpGrad, m, batch);
-            }
+            const dim3 grid((batch + kSamples - 1u) / kSamples), block(64u * kSamples);
+            if(m <= 32u)
+                hipLaunchKernelGGL((dlrmBwdF32Kernel<K, kSamples, 1>), grid, block, 0, stream, input, upstream, grad, mlpGrad, m, batch);
+            else if(m <= 64u)
+                hipLaunchKernelGGL((dlrmBwdF32Kernel<K, kSamples, 2>), grid, block, 0, stream, input, upstream, grad, mlpGrad, m, batch);
+            else
+                hipLaunchKernelGGL((dlrmBwdF32Kernel<K, kSamples, 4>), grid, block, 0, stream, input, upstream, grad, mlpGrad, m, batch);
+            return launchStatus();
         }
     } // namespace
 
