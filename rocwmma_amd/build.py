@@ -15,7 +15,7 @@ OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "librocwmma_amd.so")
 AUX_LIB_PATH = os.path.join(HERE, "librocwmma_amd_aux.so")
 
-SOURCES = ["api.hip", "gemm_wave_tile.hip", "gemm_blocked.hip", "gemm_streamk.hip", "gemm_skinny.hip", "gemm_mx.hip", "gemm_fused.hip", "gemv.hip", "dlrm.hip", "dlrm_f32.hip"]
+SOURCES = ["api.hip", "gemm_wave_tile.hip", "gemm_blocked.hip", "gemm_streamk.hip", "gemm_skinny.hip", "gemm_mx.hip", "gemm_fused.hip", "gemv.hip", "dlrm.hip", "dlrm_f32.hip", "dlrm_general.hip"]
 # test and benchmark support: fragment-API self-test kernels and measurement probes
 AUX_SOURCES = ["aux_api.hip", "selftest.hip", "mfma_ceiling.hip", "mfma_streams.hip", "stream_ceiling.hip"]
 

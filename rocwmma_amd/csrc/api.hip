@@ -13,6 +13,9 @@ namespace rocwmma_amd
                    float* y, uint32_t ldy, float alpha, float beta, hipStream_t stream);
     int launchDlrmFwd(const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, hipStream_t stream);
     int launchDlrmFwdF32(const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, hipStream_t stream);
+    int launchDlrmFwdGeneral(int dtype, const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, hipStream_t stream);
+    int launchDlrmBwdGeneral(int dtype, const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t k,
+                             uint32_t batch, hipStream_t stream);
     int launchDlrmBwdF32(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t k, uint32_t batch,
                          hipStream_t stream);
     int launchDlrmBwd(const void* input, const void* upstream, void* grad, void* mlpGrad, uint32_t m, uint32_t k,
@@ -567,11 +570,18 @@ int rocwmma_amd_gemv(uint32_t    m,
     return launchGemv(m, k, ncols, a, lda, x, ldx, y, ldy, alpha, beta, asStream(stream));
 }
 
-static int checkDlrm(uint32_t m, uint32_t k, uint32_t batch)
+// The one-wave-per-sample kernels take these shapes; the tiled kernels of dlrm_general.hip take the others.
+static bool dlrmSampleFitsAWave(uint32_t m, uint32_t k)
 {
-    if(m == 0u || batch == 0u)
+    return m <= 128u && (k == 32u || k == 64u || k == 128u || k == 256u);
+}
+
+static int checkDlrm(int dtype, uint32_t m, uint32_t k, uint32_t batch)
+{
+    if(m == 0u || k == 0u || batch == 0u)
         return ROCWMMA_AMD_INVALID_ARGUMENT;
-    if(m > 128u || (k != 32u && k != 64u && k != 128u && k != 256u))
+    // the tiled kernels read rows in 16-byte pieces
+    if(!dlrmSampleFitsAWave(m, k) && (m > 32768u || k % (dtype == ROCWMMA_AMD_F16 ? 8u : 4u) != 0u))
         return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
     return ROCWMMA_AMD_OK;
 }
@@ -580,14 +590,20 @@ int rocwmma_amd_dlrm_fwd(const void* input, void* output, uint32_t m, uint32_t k
 {
     if(!input || !output)
         return ROCWMMA_AMD_INVALID_ARGUMENT;
-    int rc = checkDlrm(m, k, batch);
+    int rc = checkDlrm(ROCWMMA_AMD_F16, m, k, batch);
     if(rc != ROCWMMA_AMD_OK)
         return rc;
     if(!aligned16(input) || !aligned16(output))
         return ROCWMMA_AMD_BAD_ALIGNMENT;
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
-    return launchDlrmFwd(input, output, m, k, batch, asStream(stream));
+    if(dlrmSampleFitsAWave(m, k))
+    {
+        rc = launchDlrmFwd(input, output, m, k, batch, asStream(stream));
+        if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE) // (a sample larger than the LDS: tiles)
+            return rc;
+    }
+    return launchDlrmFwdGeneral(ROCWMMA_AMD_F16, input, output, m, k, batch, asStream(stream));
 }
 
 int rocwmma_amd_dlrm_bwd(const void* input,
@@ -601,14 +617,20 @@ int rocwmma_amd_dlrm_bwd(const void* input,
 {
     if(!input || !upstream_grad || !grad || !bottom_mlp_grad)
         return ROCWMMA_AMD_INVALID_ARGUMENT;
-    int rc = checkDlrm(m, k, batch);
+    int rc = checkDlrm(ROCWMMA_AMD_F16, m, k, batch);
     if(rc != ROCWMMA_AMD_OK)
         return rc;
     if(!aligned16(input) || !aligned16(upstream_grad) || !aligned16(grad) || !aligned16(bottom_mlp_grad))
         return ROCWMMA_AMD_BAD_ALIGNMENT;
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
-    return launchDlrmBwd(input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
+    if(dlrmSampleFitsAWave(m, k))
+    {
+        rc = launchDlrmBwd(input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
+        if(rc != ROCWMMA_AMD_UNSUPPORTED_SHAPE)
+            return rc;
+    }
+    return launchDlrmBwdGeneral(ROCWMMA_AMD_F16, input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
 }
 
 int rocwmma_amd_dlrm_fwd_ex(int dtype, const void* input, void* output, uint32_t m, uint32_t k, uint32_t batch, void* stream)
@@ -619,14 +641,16 @@ int rocwmma_amd_dlrm_fwd_ex(int dtype, const void* input, void* output, uint32_t
         return ROCWMMA_AMD_UNSUPPORTED_TYPE;
     if(!input || !output)
         return ROCWMMA_AMD_INVALID_ARGUMENT;
-    int rc = checkDlrm(m, k, batch);
+    int rc = checkDlrm(ROCWMMA_AMD_F32, m, k, batch);
     if(rc != ROCWMMA_AMD_OK)
         return rc;
     if(!aligned16(input) || !aligned16(output))
         return ROCWMMA_AMD_BAD_ALIGNMENT;
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
-    return launchDlrmFwdF32(input, output, m, k, batch, asStream(stream));
+    if(dlrmSampleFitsAWave(m, k))
+        return launchDlrmFwdF32(input, output, m, k, batch, asStream(stream));
+    return launchDlrmFwdGeneral(ROCWMMA_AMD_F32, input, output, m, k, batch, asStream(stream));
 }
 
 int rocwmma_amd_dlrm_bwd_ex(int         dtype,
@@ -645,14 +669,16 @@ int rocwmma_amd_dlrm_bwd_ex(int         dtype,
         return ROCWMMA_AMD_UNSUPPORTED_TYPE;
     if(!input || !upstream_grad || !grad || !bottom_mlp_grad)
         return ROCWMMA_AMD_INVALID_ARGUMENT;
-    int rc = checkDlrm(m, k, batch);
+    int rc = checkDlrm(ROCWMMA_AMD_F32, m, k, batch);
     if(rc != ROCWMMA_AMD_OK)
         return rc;
     if(!aligned16(input) || !aligned16(upstream_grad) || !aligned16(grad) || !aligned16(bottom_mlp_grad))
         return ROCWMMA_AMD_BAD_ALIGNMENT;
     if(!isGfx950Current())
         return ROCWMMA_AMD_NO_DEVICE;
-    return launchDlrmBwdF32(input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
+    if(dlrmSampleFitsAWave(m, k))
+        return launchDlrmBwdF32(input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
+    return launchDlrmBwdGeneral(ROCWMMA_AMD_F32, input, upstream_grad, grad, bottom_mlp_grad, m, k, batch, asStream(stream));
 }
 
 } // extern "C"

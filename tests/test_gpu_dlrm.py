@@ -301,3 +301,106 @@ def test_typed_entry_points_take_f16_and_reject_other_types():
     with pytest.raises(rw.RocwmmaError) as e:
         rw.dlrm_fwd(to_device(inp), out, m, k, b, rw.BF16)
     assert e.value.status == 2  # ROCWMMA_AMD_UNSUPPORTED_TYPE
+
+
+# ---------------------------------------------------------------- samples that do not fit one wave (tiles of 128 x 128)
+# More than 128 feature rows or a feature width other than 32 / 64 / 128 / 256, up to the reference's largest test
+# size (m, k) = (1024, 1024) (test/dlrm/test/dlrm_test_params.hpp:51-68).
+def exact_fwd_mm(inp, m, k):
+    F = inp.astype(np.float64)
+    Z = F @ F.transpose(0, 2, 1)
+    il, jl = np.tril_indices(m, -1)
+    return np.concatenate([F[:, 0, :], Z[:, il, jl]], axis=1)
+
+
+GENERAL_SHAPES = [(3, 160, 128), (2, 129, 64), (5, 27, 96), (2, 200, 40), (3, 1, 24), (4, 2, 8), (2, 300, 512),
+                  (2, 130, 1032), (3, 257, 264), (1, 1024, 1024)]
+
+
+@pytest.mark.parametrize("b,m,k", GENERAL_SHAPES)
+def test_samples_larger_than_a_wave_run_as_tiles_of_128(b, m, k):
+    """f16, forward and backward against the oracle: m just above 128 and not a multiple of anything, k that is no power
+    of two (96, 40, 24, 8: whole 16-byte pieces is all that is asked), k that ends inside a step of the K loop
+    (1032, 264), one and two feature rows, more than one tile in every direction, the reference's largest size."""
+    width = k + m * (m - 1) // 2
+    inp = uniform_bits(1100 + m, orc.F16, b * m * k).reshape(b, m, k)
+    up = uniform_bits(1101 + m, orc.F16, b * width).reshape(b, width)
+    got = gpu_fwd(inp, m, k, b)
+    close(got, orc.dlrm_fwd(inp, m, k, b))
+    assert np.array_equal(got[:, :k], inp[:, 0, :])
+    grad, mlp = gpu_bwd(inp, up, m, k, b)
+    wgrad, wmlp = orc.dlrm_bwd(inp, up, m, k, b)
+    close(grad, wgrad)
+    assert np.array_equal(mlp, wmlp)
+
+
+@pytest.mark.parametrize("b,m,k", GENERAL_SHAPES + [(4, 27, 100), (2, 130, 36)])
+def test_float32_samples_larger_than_a_wave(b, m, k):
+    """float32, same shapes plus widths that are multiples of 4 only.  The rounding error of a float32 sum grows with
+    its length: against the CPU loop the bound is 64 eps up to 256 terms and a quarter eps per term beyond."""
+    rng = np.random.default_rng(1200 + m + k)
+    width = k + m * (m - 1) // 2
+    inp = rng.uniform(-1, 1, (b, m, k)).astype(np.float32)
+    up = rng.uniform(-1, 1, (b, width)).astype(np.float32)
+    tol = max(64, max(m, k) // 4) * EPS32
+    got = gpu_fwd32(inp, m, k, b)
+    want = orc.dlrm_fwd(inp, m, k, b, orc.F32)
+    as_accurate_as_the_cpu_loop(got, want, exact_fwd_mm(inp, m, k))
+    close32(got, want, tol)
+    assert np.array_equal(got[:, :k], inp[:, 0, :])
+    grad, mlp = gpu_bwd32(inp, up, m, k, b)
+    wgrad, wmlp = orc.dlrm_bwd(inp, up, m, k, b, orc.F32)
+    as_accurate_as_the_cpu_loop(grad, wgrad, exact_bwd(inp, up, m, k))
+    close32(grad, wgrad, tol)
+    assert np.array_equal(mlp, wmlp)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_reference_largest_size_is_exact_on_small_integers(dtype):
+    """The reference's largest DLRM test case at full size, (m, k, batch) = (1024, 1024, 64) with values -1 / 0 / 1 as its
+    tests fill them (test/dlrm/test/dlrm_test_params.hpp:51-68): every sum is an integer of at most 1024, exact in f16
+    and float32, so forward and backward must equal a float64 matrix product bit for bit (torch on the device is the
+    calculator here; the CPU loops would take ten minutes)."""
+    import torch
+
+    b, m, k = 64, 1024, 1024
+    width = k + m * (m - 1) // 2
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    tdt = torch.float16 if dtype == "f16" else torch.float32
+    code = rw.F16 if dtype == "f16" else rw.F32
+    F = torch.randint(-1, 2, (b, m, k), generator=gen, device="cuda").to(tdt)
+    up = torch.randint(-1, 2, (b, width), generator=gen, device="cuda").to(tdt)
+    out = torch.full((b, width), float("nan"), dtype=tdt, device="cuda")
+    rw.dlrm_fwd(F, out, m, k, b, code)
+    il = torch.tril_indices(m, m, -1, device="cuda")
+    for s0 in range(0, b, 8):  # (eight samples at a time: float64 copies are 8 MiB a sample)
+        F64 = F[s0:s0 + 8].double()
+        Z = torch.bmm(F64, F64.transpose(1, 2))
+        assert torch.equal(out[s0:s0 + 8, k:].double(), Z[:, il[0], il[1]]), s0
+    assert torch.equal(out[:, :k], F[:, 0, :])
+    grad = torch.full((b, m, k), float("nan"), dtype=tdt, device="cuda")
+    mlp = torch.full((b, k), float("nan"), dtype=tdt, device="cuda")
+    rw.dlrm_bwd(F, up, grad, mlp, m, k, b, code)
+    for s0 in range(0, b, 8):
+        G = torch.zeros((8, m, m), dtype=torch.float64, device="cuda")
+        G[:, il[0], il[1]] = up[s0:s0 + 8, k:].double()
+        want = torch.bmm(G + G.transpose(1, 2), F[s0:s0 + 8].double())
+        assert torch.equal(grad[s0:s0 + 8].double(), want), s0
+    assert torch.equal(mlp, up[:, :k])
+
+
+def test_large_samples_are_independent_of_non_finite_neighbours():
+    """Rows beyond a sample's last belong to the next sample: the tiles must not read them (0 * Inf would leak)."""
+    b, m, k = 3, 150, 72
+    inp = uniform_bits(1301, orc.F16, b * m * k).reshape(b, m, k).copy()
+    width = k + m * (m - 1) // 2
+    up = uniform_bits(1302, orc.F16, b * width).reshape(b, width)
+    want_f = orc.dlrm_fwd(inp, m, k, b)
+    want_g, _ = orc.dlrm_bwd(inp, up, m, k, b)
+    poisoned = inp.copy()
+    poisoned[1] = 0x7C00  # +Inf everywhere in the middle sample
+    got_f = gpu_fwd(poisoned, m, k, b)
+    got_g, _ = gpu_bwd(poisoned, up, m, k, b)
+    for s in (0, 2):
+        close(got_f[s], want_f[s])
+        close(got_g[s], want_g[s])

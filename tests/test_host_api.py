@@ -128,9 +128,9 @@ def test_gemv_and_dlrm_argument_validation(lib):
     assert f(64, 64, 1, None, 64, 8192, 64, 12288, 64, 1.0, 0.0, None) == 1
     g = lib.rocwmma_amd_dlrm_fwd
     assert g(None, 4096, 27, 128, 8, None) == 1
-    assert g(4096, 8192, 129, 128, 8, None) == 3
-    assert g(4096, 8192, 27, 100, 8, None) == 3
-    assert g(4096, 8192, 27, 128, 0, None) == 1
+    assert g(4096, 8192, 40000, 128, 8, None) == 3
+    assert g(4096, 8192, 27, 100, 8, None) == 3  # (rows of f16 must be whole 16-byte pieces)
+    assert g(4096, 8192, 27, 128, 0, None) == 1 and g(4096, 8192, 27, 0, 8, None) == 1
     h = lib.rocwmma_amd_dlrm_bwd
     assert h(4096, 8192, 12288, None, 27, 128, 8, None) == 1
     assert h(4096, 8192, 12290, 16384, 27, 128, 8, None) == 4
@@ -140,8 +140,8 @@ def test_gemv_and_dlrm_argument_validation(lib):
     assert gx(BF16, 4096, 8192, 27, 128, 8, None) == 2 and hx(I8, 4096, 8192, 12288, 16384, 27, 128, 8, None) == 2
     for t in (F16, F32):
         assert gx(t, None, 4096, 27, 128, 8, None) == 1
-        assert gx(t, 4096, 8192, 129, 128, 8, None) == 3
-        assert gx(t, 4096, 8192, 27, 100, 8, None) == 3
+        assert gx(t, 4096, 8192, 40000, 128, 8, None) == 3
+        assert gx(t, 4096, 8192, 27, 102, 8, None) == 3 and hx(t, 4096, 8192, 12288, 16384, 200, 1026, 8, None) == 3
         assert hx(t, 4096, 8192, 12288, None, 27, 128, 8, None) == 1
         assert hx(t, 4096, 8192, 12290, 16384, 27, 128, 8, None) == 4
 
