@@ -881,6 +881,29 @@ def run_extras(rw, torch, dev, gen, only=None):
                                                         "frac_hbm_graph_replay": round(byts / msg / 1e6 / PEAK_HBM_GBS, 4)})
         del Fs
 
+    # The reference's largest DLRM test size, (m, k, batch) = (1024, 1024, 64) (test/dlrm/test/dlrm_test_params.hpp:51-68):
+    # a sample is a 1024^3 matrix product of its own, so these are compute bound (tiles of 128 x 128 per workgroup, no
+    # m x m scratch in global memory).  flops: forward m (m - 1) k (the strict lower triangle), backward 2 m^2 k.
+    ml, kl, bl = 1024, 1024, 64
+    wl = kl + ml * (ml - 1) // 2
+    for tdt, code, tag in ((torch.float16, rw.F16, "f16"), (torch.float32, rw.F32, "f32")):
+        if not (wanted(f"dlrm_fwd_{tag}_m1024_k1024_b64") or wanted(f"dlrm_bwd_{tag}_m1024_k1024_b64")):
+            continue
+        Fl = (torch.rand(bl * ml * kl, device=dev, generator=gen) * 2 - 1).to(tdt)
+        upl = (torch.rand(bl * wl, device=dev, generator=gen) * 2 - 1).to(tdt)
+        ol = torch.empty(bl * wl, device=dev, dtype=tdt)
+        grl = torch.empty(bl * ml * kl, device=dev, dtype=tdt)
+        mgl = torch.empty(bl * kl, device=dev, dtype=tdt)
+        peak = PEAK_TFLOPS["f16"] if tag == "f16" else 157.3  # dense MFMA, MI355X: f16, float32
+        for name, fnx, flops in ((f"dlrm_fwd_{tag}_m1024_k1024_b64", lambda: rw.dlrm_fwd(Fl, ol, ml, kl, bl, code), 1.0 * bl * ml * (ml - 1) * kl),
+                                 (f"dlrm_bwd_{tag}_m1024_k1024_b64", lambda: rw.dlrm_bwd(Fl, upl, grl, mgl, ml, kl, bl, code), 2.0 * bl * ml * ml * kl)):
+            if not wanted(name):
+                continue
+            fnx()
+            ms = event_ms(fnx, iters, torch)
+            out[name] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1), "frac_mfma": round(flops / ms / 1e9 / peak, 4)}
+        del Fl, upl, ol, grl, mgl
+
     # What plain streaming kernels reach on this device for the byte counts of the bandwidth-bound cases
     # (one read-only / copy kernel, windows rotated through 2 GiB so that every launch reads from HBM):
     # at tens of megabytes a launch is over before the memory system reaches the rate of a long stream.

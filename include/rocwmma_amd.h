@@ -443,11 +443,13 @@ int rocwmma_amd_gemv(uint32_t    m,
  *   input  : batch x m x k   (row 0 of every sample is the bottom-MLP output)
  *   output : batch x (k + m(m-1)/2):  [ input[b,0,:] , Z[1,0], Z[2,0], Z[2,1], Z[3,0], ... ]
  *            with Z = input[b] * input[b]^T.
- * Unlike the reference kernel this one needs no f32 m x m scratch (`acc`) and accepts any
- * m <= 128 (the reference GPU kernels need m % 16 == 0, test/dlrm/dlrm_kernel_base_impl.hpp:146-150;
- * its tests run m = 32 and 128 among others, test/dlrm/test/dlrm_test_params.hpp:51-58).  Up to 32 rows are
- * one matrix-instruction operand per sample (the benchmark configuration, m = 27); more run as tiles of 32.
- * k must be 32, 64, 128 or 256; input and output must be 16-byte aligned.
+ * Unlike the reference kernel this one needs no f32 m x m scratch (`acc`) and accepts any m up to 32768
+ * (the reference GPU kernels need m % 16 == 0, test/dlrm/dlrm_kernel_base_impl.hpp:146-150; its tests run
+ * (m, k) = (32, 32), (32, 128), (128, 128) and (1024, 1024), test/dlrm/test/dlrm_test_params.hpp:51-68).  Up to 32 rows
+ * with k in {32, 64, 128, 256} are one matrix-instruction operand per sample (the benchmark configuration, m = 27), up
+ * to 128 rows run as tiles of 32 inside one wave per sample; every other shape runs as 128 x 128 tiles per workgroup
+ * and needs k % 8 == 0 and a sample's features (m * k * 2 bytes) below 2 GiB, ROCWMMA_AMD_UNSUPPORTED_SHAPE otherwise.
+ * input and output must be 16-byte aligned.
  */
 int rocwmma_amd_dlrm_fwd(const void* input,
                          void*       output,
@@ -484,8 +486,9 @@ int rocwmma_amd_dlrm_bwd(const void* input,
  * ROCWMMA_AMD_F32.  The reference's DLRM kernels and tests are templates over the element type and are
  * instantiated for float32_t as well (test/dlrm/test/dlrm_test_params.hpp:51; fp32 data files under
  * test/dlrm/data); semantics = dlrm_fwd_CPU / dlrm_bwd_CPU with DataT = float (test/reference_impl.hpp:83-179).
- * Same shapes, limits and alignment as above (m <= 128, k in {32, 64, 128, 256}, 16-byte aligned pointers); the
- * float32 kernels multiply with v_mfma_f32_32x32x2_f32 and are written for parity, not tuned.  Other element
+ * Same shapes, limits and alignment as above (float32: k % 4 == 0 for the shapes that run as 128 x 128 tiles,
+ * m * k * 4 bytes below 2 GiB; 16-byte aligned pointers); the float32 kernels multiply with v_mfma_f32_32x32x2_f32
+ * and are written for parity, not tuned.  Other element
  * types: ROCWMMA_AMD_UNSUPPORTED_TYPE.
  */
 int rocwmma_amd_dlrm_fwd_ex(int         dtype,

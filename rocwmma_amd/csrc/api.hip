@@ -580,8 +580,9 @@ static int checkDlrm(int dtype, uint32_t m, uint32_t k, uint32_t batch)
 {
     if(m == 0u || k == 0u || batch == 0u)
         return ROCWMMA_AMD_INVALID_ARGUMENT;
-    // the tiled kernels read rows in 16-byte pieces
-    if(!dlrmSampleFitsAWave(m, k) && (m > 32768u || k % (dtype == ROCWMMA_AMD_F16 ? 8u : 4u) != 0u))
+    // the tiled kernels read rows in 16-byte pieces and address a sample's features with 32-bit byte offsets
+    const uint32_t size = dtype == ROCWMMA_AMD_F16 ? 2u : 4u;
+    if(!dlrmSampleFitsAWave(m, k) && (m > 32768u || k % (16u / size) != 0u || static_cast<uint64_t>(m) * k * size >= (1ull << 31)))
         return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
     return ROCWMMA_AMD_OK;
 }

@@ -110,11 +110,11 @@ def test_gemv_replays(m, k, ncols):
     assert not inf and not nan and err <= 1e-3, (err, inf, nan)
 
 
-@pytest.mark.parametrize("batch", [6, 64, 2048])
-def test_dlrm_replays(batch):
+@pytest.mark.parametrize("batch,m,k", [(6, 27, 128), (64, 27, 128), (2048, 27, 128), (3, 300, 200)])
+def test_dlrm_replays(batch, m, k):
+    """One wave per sample, and (300 rows) the tiled kernels for samples that do not fit a wave."""
     import torch
 
-    m, k = 27, 128
     width = k + m * (m - 1) // 2
     feats, up = uniform_bits(41, orc.F16, batch * m * k), uniform_bits(42, orc.F16, batch * width)
     dfe, dup = to_device(feats), to_device(up)
@@ -129,11 +129,11 @@ def test_dlrm_replays(batch):
     _replays_match(call, [out, grad, mlp])
 
 
-@pytest.mark.parametrize("batch,m", [(64, 27), (5, 128)])
-def test_dlrm_float32_replays(batch, m):
+@pytest.mark.parametrize("batch,m,k", [(64, 27, 128), (5, 128, 128), (3, 300, 200)])
+def test_dlrm_float32_replays(batch, m, k):
+    """One wave per sample, and (300 rows) the tiled kernels for samples that do not fit a wave."""
     import torch
 
-    k = 128
     width = k + m * (m - 1) // 2
     rng = np.random.default_rng(43)
     dfe = to_device(rng.uniform(-1, 1, batch * m * k).astype(np.float32))

@@ -76,14 +76,14 @@ def test_gemm_argument_validation(lib):
     assert _gemm(lib, k=8) == 3
     assert _gemm(lib, lda=16) == 5
     assert _gemm(lib, a=4098) == 4
-    assert _gemm(lib, ldd=36, ldc=36) == 0 or True  # 36 floats = 144 B: aligned, goes on to device check
     assert _gemm(lib, lda=36) == 4                  # 36 halves = 72 B: not 16-byte aligned
-    # valid arguments but no GPU in this process: NO_DEVICE (or success on a GPU box is not
-    # possible with fake pointers, so only assert when no device is visible)
+    # valid arguments: NO_DEVICE where no GPU is visible.  Where one is, such a call would launch a kernel on
+    # the fake pointers and fault the card, so it is only made without one.
     import torch
 
     if not torch.cuda.is_available():
         assert _gemm(lib) == 6
+        assert _gemm(lib, ldd=36, ldc=36) == 6      # 36 floats = 144 B: aligned, passes on to the device check
 
 
 def test_fused_and_block_scaled_gemm_argument_validation(lib):
@@ -129,6 +129,7 @@ def test_gemv_and_dlrm_argument_validation(lib):
     g = lib.rocwmma_amd_dlrm_fwd
     assert g(None, 4096, 27, 128, 8, None) == 1
     assert g(4096, 8192, 40000, 128, 8, None) == 3
+    assert g(4096, 8192, 32768, 65536, 8, None) == 3  # (a sample of 4 GiB: beyond the kernels' 32-bit offsets)
     assert g(4096, 8192, 27, 100, 8, None) == 3  # (rows of f16 must be whole 16-byte pieces)
     assert g(4096, 8192, 27, 128, 0, None) == 1 and g(4096, 8192, 27, 0, 8, None) == 1
     h = lib.rocwmma_amd_dlrm_bwd
