@@ -33,7 +33,6 @@ namespace rocwmma_amd
 
         constexpr uint32_t kTile       = 128; // workgroup tile edge
         constexpr uint32_t kWaveTile   = 64;
-        constexpr uint32_t kMaxGridY   = 32768;
         constexpr uint32_t kMaxRows    = 32768; // m * (m - 1) stays below 2^32
         constexpr uint32_t kNowhere    = 0x80000000u; // beyond every sample: a bounds-checked load there returns zero
 
@@ -50,9 +49,17 @@ namespace rocwmma_amd
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
 
-        ROCWMMA_DEVICE inline uint32_t sampleOfBlock()
+        // Which (sample, tile) a workgroup takes.  Workgroups are handed to the device's 8 XCDs in turn (workgroup w
+        // runs on XCD w % 8), and every XCD has an L2 of its own: all tiles of a sample go to one XCD, sample s to XCD
+        // s % 8, so that a sample's operands are fetched into one L2 once instead of into all eight (measured at
+        // (1024, 1024, 64) in f16: 955 MiB fetched per forward launch for 128 MiB of features with the tiles of a
+        // sample dealt out over the XCDs).  The grid is 8 * ceil(batch / 8) * tiles workgroups.
+        constexpr uint32_t kXcds = 8;
+        ROCWMMA_DEVICE inline void sampleAndTile(uint32_t tiles, uint32_t& sample, uint32_t& tile)
         {
-            return blockIdx.z * gridDim.y + blockIdx.y;
+            const uint32_t slot = blockIdx.x / kXcds;
+            sample              = (slot / tiles) * kXcds + blockIdx.x % kXcds;
+            tile                = slot % tiles;
         }
 
         // ------------------------------------------------------------------ operands through LDS
@@ -107,23 +114,26 @@ namespace rocwmma_amd
             return *reinterpret_cast<const u32x4_t*>(tile + (block32 * 32u + (lane & 31u)) * kRowPitch + ks * 32u + (lane >> 5) * 16u);
         }
 
-        // issues the two transposing reads of the fragment of 32-column block `block32` at K step `ks` of a "columns"
-        // tile: lane l gets column block32 * 32 + l % 32 and contraction rows ks * 16 + (l / 32) * 8 + 0..7.  The
-        // caller waits (lgkmcnt) before it touches `words`.
-        ROCWMMA_DEVICE inline void columnsFragmentIssue(uint32_t (&words)[4], uint32_t ldsTile, uint32_t block32, uint32_t ks, uint32_t lane)
+        // fragment words of 32-column block `block32` at K step `ks` of a "columns" tile: lane l gets column
+        // block32 * 32 + l % 32 and contraction rows ks * 16 + (l / 32) * 8 + 0..7, as two transposing 8-byte reads
+        // (through the compiler's builtin, so that it keeps the wait counters and schedules the reads itself)
+        typedef short s16x4_t __attribute__((ext_vector_type(4)));
+        ROCWMMA_DEVICE inline u32x4_t columnsFragment(const char* tile, uint32_t block32, uint32_t ks, uint32_t lane)
         {
             const uint32_t group = lane >> 4, s16 = lane & 15u;
+            u32x4_t        words;
 #pragma unroll
             for(uint32_t kk = 0; kk < 2u; ++kk)
             {
-                const uint32_t row  = ks * 16u + (group >> 1) * 8u + kk * 4u + (s16 >> 2);
-                const uint32_t seg  = block32 * 2u + (group & 1u);
-                const uint32_t addr = ldsTile + row * kColBytes + ((seg ^ segmentSwizzle(row)) << 5) + ((s16 & 3u) << 3);
-                u32x2_t        v;
-                asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
-                words[2u * kk]      = v[0];
-                words[2u * kk + 1u] = v[1];
+                const uint32_t row = ks * 16u + (group >> 1) * 8u + kk * 4u + (s16 >> 2);
+                const uint32_t seg = block32 * 2u + (group & 1u);
+                const char*    at  = tile + row * kColBytes + ((seg ^ segmentSwizzle(row)) << 5) + ((s16 & 3u) << 3);
+                const s16x4_t  v   = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)at);
+                const u32x2_t  w   = __builtin_bit_cast(u32x2_t, v);
+                words[2u * kk]      = w[0];
+                words[2u * kk + 1u] = w[1];
             }
+            return words;
         }
 
         template <typename Frag>
@@ -154,8 +164,8 @@ namespace rocwmma_amd
         // per stage, four v_mfma_f32_32x32x2_f32 per piece and block, one per word (the order in which K is contracted
         // is free as long as both multiplicands agree: instruction t of a piece contracts word t of both lane halves)
         template <typename T>
-        __global__ void __launch_bounds__(256)
-            dlrmFwdStagedKernel(const T* __restrict__ input, T* __restrict__ output, uint32_t m, uint32_t k, uint32_t batch)
+        __global__ void __launch_bounds__(256, 3)
+            dlrmFwdStagedKernel(const T* __restrict__ input, T* __restrict__ output, uint32_t m, uint32_t k, uint32_t batch, uint32_t tiles)
         {
             constexpr uint32_t KI = sizeof(T) == 2u ? 16u : 2u;
             using FragK           = fragment<matrix_a, 32, 32, KI, T, row_major>;
@@ -169,14 +179,14 @@ namespace rocwmma_amd
             char* const ldsA = lds;
             char* const ldsB = lds + kRowsBytes;
 
-            const uint32_t sample = sampleOfBlock();
+            uint32_t sample, t; // t: tiles of the lower triangle, row by row
+            sampleAndTile(tiles, sample, t);
             if(sample >= batch) // (the whole workgroup)
                 return;
             const uint32_t tid  = threadIdx.x;
             const uint32_t lane = tid & 63u;
             const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-            const uint32_t t = blockIdx.x; // tiles of the lower triangle, row by row
             uint32_t       I = static_cast<uint32_t>((__builtin_sqrtf(8.0f * static_cast<float>(t) + 1.0f) - 1.0f) * 0.5f);
             while(I * (I + 1u) / 2u > t)
                 --I;
@@ -306,7 +316,7 @@ namespace rocwmma_amd
                 }
         }
 
-        __global__ void __launch_bounds__(256) dlrmBwdStagedF16Kernel(const float16_t* __restrict__ input,
+        __global__ void __launch_bounds__(256, 3) dlrmBwdStagedF16Kernel(const float16_t* __restrict__ input,
                                                                          const float16_t* __restrict__ upstream,
                                                                          float16_t* __restrict__ grad,
                                                                          float16_t* __restrict__ mlpGrad,
@@ -321,13 +331,14 @@ namespace rocwmma_amd
             __shared__ __attribute__((aligned(16))) char ldsS[kRowsBytes]; // "rows" or "columns" layout, by stage
             __shared__ __attribute__((aligned(16))) char ldsF[kColsBytes]; // "columns" layout
 
-            const uint32_t sample = sampleOfBlock();
+            uint32_t sample, t;
+            sampleAndTile(((m + kTile - 1u) / kTile) * colTiles, sample, t);
             if(sample >= batch) // (the whole workgroup)
                 return;
             const uint32_t tid  = threadIdx.x;
             const uint32_t lane = tid & 63u;
             const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-            const uint32_t I = blockIdx.x / colTiles, N = blockIdx.x % colTiles;
+            const uint32_t I = t / colTiles, N = t % colTiles;
             const uint32_t I0 = I * kTile, N0 = N * kTile;
 
             const size_t     width = packedRow(k, m);
@@ -335,14 +346,12 @@ namespace rocwmma_amd
             const float16_t* up    = upstream + static_cast<size_t>(sample) * width;
             float16_t*       dst   = grad + static_cast<size_t>(sample) * m * k;
 
-            if(blockIdx.x == 0u) // bottom-MLP gradient = the first k entries of the upstream row
+            if(t == 0u) // bottom-MLP gradient = the first k entries of the upstream row
                 for(uint32_t e = tid; e < k; e += 256u)
                     mlpGrad[static_cast<size_t>(sample) * k + e] = up[e];
 
             const uint32_t wr = wave >> 1, wc = wave & 1u;
             const bool     waveLive = I0 + wr * kWaveTile < m && N0 + wc * kWaveTile < k; // (every wave stages and meets the barriers)
-            const uint32_t ldsSBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds::LdsPtr)ldsS));
-            const uint32_t ldsFBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds::LdsPtr)ldsF));
 
             // Where a stage of 64 contraction indices c0 .. lies against the tile's rows I0 .. I0 + 127 decides how S
             // arrives (workgroup uniform):
@@ -426,44 +435,15 @@ namespace rocwmma_amd
 #pragma unroll
                     for(uint32_t ks = 0; ks < kStageK / 16u; ++ks)
                     {
-                        uint32_t fw[2][4], sw[2][4];
-#pragma unroll
-                        for(uint32_t j = 0; j < 2u; ++j)
-                            columnsFragmentIssue(fw[j], ldsFBase, wc * 2u + j, ks, lane);
                         FragK16 a[2];
-                        if(where == Above)
-                        {
-#pragma unroll
-                            for(uint32_t i = 0; i < 2u; ++i)
-                                columnsFragmentIssue(sw[i], ldsSBase, wr * 2u + i, ks, lane);
-                        }
-                        else
-                        {
-#pragma unroll
-                            for(uint32_t i = 0; i < 2u; ++i)
-                                a[i] = fragmentOf<FragK16>(rowsFragment(ldsS, wr * 2u + i, ks, lane));
-                        }
-                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                        FragF b[2];
+                        FragF   b[2];
 #pragma unroll
                         for(uint32_t j = 0; j < 2u; ++j)
+                            b[j] = fragmentOf<FragF>(columnsFragment(ldsF, wc * 2u + j, ks, lane));
 #pragma unroll
-                            for(uint32_t w = 0; w < 4u; ++w)
-                            {
-                                asm volatile("" : "+v"(fw[j][w]));
-                                reinterpret_cast<uint32_t*>(b[j].x)[w] = fw[j][w];
-                            }
-                        if(where == Above)
-                        {
-#pragma unroll
-                            for(uint32_t i = 0; i < 2u; ++i)
-#pragma unroll
-                                for(uint32_t w = 0; w < 4u; ++w)
-                                {
-                                    asm volatile("" : "+v"(sw[i][w]));
-                                    reinterpret_cast<uint32_t*>(a[i].x)[w] = sw[i][w];
-                                }
-                        }
+                        for(uint32_t i = 0; i < 2u; ++i)
+                            a[i] = fragmentOf<FragK16>(where == Above ? columnsFragment(ldsS, wr * 2u + i, ks, lane)
+                                                                      : rowsFragment(ldsS, wr * 2u + i, ks, lane));
 #pragma unroll
                         for(uint32_t i = 0; i < 2u; ++i)
 #pragma unroll
@@ -505,7 +485,7 @@ namespace rocwmma_amd
         constexpr uint32_t kColPitch32 = 544;
         constexpr uint32_t kColsBytes32 = kStageK32 * kColPitch32; // 17408
 
-        __global__ void __launch_bounds__(256) dlrmBwdStagedF32Kernel(const float* __restrict__ input,
+        __global__ void __launch_bounds__(256, 3) dlrmBwdStagedF32Kernel(const float* __restrict__ input,
                                                                          const float* __restrict__ upstream,
                                                                          float* __restrict__ grad,
                                                                          float* __restrict__ mlpGrad,
@@ -522,13 +502,14 @@ namespace rocwmma_amd
             __shared__ __attribute__((aligned(16))) char ldsS[kRowsBytes]; // "rows" or "columns" layout, by stage
             __shared__ __attribute__((aligned(16))) char ldsF[kColsBytes32]; // "columns" layout
 
-            const uint32_t sample = sampleOfBlock();
+            uint32_t sample, t;
+            sampleAndTile(((m + kTile - 1u) / kTile) * colTiles, sample, t);
             if(sample >= batch) // (the whole workgroup)
                 return;
             const uint32_t tid  = threadIdx.x;
             const uint32_t lane = tid & 63u;
             const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-            const uint32_t I = blockIdx.x / colTiles, N = blockIdx.x % colTiles;
+            const uint32_t I = t / colTiles, N = t % colTiles;
             const uint32_t I0 = I * kTile, N0 = N * kTile;
 
             const size_t width = packedRow(k, m);
@@ -536,7 +517,7 @@ namespace rocwmma_amd
             const float* up    = upstream + static_cast<size_t>(sample) * width;
             float*       dst   = grad + static_cast<size_t>(sample) * m * k;
 
-            if(blockIdx.x == 0u) // bottom-MLP gradient = the first k entries of the upstream row
+            if(t == 0u) // bottom-MLP gradient = the first k entries of the upstream row
                 for(uint32_t e = tid; e < k; e += 256u)
                     mlpGrad[static_cast<size_t>(sample) * k + e] = up[e];
 
@@ -679,10 +660,11 @@ namespace rocwmma_amd
                     }
         }
 
-        inline dim3 gridFor(uint32_t tiles, uint32_t batch)
+        // workgroups of a launch (see sampleAndTile), 0 if they do not fit a grid dimension
+        inline uint32_t gridFor(uint32_t tiles, uint32_t batch)
         {
-            const uint32_t y = batch < kMaxGridY ? batch : kMaxGridY;
-            return dim3(tiles, y, (batch + y - 1u) / y);
+            const uint64_t workgroups = static_cast<uint64_t>((batch + kXcds - 1u) / kXcds) * kXcds * tiles;
+            return workgroups <= 0x7FFFFFFFull ? static_cast<uint32_t>(workgroups) : 0u;
         }
     } // namespace
 
@@ -693,14 +675,16 @@ namespace rocwmma_amd
         const uint32_t size = dtype == ROCWMMA_AMD_F16 ? 2u : 4u;
         if(m > kMaxRows || k == 0u || k % (16u / size) != 0u || static_cast<uint64_t>(m) * k * size >= (1ull << 31))
             return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-        const uint32_t side = (m + kTile - 1u) / kTile;
-        const dim3     grid = gridFor(side * (side + 1u) / 2u, batch);
+        const uint32_t side = (m + kTile - 1u) / kTile, tiles = side * (side + 1u) / 2u;
+        const uint32_t grid = gridFor(tiles, batch);
+        if(grid == 0u)
+            return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
         if(dtype == ROCWMMA_AMD_F16)
-            hipLaunchKernelGGL(dlrmFwdStagedKernel<float16_t>, grid, dim3(256), 0, stream, static_cast<const float16_t*>(input),
-                               static_cast<float16_t*>(output), m, k, batch);
+            hipLaunchKernelGGL(dlrmFwdStagedKernel<float16_t>, dim3(grid), dim3(256), 0, stream, static_cast<const float16_t*>(input),
+                               static_cast<float16_t*>(output), m, k, batch, tiles);
         else
-            hipLaunchKernelGGL(dlrmFwdStagedKernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(input),
-                               static_cast<float*>(output), m, k, batch);
+            hipLaunchKernelGGL(dlrmFwdStagedKernel<float>, dim3(grid), dim3(256), 0, stream, static_cast<const float*>(input),
+                               static_cast<float*>(output), m, k, batch, tiles);
         return launchStatus();
     }
 
@@ -713,13 +697,15 @@ namespace rocwmma_amd
         const uint32_t rowTiles = (m + kTile - 1u) / kTile, colTiles = (k + kTile - 1u) / kTile;
         if(static_cast<uint64_t>(rowTiles) * colTiles > 0x7FFFFFFFull)
             return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
-        const dim3 grid = gridFor(rowTiles * colTiles, batch);
+        const uint32_t grid = gridFor(rowTiles * colTiles, batch);
+        if(grid == 0u)
+            return ROCWMMA_AMD_UNSUPPORTED_SHAPE;
         if(dtype == ROCWMMA_AMD_F16)
-            hipLaunchKernelGGL(dlrmBwdStagedF16Kernel, grid, dim3(256), 0, stream, static_cast<const float16_t*>(input),
+            hipLaunchKernelGGL(dlrmBwdStagedF16Kernel, dim3(grid), dim3(256), 0, stream, static_cast<const float16_t*>(input),
                                static_cast<const float16_t*>(upstream), static_cast<float16_t*>(grad), static_cast<float16_t*>(mlpGrad), m,
                                k, batch, colTiles);
         else
-            hipLaunchKernelGGL(dlrmBwdStagedF32Kernel, grid, dim3(256), 0, stream, static_cast<const float*>(input),
+            hipLaunchKernelGGL(dlrmBwdStagedF32Kernel, dim3(grid), dim3(256), 0, stream, static_cast<const float*>(input),
                                static_cast<const float*>(upstream), static_cast<float*>(grad), static_cast<float*>(mlpGrad), m, k, batch,
                                colTiles);
         return launchStatus();
