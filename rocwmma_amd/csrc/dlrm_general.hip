@@ -65,8 +65,8 @@ namespace rocwmma_amd
         // ------------------------------------------------------------------ operands through LDS
         // In the fragment layout consecutive lanes hold different rows, and a global load whose lanes touch 32
         // different cache lines is served at a fraction of the rate of one whose lanes read consecutive addresses
-        // (operands straight from global memory: 204 instead of 400 TFLOP/s forward, 110 instead of 290 backward at
-        // (1024, 1024, 64) in f16).  So a thread fetches consecutive 16-byte pieces of a tile row into registers (one
+        // (with operands straight from global memory the f16 kernels ran at half (forward) and at 0.4 (backward) of
+        // the rate at (1024, 1024, 64)).  So a thread fetches consecutive 16-byte pieces of a tile row into registers (one
         // stage ahead of the multiplication), the pieces go to LDS, and the fragments come from there.
         //
         // Two LDS layouts for float16, 64 contraction indices per stage (float32 below):
