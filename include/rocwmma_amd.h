@@ -178,8 +178,8 @@ int rocwmma_amd_gemm_ex(int         algo,
  * The reference has no counterpart: its GEMM hosts launch plain 2-D grids
  * (samples/perf_hgemm.cpp:810-812).
  *
- * Types: F16 / BF16 inputs with F32 C/D in every layout pair; I8 -> I32 and E4M3 / E5M2 -> F32 with
- * row-major A and col-major B.  m and n multiples of 256, k a multiple of 128 bytes' worth of
+ * Types: F16 / BF16 inputs with F32 C/D, I8 -> I32 and E4M3 / E5M2 -> F32, each in every layout
+ * pair.  m and n multiples of 256, k a multiple of 128 bytes' worth of
  * elements; other shapes return ROCWMMA_AMD_UNSUPPORTED_SHAPE (use rocwmma_amd_gemm).
  * workspace: device memory, 256-byte aligned, at least rocwmma_amd_gemm_streamk_workspace_size()
  * bytes (64 MiB + 1.25 KiB on a 256-unit device); contents need not be initialised and are not

@@ -185,18 +185,13 @@ namespace rocwmma_amd
         {
             const bool ak = layoutA == ROCWMMA_AMD_ROW_MAJOR;
             const bool bk = layoutB == ROCWMMA_AMD_COL_MAJOR;
-            if constexpr(sizeof(InT) == 2u)
-            {
-                if(ak && !bk)
-                    return launchStreamK<BigConfig<InT, OutT, CompT, true, false>>(g, ws, wsBytes, stream);
-                if(!ak && bk)
-                    return launchStreamK<BigConfig<InT, OutT, CompT, false, true>>(g, ws, wsBytes, stream);
-                if(!ak && !bk)
-                    return launchStreamK<BigConfig<InT, OutT, CompT, false, false>>(g, ws, wsBytes, stream);
-            }
-            if(ak && bk)
-                return launchStreamK<BigConfig<InT, OutT, CompT, true, true>>(g, ws, wsBytes, stream);
-            return ROCWMMA_AMD_UNSUPPORTED_SHAPE; // 8-bit operands: the K-contiguous pairing only
+            if(ak && !bk)
+                return launchStreamK<BigConfig<InT, OutT, CompT, true, false>>(g, ws, wsBytes, stream);
+            if(!ak && bk)
+                return launchStreamK<BigConfig<InT, OutT, CompT, false, true>>(g, ws, wsBytes, stream);
+            if(!ak && !bk)
+                return launchStreamK<BigConfig<InT, OutT, CompT, false, false>>(g, ws, wsBytes, stream);
+            return launchStreamK<BigConfig<InT, OutT, CompT, true, true>>(g, ws, wsBytes, stream);
         }
     } // namespace
 
