@@ -114,6 +114,10 @@ def parse_args():
     return ap.parse_args()
 
 
+def compute_units_of(rw):
+    return rw.device_info()["compute_units"]
+
+
 def event_ms(fn, iters, torch):
     """Average duration of fn() in ms over `iters` launches, events on the current stream."""
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -946,6 +950,16 @@ def run_extras(rw, torch, dev, gen, only=None):
             moved = nbytes * {rw.STREAM_COPY: 2.0, rw.STREAM_COPY_READ_MORE: 2.1}.get(mode, 1.0)
             ceil[tag] = {"ms": round(ms, 5), "ms_graph_replay": None if msg is None else round(msg, 5),
                          "gbs": round(moved / best / 1e6, 1), "frac_hbm": round(moved / best / 1e6 / PEAK_HBM_GBS, 4)}
+        # what the compute units can draw from their L2s: 16 MiB (one workgroup per compute unit re-reading its
+        # own 64 KiB, 2 MiB per XCD) read 256 times in one launch; the operand streams of the tiled kernels
+        # (L2 -> LDS copies of the GEMM, of the tiled DLRM kernels) are a fraction of this rate
+        nres = 16 * MiB
+        res_fn = lambda: rw.bench_stream(rw.STREAM_READ_RESIDENT, src, dst, nres)
+        res_fn()
+        ms = event_ms(res_fn, iters, torch)
+        moved = float(nres) * rw.STREAM_RESIDENT_PASSES
+        ceil["l2_resident_read_16MiB"] = {"ms": round(ms, 5), "gbs": round(moved / ms / 1e6, 1),
+                                          "gbs_per_compute_unit": round(moved / ms / 1e6 / compute_units_of(rw), 1)}
         del src, dst
         out["stream_ceiling"] = ceil
         # the bandwidth-bound cases against the plain stream of the nearest size and kind

@@ -145,9 +145,13 @@ int rocwmma_amd_bench_mfma_streams(int         kind,
  * mode 1 writes `dst`, mode 2 copies `src` to `dst`, mode 3 copies `src` to `dst` and reads a tenth as much again
  * from the `bytes` bytes behind `src`'s first `bytes` (so `src` holds 2 * bytes; 4 writable bytes behind `dst`'s
  * `bytes`): 1.1 bytes read per byte written, the mix of the DLRM backward pass.  The bandwidth-bound workloads
- * are priced against what this reaches for their byte counts on the same device.  Has no counterpart in the
- * reference.
+ * are priced against what this reaches for their byte counts on the same device.  mode 4 reads `src`'s `bytes`
+ * ROCWMMA_AMD_STREAM_RESIDENT_PASSES times over, one workgroup of 1024 threads per 64 KiB chunk re-reading its own
+ * chunk (4 writable bytes at `dst`): with 16 MiB (one workgroup per compute unit, 2 MiB per XCD) every pass after the
+ * first is served by the L2s, which is the rate the operand streams of the tiled kernels are priced against.
+ * Has no counterpart in the reference.
  */
+#define ROCWMMA_AMD_STREAM_RESIDENT_PASSES 256
 int rocwmma_amd_bench_stream(int mode, const void* src, void* dst, size_t bytes, void* stream);
 
 #ifdef __cplusplus

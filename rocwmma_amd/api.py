@@ -366,7 +366,8 @@ def selftest_tiled_gemm(layout_a, layout_b, m, n, k, a, b, c, d, alpha, beta):
     return d
 
 
-STREAM_READ, STREAM_WRITE, STREAM_COPY, STREAM_COPY_READ_MORE = 0, 1, 2, 3
+STREAM_READ, STREAM_WRITE, STREAM_COPY, STREAM_COPY_READ_MORE, STREAM_READ_RESIDENT = 0, 1, 2, 3, 4
+STREAM_RESIDENT_PASSES = 256  # ROCWMMA_AMD_STREAM_RESIDENT_PASSES: mode 4 reads its bytes this many times
 
 
 def bench_stream(mode, src, dst, nbytes, stream=None):

@@ -164,7 +164,7 @@ namespace rocwmma_amd
         // per stage, four v_mfma_f32_32x32x2_f32 per piece and block, one per word (the order in which K is contracted
         // is free as long as both multiplicands agree: instruction t of a piece contracts word t of both lane halves)
         template <typename T>
-        __global__ void __launch_bounds__(256, 3)
+        __global__ void __launch_bounds__(256, sizeof(T) == 2u ? 4 : 3) // (waves per SIMD that fit without spills)
             dlrmFwdStagedKernel(const T* __restrict__ input, T* __restrict__ output, uint32_t m, uint32_t k, uint32_t batch, uint32_t tiles)
         {
             constexpr uint32_t KI = sizeof(T) == 2u ? 16u : 2u;

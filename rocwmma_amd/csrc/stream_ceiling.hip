@@ -84,9 +84,40 @@ namespace rocwmma_amd
             if(ExtraReads && acc == 0x12345678u) // (keeps the extra loads alive; practically never true)
                 sink[0] = acc;
         }
+
+        // What a compute unit can draw from its XCD's L2: one workgroup of 1024 threads per 64 KiB chunk reads its own
+        // chunk kResidentPasses times with plain 16-byte loads, all of the chunk in flight at once.  A chunk is twice
+        // the vector L1, read cyclically, so every pass misses the L1; workgroup w runs on XCD w % 8, so with 16 MiB
+        // (one workgroup per compute unit) every L2 holds 2 MiB of its 4: every pass after the first hits the L2.
+        // The operand streams of the tiled kernels (GEMM, the tiled DLRM kernels, the M = 128 weight-streaming case)
+        // are priced against this.
+        constexpr uint32_t kResidentPasses = 256;
+        constexpr size_t   kResidentChunkVecs = 65536u / 16u;
+
+        __global__ void __launch_bounds__(kWideThreads) streamResidentReadKernel(const u32x4* __restrict__ src, uint32_t* sink)
+        {
+            const u32x4* mine = src + static_cast<size_t>(blockIdx.x) * kResidentChunkVecs + threadIdx.x;
+            uint32_t     acc  = 0;
+#pragma unroll 1
+            for(uint32_t pass = 0; pass < kResidentPasses; ++pass)
+            {
+                const u32x4* from = mine;
+                asm volatile("" : "+v"(from)); // (the same addresses every pass: keeps the loads inside the loop)
+                u32x4 v[kWideUnroll];
+#pragma unroll
+                for(uint32_t u = 0; u < kWideUnroll; ++u)
+                    v[u] = from[u * kWideThreads];
+#pragma unroll
+                for(uint32_t u = 0; u < kWideUnroll; ++u)
+                    acc += v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+            }
+            if(acc == 0x12345678u) // (keeps the loads alive; practically never true)
+                sink[0] = acc;
+        }
     } // namespace
 
-    // mode 0: read `bytes` from src; 1: write `bytes` to dst; 2: copy `bytes` from src to dst; 3: copy with a tenth more reads.
+    // mode 0: read `bytes` from src; 1: write `bytes` to dst; 2: copy `bytes` from src to dst; 3: copy with a tenth more reads;
+    // 4: read `bytes` 256 times, cache resident.
     // bytes must be a multiple of 64 KiB (whole trips of the unrolled loops for every workgroup size used).
     int benchStream(int mode, const void* src, void* dst, size_t bytes, hipStream_t stream)
     {
@@ -127,6 +158,12 @@ namespace rocwmma_amd
             hipLaunchKernelGGL(streamCopyKernel<true>, dim3(static_cast<uint32_t>(grid)), dim3(kWideThreads), 0, stream,
                                static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), vecs,
                                reinterpret_cast<uint32_t*>(static_cast<char*>(dst) + bytes));
+            break;
+        case 4: // read every 64 KiB chunk of `bytes` kResidentPasses times, one workgroup per chunk (4 bytes of dst are the sink)
+            if(!src || !dst)
+                return ROCWMMA_AMD_INVALID_ARGUMENT;
+            hipLaunchKernelGGL(streamResidentReadKernel, dim3(static_cast<uint32_t>(bytes / 65536u)), dim3(kWideThreads), 0, stream,
+                               static_cast<const u32x4*>(src), static_cast<uint32_t*>(dst));
             break;
         default:
             return ROCWMMA_AMD_INVALID_ARGUMENT;

@@ -68,6 +68,14 @@ def test_memory_stream_probes_move_what_they_say():
     assert int(dst[n:].sum()) == 0
     rw.bench_stream(rw.STREAM_READ, src, dst, n)
     torch.cuda.synchronize()
+    # the cache-resident read: reads its bytes over and over and writes nothing but (practically never) its sink word
+    dst.zero_()
+    rw.bench_stream(rw.STREAM_READ_RESIDENT, src, dst, n)
+    torch.cuda.synchronize()
+    assert int(dst[4:].sum()) == 0
+    with pytest.raises(rw.RocwmmaError) as e:
+        rw.bench_stream(5, src, dst, n)
+    assert e.value.status == 1
     with pytest.raises(rw.RocwmmaError) as e:  # whole 64 KiB trips only
         rw.bench_stream(rw.STREAM_COPY, src, dst, n + 32768)
     assert e.value.status == 3
