@@ -313,7 +313,7 @@ def exact_fwd_mm(inp, m, k):
     return np.concatenate([F[:, 0, :], Z[:, il, jl]], axis=1)
 
 
-GENERAL_SHAPES = [(3, 160, 128), (2, 129, 64), (5, 27, 96), (2, 200, 40), (3, 1, 24), (4, 2, 8), (2, 300, 512),
+GENERAL_SHAPES = [(3, 160, 128), (11, 129, 64), (5, 27, 96), (2, 200, 40), (3, 1, 24), (4, 2, 8), (2, 300, 512),
                   (2, 130, 1032), (3, 257, 264), (1, 1024, 1024)]
 
 
@@ -321,7 +321,8 @@ GENERAL_SHAPES = [(3, 160, 128), (2, 129, 64), (5, 27, 96), (2, 200, 40), (3, 1,
 def test_samples_larger_than_a_wave_run_as_tiles_of_128(b, m, k):
     """f16, forward and backward against the oracle: m just above 128 and not a multiple of anything, k that is no power
     of two (96, 40, 24, 8: whole 16-byte pieces is all that is asked), k that ends inside a step of the K loop
-    (1032, 264), one and two feature rows, more than one tile in every direction, the reference's largest size."""
+    (1032, 264), one and two feature rows, more than one tile in every direction, a batch that is no multiple of the
+    eight XCDs the samples are dealt to, the reference's largest size."""
     width = k + m * (m - 1) // 2
     inp = uniform_bits(1100 + m, orc.F16, b * m * k).reshape(b, m, k)
     up = uniform_bits(1101 + m, orc.F16, b * width).reshape(b, width)
